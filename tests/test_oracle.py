@@ -1,0 +1,339 @@
+"""Pins for the CPU oracle: each check is chosen so that a plausible mistake (a transposed
+factor, a wrong nibble, truncation instead of round-half-even, a dropped rounding) fails it.
+None of these retype the oracle's own formula: they use exact rational arithmetic, closed forms
+(scipy's Sylvester matrix, Kronecker products in float64), brute force and invariants."""
+import hashlib
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import scipy.linalg
+
+from oracle import quarot_oracle as o
+
+F16, F32 = np.float16, np.float32
+
+
+def all_finite_f16():
+    v = np.arange(65536, dtype=np.uint16).view(F16)
+    return v[np.isfinite(v)]
+
+
+def round_fraction_to_f16(fr):
+    """Correctly rounded (nearest, ties to even) binary16 of an exact Fraction, by search over
+    the two neighbouring representable values.  Independent of numpy's float casts except for
+    the (exact) float16 -> Fraction conversion."""
+    if fr == 0:
+        return F16(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    # exponent of the binade
+    e = 0
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1
+    while Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, -14)                       # subnormal grid below 2^-14
+    ulp = Fraction(2) ** (e - 10)
+    k = a / ulp
+    lo = int(k)                           # floor
+    rem = k - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+        lo += 1
+    val = lo * ulp
+    if val >= Fraction(65520):
+        return F16(sign * np.inf)
+    return F16(sign * float(val))
+
+
+# ------------------------------------------------------------------ tables and get_hadK
+
+SHA = {12: "5ed24dfa527572b5", 20: "f1f0309c0a997831", 28: "388c0b2f668d130f", 36: "d56db1cfa5877c3f",
+       40: "e697ab89f5bb9140", 52: "f80473403896af66", 60: "73c41ef814c170ec", 108: "a213b05e570867de",
+       140: "3c0c825cdc56ba9e", 156: "a53703a157ee01fb", 172: "891685e890ac3afd"}
+
+
+def test_tables_hash_and_orthogonality():
+    t = o.hadamard_tables()
+    assert sorted(t) == sorted(SHA)
+    for k, h in t.items():
+        assert h.shape == (k, k) and set(np.unique(h)) == {-1, 1}
+        assert hashlib.sha256(np.packbits(h.reshape(-1) > 0).tobytes()).hexdigest()[:16] == SHA[k]
+        hh = h.astype(np.int64)
+        assert np.array_equal(hh @ hh.T, k * np.eye(k, dtype=np.int64))
+    # orientation matters: several tables are not symmetric
+    assert np.array_equal(t[28], t[28].T) and np.array_equal(t[36], t[36].T)
+    assert not np.array_equal(t[172], t[172].T) and not np.array_equal(t[12], t[12].T)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 1), (8192, 1), (128, 1), (32, 1), (64, 1), (11008, 172), (28672, 28),
+                                 (13824, 108), (5120, 40), (6656, 52), (17920, 140), (14336, 28), (12288, 12),
+                                 (72, 36), (19968, 156), (15360, 60), (160, 40), (80, 40), (20, 20)])
+def test_get_hadK_known_answers(n, k):
+    h, kk = o.get_hadK(n)
+    assert kk == k
+    assert (h is None) == (k == 1)
+    if h is not None:
+        assert np.array_equal(o.get_hadK(n, transpose=True)[0], h.T)
+
+
+@pytest.mark.parametrize("n", [324, 3 * 172, 100, 7, 0])
+def test_get_hadK_rejects(n):
+    with pytest.raises(AssertionError):
+        o.get_hadK(n)
+
+
+def test_sylvester_matches_scipy():
+    for m in (1, 2, 8, 64, 256):
+        assert np.array_equal(o.sylvester(m), scipy.linalg.hadamard(m))
+
+
+# ------------------------------------------------------------------ Hadamard transforms
+
+@pytest.mark.parametrize("n", [8, 16, 64, 24, 40, 56, 72, 344, 104])
+def test_matmul_hadU_equals_kron_closed_form(n):
+    rng = np.random.default_rng(n)
+    x = rng.standard_normal((5, n))
+    hadk, k = o.get_hadK(n)
+    hm = scipy.linalg.hadamard(n // k).astype(np.float64)
+    full = hm if k == 1 else np.kron(hadk, hm)
+    want = x @ full.T / np.sqrt(n)
+    got = o.matmul_hadU(x)
+    # float32 sqrt(n) inside matmul_hadU limits agreement to ~1e-7 relative
+    np.testing.assert_allclose(got, want, rtol=2e-7, atol=1e-12)
+    np.testing.assert_allclose(o.hadamard_closed_form(x), want, rtol=1e-13, atol=1e-13)
+    # transposed factor inverts it (orthonormal), and differs when hadK is not symmetric
+    back = o.matmul_hadU(got, transpose=True) if k > 1 else o.matmul_hadU(got)
+    np.testing.assert_allclose(back, x, rtol=1e-6, atol=1e-6)
+
+
+def test_matmul_hadU_unit_vectors_give_columns():
+    n = 344  # 172 * 2
+    hadk, k = o.get_hadK(n)
+    full = np.kron(hadk, scipy.linalg.hadamard(2))
+    eye = np.eye(n)
+    got = o.matmul_hadU(eye) * np.sqrt(F32(n)).astype(np.float64)
+    np.testing.assert_allclose(got, full.T, atol=1e-9)   # row i of output = column i of kron(...)
+
+
+@pytest.mark.parametrize("n,dtype", [(64, F16), (4096, F16), (688, F16), (688, F32), (224, F32), (11008, F16)])
+def test_hadamard_staged_close_to_closed_form(n, dtype):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((3, n)).astype(dtype)
+    hadk, k = o.get_hadK(n)
+    got = o.hadamard_staged(x, hadk, k, dtype).astype(np.float64)
+    want = o.hadamard_closed_form(x.astype(np.float64))
+    tol = 2e-3 if dtype == F16 else 2e-6
+    np.testing.assert_allclose(got, want, rtol=tol, atol=tol)
+    # norm preservation
+    np.testing.assert_allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(x.astype(np.float64), axis=-1), rtol=1e-3)
+
+
+def test_fwht_natural_brute_force():
+    rng = np.random.default_rng(2)
+    for m in (1, 2, 4, 32, 128):
+        x = rng.standard_normal((4, m))
+        np.testing.assert_allclose(o.fwht_natural(x), x @ scipy.linalg.hadamard(m).astype(float).T, atol=1e-10)
+
+
+def test_kv_hadamard_involution_and_value():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((6, 128)).astype(F16)
+    y = o.kv_hadamard(x)
+    want = x.astype(np.float64) @ scipy.linalg.hadamard(128) / np.sqrt(128)
+    np.testing.assert_allclose(y.astype(np.float64), want, rtol=1e-3, atol=1e-3)
+    np.testing.assert_allclose(o.kv_hadamard(y).astype(np.float64), x.astype(np.float64), rtol=3e-3, atol=3e-3)
+
+
+# ------------------------------------------------------------------ quantizer
+
+def test_scale_is_correctly_rounded_for_every_amax():
+    amax = np.abs(all_finite_f16())
+    amax = np.unique(amax)
+    got = o.quantizer_scales(amax.reshape(-1, 1))
+    step = 97  # every 97th value by exact rational rounding (the full sweep is 31k Fractions; keep it quick)
+    for a, g in zip(amax[::step], got[::step]):
+        assert round_fraction_to_f16(Fraction(float(a)) / 7) == g, a
+    # clip ratio: torch evaluates half_tensor * python_float in float32 and rounds the float32
+    # product to fp16 (two roundings), so the pin here is torch's own CPU kernel on every amax.
+    import torch
+    t = torch.from_numpy(amax.copy()).reshape(-1, 1)
+    for clip in (0.9, 0.85, 1.0):
+        want = ((torch.max(torch.abs(t), dim=-1)[0].unsqueeze(1) / 7).to(torch.float16) * clip).numpy().reshape(-1)
+        assert np.array_equal(o.quantizer_scales(amax.reshape(-1, 1), clip=clip), want)
+
+
+def test_codes_match_torch_cpu_half_ops():
+    """The reference's CPU-capable statement of the same quantiser is torch.round(x / scale) on
+    fp16 tensors (quarot/functional/quantization.py:31); torch's CPU half kernels are an
+    independent implementation of the IEEE operations the oracle spells out in numpy."""
+    import torch
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((64, 512)) * 4).astype(F16)
+    s = o.quantizer_scales(x)
+    tx, ts = torch.from_numpy(x), torch.from_numpy(s).reshape(-1, 1)
+    want = torch.clamp(torch.round(tx / ts), -8, 7).to(torch.int8).numpy()
+    assert np.array_equal(o.sym_quant_codes(x, s), want)
+    q = torch.from_numpy(rng.integers(-30000, 30000, (64, 48)).astype(np.int32))
+    sc = torch.from_numpy((np.abs(rng.standard_normal(48)) * 0.01).astype(F16))
+    wantd = (ts * sc.reshape(1, -1)) * q.to(torch.float16)
+    assert np.array_equal(o.sym_dequant(q.numpy(), s, sc.numpy()).view(np.uint16), wantd.numpy().view(np.uint16))
+
+
+def test_codes_exact_rational_random_and_ties():
+    rng = np.random.default_rng(4)
+    xs = rng.standard_normal(400).astype(F16) * F16(3)
+    ss = np.abs(rng.standard_normal(400).astype(F16)) + F16(0.01)
+    got = o.sym_quant_codes(xs.reshape(-1, 1), ss)
+    for x, s, g in zip(xs, ss, got[:, 0]):
+        d = round_fraction_to_f16(Fraction(float(x)) / Fraction(float(s)))
+        fr = Fraction(float(d))
+        fl = fr.numerator // fr.denominator
+        rem = fr - fl
+        r = fl + (1 if (rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1)) else 0)
+        assert g == max(-8, min(7, r)), (x, s)
+    # constructed ties: x = s * (j + 0.5) exactly -> round half to even
+    s = F16(0.25)
+    halves = np.array([-8.5, -7.5, -2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.5, 6.5, 7.5, 8.5, 100.0, -100.0])
+    x = (halves * float(s)).astype(F16)
+    want = np.array([-8, -8, -2, -2, 0, 0, 2, 2, 4, 6, 7, 7, 7, -8])
+    assert np.array_equal(o.sym_quant_codes(x.reshape(1, -1), np.array([s]))[0], want)
+    # truncation toward zero (the HIP __half2int_rn trap) would give 0 for 0.75 and 1 for 1.75
+    x = np.array([0.75, 1.75, -0.75, -1.75], F16)
+    assert np.array_equal(o.sym_quant_codes(x.reshape(1, -1), np.array([F16(1)]))[0], [1, 2, -1, -2])
+
+
+def test_codes_double_rounding_case():
+    # x/s slightly below 2.5 but within half an fp16 ulp of it: fp16 division gives exactly 2.5,
+    # which then rounds to even (2); 3.5-eps likewise becomes 3.5 -> 4 (exact rounding would say 3).
+    s = F16(1 / 3)            # 0.33325195
+    found = 0
+    for target, want in ((3.5, 4), (2.5, 2), (5.5, 6)):
+        for xb in all_finite_f16():
+            if xb <= 0:
+                continue
+            exact = Fraction(float(xb)) / Fraction(float(s))
+            if exact < Fraction(target) and round_fraction_to_f16(exact) == F16(target):
+                assert o.sym_quant_codes(np.array([[xb]], F16), np.array([s]))[0, 0] == want
+                found += 1
+                break
+    assert found >= 1
+
+
+def test_zero_row_gives_zero_codes_and_zero_scale():
+    x = np.zeros((2, 8), F16)
+    p, s = o.quantizer(x)
+    assert np.all(s == 0) and np.all(p == 0)
+    # explicit zero scale with non-zero x: +-inf -> clamp
+    c = o.sym_quant_codes(np.array([[1, -1, 0]], F16), np.array([0], F16))
+    assert np.array_equal(c[0], [7, -8, 0])
+
+
+def test_pack_unpack_all_bytes_and_nibble_order():
+    b = np.arange(256, dtype=np.uint8).reshape(16, 16)
+    assert np.array_equal(o.pack_i4(o.unpack_i4(b)), b)
+    assert np.array_equal(o.unpack_i4(np.array([[0x2F]], np.uint8)), [[-1, 2]])      # low nibble first
+    assert np.array_equal(o.pack_i4(np.array([[-8, 7, 3]])), [[0x78, 0x03]])         # odd tail -> high nibble 0
+    assert o.unpack_i4(b).min() == -8 and o.unpack_i4(b).max() == 7
+    with pytest.raises(AssertionError):
+        o.pack_i4(np.array([[8, 0]]))
+
+
+# ------------------------------------------------------------------ GEMM and dequant
+
+def test_int4_matmul_known_answers():
+    k = 128
+    a = o.pack_i4(np.full((3, k), 7))
+    b = o.pack_i4(np.full((5, k), -8))
+    assert np.all(o.int4_matmul(a, b) == -56 * k)
+    assert np.all(o.int4_matmul(a, b, exact_int=True) == -56 * k)
+    # one-hot rows pick out columns of B^T
+    rng = np.random.default_rng(5)
+    bq = rng.integers(-8, 8, (7, 64))
+    onehot = np.zeros((64, 64), np.int64)
+    onehot[np.arange(64), np.arange(64)] = 1
+    assert np.array_equal(o.int4_matmul(o.pack_i4(onehot), o.pack_i4(bq)), bq.T)
+
+
+def test_int4_matmul_float_path_equals_int64():
+    rng = np.random.default_rng(6)
+    aq = rng.integers(-8, 8, (33, 448))
+    bq = rng.integers(-8, 8, (17, 448))
+    want = aq.astype(np.int64) @ bq.astype(np.int64).T
+    assert np.array_equal(o.int4_matmul(o.pack_i4(aq), o.pack_i4(bq)), want)
+    assert np.array_equal(o.int4_matmul(o.pack_i4(aq), o.pack_i4(bq), exact_int=True), want)
+
+
+def test_dequant_three_roundings_exact():
+    rng = np.random.default_rng(7)
+    q = rng.integers(-40000, 40000, (6, 9)).astype(np.int32)
+    q[0, 0], q[0, 1], q[0, 2] = 2049, 65519, 65520          # 2049 -> 2048 (tie to even), 65519 -> 65504, 65520 -> inf
+    sr = (np.abs(rng.standard_normal(6)) * 0.1).astype(F16)
+    sc = (np.abs(rng.standard_normal(9)) * 0.01).astype(F16)
+    bias = rng.standard_normal(9).astype(F16)
+    got = o.sym_dequant(q, sr, sc)
+    gotb = o.sym_dequant(q, sr, sc, bias)
+    for i in range(6):
+        for j in range(9):
+            qh = round_fraction_to_f16(Fraction(int(q[i, j])))
+            ss = round_fraction_to_f16(Fraction(float(sr[i])) * Fraction(float(sc[j])))
+            if not np.isfinite(qh):
+                assert not np.isfinite(got[i, j])
+                continue
+            y = round_fraction_to_f16(Fraction(float(ss)) * Fraction(float(qh)))
+            assert y == got[i, j]
+            assert round_fraction_to_f16(Fraction(float(y)) + Fraction(float(bias[j]))) == gotb[i, j]
+    assert o.sym_dequant(np.array([[2049]]), [F16(1)], [F16(1)])[0, 0] == F16(2048)
+
+
+def test_linear4bit_close_to_float_product():
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((16, 256)).astype(F16)
+    w = (rng.standard_normal((24, 256)) * 0.02).astype(F16)
+    ws = (np.max(np.abs(w), axis=1, keepdims=True).astype(F32) / 7).astype(F16)
+    wq = o.weight_codes_from_float(w, ws)
+    xq, xs = o.quantizer(x)
+    y = o.linear4bit(xq, xs, wq, ws).astype(np.float64)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    # 4-bit noise: correlation, not equality
+    assert np.corrcoef(y.ravel(), ref.ravel())[0, 1] > 0.95
+
+
+# ------------------------------------------------------------------ KV asymmetric int4
+
+def test_kv_asym_invariants():
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((64, 128)).astype(F16)
+    p, s, z = o.kv_asym_quant(x)
+    assert p.shape == (64, 64) and s.shape == (64, 1) and z.shape == (64, 1)
+    nib = np.stack([p & 0xF, p >> 4], -1).reshape(64, 128)
+    assert nib[np.arange(64), x.argmin(1)].max() == 0          # min -> code 0
+    assert nib[np.arange(64), x.argmax(1)].min() == 15         # max -> code 15
+    xh = o.kv_asym_dequant(p, s, z).astype(np.float64)
+    err = np.abs(xh - x.astype(np.float64))
+    assert np.all(err <= s.astype(np.float64) / 2 + 4e-3)
+    # constant vector: range clamps to fp16(1e-5), all codes 0
+    c = np.full((1, 128), 0.5, F16)
+    p, s, z = o.kv_asym_quant(c)
+    assert np.all(p == 0) and s[0, 0] == (F16(1e-5).astype(F32) / F32(15)).astype(F16) and z[0, 0] == F16(-0.5)
+
+
+def test_kv_asym_exact_rational_spot():
+    rng = np.random.default_rng(10)
+    x = (rng.standard_normal((3, 128)) * 2).astype(F16)
+    p, s, z = o.kv_asym_quant(x)
+    nib = np.stack([p & 0xF, p >> 4], -1).reshape(3, 128)
+    for r in range(3):
+        mx, mn = Fraction(float(x[r].max())), Fraction(float(x[r].min()))
+        rg = round_fraction_to_f16(mx - mn)
+        sc = round_fraction_to_f16(Fraction(float(rg)) / 15)
+        assert sc == s[r, 0] and z[r, 0] == F16(-float(mn))
+        for c in range(0, 128, 5):
+            sh = round_fraction_to_f16(Fraction(float(x[r, c])) - mn)
+            d = Fraction(float(round_fraction_to_f16(Fraction(float(sh)) / Fraction(float(sc)))))
+            fl = d.numerator // d.denominator
+            rem = d - fl
+            q = fl + (1 if (rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1)) else 0)
+            assert nib[r, c] == max(0, min(15, q))
+            back = round_fraction_to_f16(Fraction(float(round_fraction_to_f16(int(nib[r, c]) * Fraction(float(sc))))) + mn)
+            assert back == o.kv_asym_dequant(p, s, z)[r, c]
