@@ -1,0 +1,141 @@
+/*
+ * quarot_hip.h - C ABI of libquarot_hip.so: QuaRot's quantized-linear hot path on gfx950 (MI355X).
+ *
+ * Conventions
+ *   - Every pointer except `stream` and `hadK`-when-K==1 is a DEVICE pointer owned by the caller.
+ *     The library never allocates, frees or synchronises; kernels are enqueued on `stream`
+ *     (a hipStream_t passed as void*, NULL = the default stream).
+ *   - Matrices are dense row-major.  "int4 packed" means two two's-complement nibbles per byte,
+ *     even column in the LOW nibble (reference: quarot/kernels/include/int4.h:86-98,
+ *     quarot/functional/quantization.py:42-49).
+ *   - fp16 is IEEE binary16.  Every fp16 operation the reference performs is performed here as one
+ *     correctly rounded operation in the same order, so codes and dequantised values are bit-exact.
+ *   - Return value: 0 = success; < 0 = argument error (QR_E_*), nothing was launched;
+ *     > 0 = a hipError_t reported by the launch.  qr_strerror() explains either.
+ *
+ * Reference paths are relative to the spcl/QuaRot source tree.
+ */
+#ifndef QUAROT_HIP_H
+#define QUAROT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QR_OK            0
+#define QR_E_NULL       -1   /* a required pointer is NULL */
+#define QR_E_SHAPE      -2   /* a size is negative, zero where it may not be, or violates a divisibility rule */
+#define QR_E_UNSUPPORTED -3  /* valid for the reference but outside what this build implements */
+#define QR_E_ALIGN      -4   /* a pointer is not aligned as the entry point requires */
+#define QR_E_DTYPE      -5   /* unknown dtype / mode code */
+
+#define QR_DTYPE_F16 0
+#define QR_DTYPE_F32 1
+
+/* Library version (major*10000 + minor*100 + patch). */
+int qr_version(void);
+
+/* Human-readable text for a return code of any entry point (static storage). */
+const char* qr_strerror(int code);
+
+/*
+ * Online Hadamard transform along the last axis:  y = x . (hadK (x) H_{n/K})^T * scale.
+ * Replaces fast_hadamard_transform.hadamard_transform + `hadK @ input` as called by
+ * matmul_hadU_cuda (quarot/functional/hadamard.py:92-101) and matmul_had_cuda
+ * (quarot/transformers/kv_cache.py:30-33).
+ *   x, y    [rows, n] of `dtype` (QR_DTYPE_F16 or QR_DTYPE_F32); y may alias x.
+ *   K       1, or the order of hadK; n % K == 0 and n / K a power of two, 8 <= n/K, n <= 32768.
+ *   hadK    [K, K] row-major of `dtype` (the module's had_rem_dim buffer), ignored when K == 1.
+ *           Entries must be exactly representable in fp16 (the reference's tables are +-1).
+ *   scale   applied in fp32 after the butterflies (the reference passes 1/sqrt(n)).
+ * Numerics: butterflies and scale in fp32.  QR_DTYPE_F16: the power-of-two stage is rounded to fp16
+ * before the hadK stage, whose fp32 accumulation is rounded to fp16 (the reference's staging).
+ * QR_DTYPE_F32: fp32 throughout.
+ */
+int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, const void* hadK,
+                int dtype, float scale, void* stream);
+
+/*
+ * Symmetric int4 quantisation with given per-row scales.
+ * Replaces sym_quant_host / sym_quantize_f16_i4_kernel (quarot/kernels/quant.cu:11-61), bound as
+ * quarot._CUDA.sym_quant (quarot/kernels/bindings.cpp:27-44).
+ *   x fp16 [rows, cols], scale fp16 [rows]  ->  q uint8 [rows, ceil(cols/2)]
+ *   q = clamp(round_half_even(fp16(x / scale)), -8, 7); 0/0 gives code 0; odd cols leave the last
+ *   high nibble 0.
+ */
+int qr_sym_quant_f16_i4(const void* x, const void* scale, int64_t rows, int64_t cols, void* q,
+                        void* stream);
+
+/*
+ * Per-token quantiser: row abs-max -> scale -> codes, one pass over x.
+ * Replaces Quantizer.forward (quarot/nn/quantization.py:9-13) = four torch kernels + sym_quant.
+ *   scales[r] = fp16( float(fp16(amax_r / 7)) * clip ),  q as qr_sym_quant_f16_i4.
+ *   x fp16 [rows, cols] -> q uint8 [rows, ceil(cols/2)], scales fp16 [rows]
+ */
+int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, int64_t cols, void* q,
+                            void* scales, void* stream);
+
+/*
+ * Fused OnlineHadamard + Quantizer (quarot/nn/hadamard.py:17-23 then quarot/nn/quantization.py:9-13):
+ * the transformed row is rounded to fp16 exactly as qr_hadamard(QR_DTYPE_F16 input) would store it
+ * and quantised from there, without the fp16 tensor making a round trip through HBM.
+ *   x fp16 [rows, n]; mode QR_DTYPE_F16 (fp16 staging) or QR_DTYPE_F32 (OnlineHadamard force_fp32:
+ *   hadK is then fp32 [K,K]); y_or_null: optional fp16 [rows, n] copy of the transformed rows.
+ */
+int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, int K, const void* hadK,
+                                int mode, float scale, float clip, void* q, void* scales,
+                                void* y_or_null, void* stream);
+
+/*
+ * int4 x int4 -> int32 GEMM:  C[M, N] = unpack(A)[M, K] . unpack(B)[N, K]^T.
+ * Replaces matmul_host (quarot/kernels/gemm.cu:7-46), bound as quarot._CUDA.matmul
+ * (quarot/kernels/bindings.cpp:9-25).
+ *   A uint8 [M, K/2], B uint8 [N, K/2], C int32 [M, N]; K % 64 == 0 (quarot/__init__.py:38),
+ *   K <= 131008; A and B 16-byte aligned.
+ */
+int qr_matmul_i4_i32(const void* A, const void* B, int64_t M, int64_t N, int64_t K, void* C,
+                     void* stream);
+
+/*
+ * y[r, c] = fp16( fp16(scale_row[r] * scale_col[c]) * fp16_rn(q[r, c]) ).
+ * Replaces sym_dequant_host / sym_dequantize_i32_f16_kernel (quarot/kernels/quant.cu:64-97), bound
+ * as quarot._CUDA.sym_dequant with bits == 32 (quarot/kernels/bindings.cpp:47-87).
+ */
+int qr_sym_dequant_i32_f16(const void* q, const void* scale_row, const void* scale_col,
+                           int64_t rows, int64_t cols, void* y, void* stream);
+
+/*
+ * Linear4bit.forward in one kernel (quarot/nn/linear.py:42-56): the GEMM above with the dequant
+ * (and the optional fp16 bias add, a fourth rounded operation) applied to the accumulators.
+ *   A uint8 [M, K/2], sA fp16 [M], W uint8 [N, K/2], sW fp16 [N], bias fp16 [N] or NULL -> y fp16 [M, N]
+ */
+int qr_linear_i4_f16(const void* A, const void* sA, const void* W, const void* sW,
+                     const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y,
+                     void* stream);
+
+/*
+ * KV-cache path: optional Hadamard over the head dimension, then per-vector asymmetric int4.
+ * Replaces matmul_had_cuda + asym_quantize_and_pack_i4 (quarot/transformers/kv_cache.py:10-33).
+ *   x fp16 [vectors, dim], dim a power of two in [16, 256].
+ *   had_mode: 0 = none (V), 1 = FWHT * 1/sqrt(dim) rounded to fp16 (K).
+ *   q uint8 [vectors, dim/2]; scale, zero fp16 [vectors]:
+ *   scale = max(fp16(max - min), fp16(1e-5)) / 15, zero = -min,
+ *   q = clamp(round_half_even(fp16(fp16(x + zero) / scale)), 0, 15).
+ */
+int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int had_mode, void* q,
+                       void* scale, void* zero, void* stream);
+
+/*
+ * Inverse of the above: y = fp16( fp16(nibble * scale) - zero )
+ * (unpack_i4_and_asym_dequantize, quarot/transformers/kv_cache.py:24-28).
+ */
+int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void* zero, int64_t vectors,
+                         int dim, void* y, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QUAROT_HIP_H */

@@ -1,0 +1,187 @@
+"""quarot_amd: QuaRot's quantized-linear hot path on MI355X (gfx950).
+
+Drop-in for the top level of the reference's ``quarot`` package (quarot/__init__.py:9-71):
+``matmul``, ``sym_quant``, ``sym_dequant``, ``PackedQuantizedTensor`` keep their signatures,
+assertions and output shapes; they call hand-written HIP kernels in ``libquarot_hip.so`` through
+its C ABI.  Extras that fuse adjacent steps are listed after the reference's names.
+
+    import quarot_amd as quarot
+"""
+import torch
+
+from . import _lib
+from . import functional
+from . import nn
+
+__all__ = [
+    "matmul", "sym_quant", "sym_dequant", "PackedQuantizedTensor",      # the reference's names
+    "quantize_rows", "hadamard_quantize", "linear_i4",                  # fused entry points
+]
+
+
+def _flat2d(x: torch.Tensor):
+    """[..., C] -> ([R, C] view, leading shape).  Same contract as the reference's
+    flatten_last_dim_and_return_shape (quarot/__init__.py:31-34): `view`, so it raises on
+    layouts that cannot be flattened without a copy."""
+    lead = x.shape[:-1]
+    return x.view(-1, x.shape[-1]), lead
+
+
+def _require_gpu_contiguous(fn, **tensors):
+    """The checks of quarot/kernels/bindings.cpp:11-16,29-34,52-64 (contiguous, on the GPU, one
+    device) raised as RuntimeError like torch::check* does."""
+    dev = None
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(f"{fn}: expected {name} to be a GPU tensor, got {t.device}")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{fn}: expected {name} to be contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"{fn}: expected all tensors on {dev}, but {name} is on {t.device}")
+    return dev
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def matmul(A, B):
+    """int4 x int4 -> int32: unpack(A) @ unpack(B).T  (quarot/__init__.py:37-41).
+    A uint8 [..., K/2], B uint8 [..., K/2] -> int32 [*A.shape[:-1], *B.shape[:-1]]."""
+    assert A.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(A.shape[-1])
+    A2, a_lead = _flat2d(A)
+    B2, b_lead = _flat2d(B)
+    dev = _require_gpu_contiguous("matmul", A=A2, B=B2)
+    if A2.dtype != torch.uint8 or B2.dtype != torch.uint8:
+        raise RuntimeError("matmul: expected packed uint8 operands")
+    if A2.shape[1] != B2.shape[1]:
+        raise RuntimeError(f"matmul: inner sizes differ ({A2.shape[1]} vs {B2.shape[1]} packed bytes)")
+    M, N, K = A2.shape[0], B2.shape[0], A2.shape[1] * 2
+    C = torch.empty((M, N), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_matmul_i4_i32(_ptr(A2), _ptr(B2), M, N, K, _ptr(C), _lib.stream_ptr(dev)))
+    return C.view(*a_lead, *b_lead)
+
+
+def sym_quant(x, scale):
+    """Symmetric int4 quantise + pack with given per-row scales (quarot/__init__.py:43-46).
+    x fp16 [..., C], scale fp16 (one per row, any shape) -> uint8 [..., ceil(C/2)]."""
+    assert x.dtype == scale.dtype == torch.float16
+    x2, lead = _flat2d(x)
+    s = scale.view(-1)
+    dev = _require_gpu_contiguous("sym_quant", x=x2, scale=s)
+    if s.shape[0] != x2.shape[0]:
+        raise RuntimeError(f"sym_quant: expected scale of size {x2.shape[0]}, got {s.shape[0]}")
+    rows, cols = x2.shape
+    q = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_sym_quant_f16_i4(_ptr(x2), _ptr(s), rows, cols, _ptr(q), _lib.stream_ptr(dev)))
+    return q.view(*lead, -1)
+
+
+def sym_dequant(q, scale_row, scale_col, bits=32):
+    """fp16((scale_row * scale_col) * half(q))  (quarot/__init__.py:48-52)."""
+    assert q.dtype == torch.int32
+    assert scale_row.dtype == scale_col.dtype == torch.float16
+    q2, lead = _flat2d(q)
+    sr = scale_row.view(-1)
+    dev = _require_gpu_contiguous("sym_dequant", q=q2, scale_row=sr, scale_col=scale_col)
+    rows, cols = q2.shape
+    if sr.shape[0] != rows:
+        raise RuntimeError(f"sym_dequant: expected scale_row of size {rows}, got {sr.shape[0]}")
+    if scale_col.shape[0] != cols:
+        raise RuntimeError(f"sym_dequant: expected scale_col of size {cols}, got {scale_col.shape[0]}")
+    if bits != 32:
+        raise RuntimeError("Unsupported data type")       # quarot/kernels/bindings.cpp:76-84
+    y = torch.empty((rows, cols), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_sym_dequant_i32_f16(_ptr(q2), _ptr(sr), _ptr(scale_col), rows, cols, _ptr(y),
+                                                     _lib.stream_ptr(dev)))
+    return y.view(*lead, -1)
+
+
+class PackedQuantizedTensor:
+    """Carrier of packed int4 codes and their per-row scales (quarot/__init__.py:55-71)."""
+
+    def __init__(self, quantized_x: torch.Tensor, scales_x: torch.Tensor):
+        self.quantized_x = quantized_x
+        self.scales_x = scales_x
+
+    def size(self):
+        return self.quantized_x.size()
+
+    @property
+    def device(self):
+        return self.quantized_x.device
+
+    @property
+    def dtype(self):
+        return self.quantized_x.dtype
+
+
+# ------------------------------------------------------------------------------------------------
+# fused entry points (no counterpart of their own in the reference; each equals a chain of its calls)
+
+def quantize_rows(x, clip_ratio=1.0):
+    """Quantizer.forward in one kernel (quarot/nn/quantization.py:9-13): returns
+    (packed uint8 [..., C/2], scales fp16 with the reference's [R, 1]-after-unsqueeze(1) shape)."""
+    assert x.dtype == torch.float16
+    x2, lead = _flat2d(x)
+    dev = _require_gpu_contiguous("quantize_rows", x=x2)
+    rows, cols = x2.shape
+    q = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=dev)
+    s = torch.empty((rows,), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_quantize_rows_f16_i4(_ptr(x2), float(clip_ratio), rows, cols, _ptr(q), _ptr(s),
+                                                      _lib.stream_ptr(dev)))
+    # torch.max(dim=-1)[0].unsqueeze(1) on [..., C] gives shape lead[:1] + (1,) + lead[1:]
+    s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
+    return q.view(*lead, -1), s.view(s_shape)
+
+
+def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_transformed=False):
+    """OnlineHadamard.forward followed by Quantizer.forward in one kernel
+    (quarot/nn/hadamard.py:17-23 + quarot/nn/quantization.py:9-13)."""
+    assert x.dtype == torch.float16
+    x2, lead = _flat2d(x)
+    dev = _require_gpu_contiguous("hadamard_quantize", x=x2, hadK=hadK)
+    rows, n = x2.shape
+    want = torch.float32 if force_fp32 else torch.float16
+    if hadK is not None and hadK.dtype != want:
+        hadK = hadK.to(want)
+    q = torch.empty((rows, n // 2), dtype=torch.uint8, device=dev)
+    s = torch.empty((rows,), dtype=torch.float16, device=dev)
+    y = torch.empty_like(x2) if return_transformed else None
+    scale = float(1.0 / torch.tensor(n).sqrt())
+    mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
+                                                          float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
+                                                          _lib.stream_ptr(dev)))
+    s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
+    packed = PackedQuantizedTensor(q.view(*lead, -1), s.view(s_shape))
+    return (packed, y.view(x.shape)) if return_transformed else packed
+
+
+def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
+    """Linear4bit.forward in one kernel (quarot/nn/linear.py:42-56): matmul + sym_dequant (+ bias)."""
+    assert x_q.shape[-1] % 32 == 0, "A.shape[-1]: {} must be multiplication of 32".format(x_q.shape[-1])
+    assert scales_x.dtype == weight_scales.dtype == torch.float16
+    a2, lead = _flat2d(x_q)
+    sx = scales_x.view(-1)
+    sw = weight_scales.view(-1)
+    dev = _require_gpu_contiguous("linear_i4", x=a2, scales_x=sx, weight=weight, weight_scales=sw, bias=bias)
+    M, N, K = a2.shape[0], weight.shape[0], a2.shape[1] * 2
+    if weight.shape[1] != a2.shape[1] or sx.shape[0] != M or sw.shape[0] != N:
+        raise RuntimeError("linear_i4: inconsistent operand sizes")
+    if bias is not None and (bias.dtype != torch.float16 or bias.numel() != N):
+        raise RuntimeError("linear_i4: bias must be fp16 of size out_features")
+    y = torch.empty((M, N), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_linear_i4_f16(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K,
+                                               _ptr(y), _lib.stream_ptr(dev)))
+    return y.view(*lead, N)

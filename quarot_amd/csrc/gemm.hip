@@ -1,0 +1,214 @@
+// int4 x int4 -> int32 GEMM on the gfx950 int8 matrix cores, with an optional fused fp16 dequant
+// epilogue.  C[M, N] = unpack(A)[M, K] . unpack(B)[N, K]^T, both operands K-contiguous, packed two
+// nibbles per byte (even k in the low nibble).
+//
+// Feeding int4 to an int8 MFMA without sign extension: for a 32-bit word p holding 8 nibbles,
+//     lo = (p << 4) & 0xF0F0F0F0   holds 16 * v[even k] in each byte (as a signed int8)
+//     hi =  p       & 0xF0F0F0F0   holds 16 * v[odd k]
+// Both operands are scaled by 16, so every product is 256 * a * b and the accumulator is exactly
+// 256 * (the int4 dot product); an arithmetic shift by 8 at the end restores it.  Even and odd k
+// go to different MFMA issues; that permutation of k is the same for A and B, so dot products are
+// unchanged.  |acc| <= 256 * 64 * K requires K < 131072.
+#include "qr_common.h"
+
+namespace {
+
+constexpr int GT = 256;     // threads per workgroup (4 waves)
+
+// LDS holds, per stage, (BM + BN) rows of 64 packed bytes (128 k values) as four 16-byte chunks.
+// The chunk position is XOR-swizzled with bits 2..3 of the row so that the 16 rows a quarter-wave
+// reads in one ds_read_b128 beat fall in 16 different 16-byte bank groups.
+__device__ __forceinline__ int lds_slot(int row, int chunk) { return row * 4 + (chunk ^ ((row >> 2) & 3)); }
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
+__global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                     int M, int N, int Kb, int32_t* __restrict__ C,
+                                                     f16* __restrict__ Y, const f16* __restrict__ sA,
+                                                     const f16* __restrict__ sB, const f16* __restrict__ bias,
+                                                     int tiles_m, int tiles_n) {
+    static_assert(WAVES_M * WAVES_N == GT / QR_WAVE, "four waves");
+    constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;     // per-wave output tile
+    constexpr int IM = TM / 32, JN = TN / 32;               // 32x32 MFMA tiles per wave
+    constexpr int CH = (BM + BN) * 4;                       // 16-byte chunks per stage
+    constexpr int NL = (CH + GT - 1) / GT;                  // chunks each thread moves per stage
+    static_assert(TM % 32 == 0 && TN % 32 == 0, "tile shape");
+    __shared__ u32x4 lds[2][CH];
+
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Give every XCD a
+    // contiguous range of tile ids, and walk tiles in groups of GROUP_M rows so that the tiles in
+    // flight on one XCD share A rows and B rows.
+    const int nxcd = 8;
+    const int per_xcd = gridDim.x / nxcd;
+    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (tile >= tiles_m * tiles_n) return;
+    constexpr int GROUP_M = 8;
+    const int group_sz = GROUP_M * tiles_n;
+    const int g = tile / group_sz;
+    const int gm0 = g * GROUP_M;
+    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
+    const int tm = gm0 + (tile - g * group_sz) % gh;
+    const int tn = (tile - g * group_sz) / gh;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    // Global -> LDS staging: chunk id = tid + i * GT; 4 consecutive threads fetch one row's 64 bytes.
+    // Rows beyond M (or N) are clamped to the last valid row: they are read but never stored.
+    const uint8_t* src[NL];
+    int dst[NL];
+    int coff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        int qid = tid + i * GT;
+        if (qid >= CH) qid = CH - 1;        // (BM + BN) * 4 not a multiple of 256: the tail repeats the last chunk
+        const int row = qid >> 2, c = qid & 3;
+        if (row < BM) {
+            int gr = m0 + row;
+            gr = gr < M ? gr : M - 1;
+            src[i] = A + (int64_t)gr * Kb + c * 16;
+        } else {
+            int gr = n0 + row - BM;
+            gr = gr < N ? gr : N - 1;
+            src[i] = B + (int64_t)gr * Kb + c * 16;
+        }
+        coff[i] = c * 16;
+        dst[i] = lds_slot(row, c);
+    }
+
+    i32x16 acc[IM][JN];
+#pragma unroll
+    for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    const int ksteps = (Kb + 63) / 64;
+    u32x4 pre[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i)
+        pre[i] = (coff[i] < Kb) ? *(const u32x4*)(src[i]) : u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < NL; ++i) lds[0][dst[i]] = pre[i];
+    __syncthreads();
+
+    const int arow = wm * TM + (lane & 31);
+    const int brow = BM + wn * TN + (lane & 31);
+    const int khalf = lane >> 5;
+
+    for (int ks = 0; ks < ksteps; ++ks) {
+        const bool more = ks + 1 < ksteps;
+        if (more) {
+            const int kb = (ks + 1) * 64;
+#pragma unroll
+            for (int i = 0; i < NL; ++i)
+                pre[i] = (kb + coff[i] < Kb) ? *(const u32x4*)(src[i] + kb) : u32x4{0, 0, 0, 0};
+        }
+        const u32x4* buf = lds[ks & 1];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
+#pragma unroll
+            for (int i = 0; i < IM; ++i) {
+                u32x4 p = buf[lds_slot(arow + i * 32, s * 2 + khalf)];
+                alo[i] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+                ahi[i] = (i32x4)(p & 0xF0F0F0F0u);
+            }
+#pragma unroll
+            for (int j = 0; j < JN; ++j) {
+                u32x4 p = buf[lds_slot(brow + j * 32, s * 2 + khalf)];
+                blo[j] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+                bhi[j] = (i32x4)(p & 0xF0F0F0F0u);
+            }
+#pragma unroll
+            for (int i = 0; i < IM; ++i)
+#pragma unroll
+                for (int j = 0; j < JN; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[i], blo[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[i], bhi[j], acc[i][j], 0, 0, 0);
+                }
+        }
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < NL; ++i) lds[(ks + 1) & 1][dst[i]] = pre[i];
+        }
+        __syncthreads();
+    }
+
+    // Epilogue.  32x32 accumulator layout: lane l, register v -> row (v/4)*8 + (l/32)*4 + v%4, column l%32.
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+        const int col = n0 + wn * TN + j * 32 + (lane & 31);
+        if (col >= N) continue;
+        f16 sb = (f16)0, bb = (f16)0;
+        if (DEQ) {
+            sb = sB[col];
+            if (bias) bb = bias[col];
+        }
+#pragma unroll
+        for (int i = 0; i < IM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = m0 + wm * TM + i * 32 + (v >> 2) * 8 + khalf * 4 + (v & 3);
+                if (row >= M) continue;
+                const int val = acc[i][j][v] >> 8;
+                if (DEQ) {
+                    f16 yv = (f16)(sA[row] * sb) * (f16)(float)val;
+                    if (bias) yv = yv + bb;
+                    Y[(int64_t)row * N + col] = yv;
+                } else {
+                    C[(int64_t)row * N + col] = val;
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+               const void* bias, hipStream_t st) {
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles > 0x3fffffff) return QR_E_SHAPE;
+    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    if (Y)
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(GT), 0, st>>>(
+            (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, (const f16*)sA, (const f16*)sB,
+            (const f16*)bias, tiles_m, tiles_n);
+    else
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(GT), 0, st>>>(
+            (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr, nullptr, nullptr, nullptr, tiles_m,
+            tiles_n);
+    return qr_launch_status();
+}
+
+int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K, void* C, void* Y, const void* sA,
+                  const void* sB, const void* bias, hipStream_t st) {
+    if (M < 0 || N < 0 || K < 0) return QR_E_SHAPE;
+    if (M == 0 || N == 0) return QR_OK;
+    if (K == 0 || K % 64 != 0 || K > 131008 || M > 0x7fffffff || N > 0x7fffffff) return QR_E_SHAPE;
+    if (!A || !B || (!C && !Y)) return QR_E_NULL;
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return QR_E_ALIGN;
+    const int m = (int)M, n = (int)N, kb = (int)(K / 2);
+    const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+    if (M <= 32) return launch_cfg<32, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 64) return launch_cfg<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t256 >= 512) return launch_cfg<256, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
+    if (t128x256 >= 256) return launch_cfg<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+}
+
+}  // namespace
+
+extern "C" int qr_matmul_i4_i32(const void* A, const void* B, int64_t M, int64_t N, int64_t K, void* C, void* stream) {
+    if (M > 0 && N > 0 && !C) return QR_E_NULL;
+    return gemm_dispatch(A, B, M, N, K, C, nullptr, nullptr, nullptr, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int qr_linear_i4_f16(const void* A, const void* sA, const void* W, const void* sW, const void* bias_or_null,
+                                int64_t M, int64_t N, int64_t K, void* y, void* stream) {
+    if (M > 0 && N > 0 && (!y || !sA || !sW)) return QR_E_NULL;
+    return gemm_dispatch(A, W, M, N, K, nullptr, y, sA, sW, bias_or_null, (hipStream_t)stream);
+}

@@ -1,0 +1,197 @@
+// KV-cache path: per-head Hadamard (optional) + per-vector asymmetric int4 quantise/pack, and the
+// inverse dequantiser.  A vector of `dim` halves is spread over dim/8 adjacent lanes, 16 bytes each;
+// a wave handles 512/dim vectors, so all global accesses are full-width and coalesced.
+#include "qr_common.h"
+
+namespace {
+
+constexpr int KT = 256;
+
+template <int MASK>
+__device__ __forceinline__ float kv_lane_xor(float v) {
+    int i = __builtin_bit_cast(int, v);
+    int r;
+    if constexpr (MASK == 1) r = __builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true);
+    else if constexpr (MASK == 2) r = __builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true);
+    else if constexpr (MASK == 4) r = __builtin_amdgcn_ds_swizzle(i, 0x101F);
+    else if constexpr (MASK == 8) r = __builtin_amdgcn_mov_dpp(i, 0x128, 0xF, 0xF, true);
+    else r = __builtin_amdgcn_ds_swizzle(i, 0x401F);   // MASK == 16
+    return __builtin_bit_cast(float, r);
+}
+
+template <int MASK>
+__device__ __forceinline__ void kv_butterfly(float (&v)[8], int lane) {
+    const bool upper = (lane & MASK) != 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float p = kv_lane_xor<MASK>(v[e]);
+        v[e] = upper ? p - v[e] : v[e] + p;
+    }
+}
+
+template <int MASK>
+__device__ __forceinline__ void kv_minmax(float& mn, float& mx) {
+    float a = kv_lane_xor<MASK>(mn), b = kv_lane_xor<MASK>(mx);
+    mn = a < mn ? a : mn;
+    mx = b > mx ? b : mx;
+}
+
+// LG = log2(lanes per vector) = log2(dim) - 3, 1..5
+template <int LG, bool HAD>
+__global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ x, int64_t nchunks, float hscale,
+                                                      u32* __restrict__ q, f16* __restrict__ scale,
+                                                      f16* __restrict__ zero) {
+    const int lane = threadIdx.x & 63;
+    const int64_t stride = (int64_t)gridDim.x * KT;      // multiple of 64 > lanes per vector
+    for (int64_t c0 = (int64_t)blockIdx.x * KT; c0 < nchunks; c0 += stride) {
+        const int64_t c = c0 + threadIdx.x;
+        const bool live = c < nchunks;                   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
+        u32x4 raw = live ? __builtin_nontemporal_load(x + c) : u32x4{0, 0, 0, 0};
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = (float)f16_from_bits((unsigned short)(raw[i] & 0xffffu));
+            v[2 * i + 1] = (float)f16_from_bits((unsigned short)(raw[i] >> 16));
+        }
+        if (HAD) {
+#pragma unroll
+            for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if ((i & h) == 0) {
+                        float a = v[i], b = v[i | h];
+                        v[i] = a + b;
+                        v[i | h] = a - b;
+                    }
+            if (LG > 0) kv_butterfly<1>(v, lane);
+            if (LG > 1) kv_butterfly<2>(v, lane);
+            if (LG > 2) kv_butterfly<4>(v, lane);
+            if (LG > 3) kv_butterfly<8>(v, lane);
+            if (LG > 4) kv_butterfly<16>(v, lane);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (float)(f16)(v[e] * hscale);   // the transform's fp16 output
+        }
+        float mn = v[0], mx = v[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) {
+            mn = v[e] < mn ? v[e] : mn;
+            mx = v[e] > mx ? v[e] : mx;
+        }
+        if (LG > 0) kv_minmax<1>(mn, mx);
+        if (LG > 1) kv_minmax<2>(mn, mx);
+        if (LG > 2) kv_minmax<4>(mn, mx);
+        if (LG > 3) kv_minmax<8>(mn, mx);
+        if (LG > 4) kv_minmax<16>(mn, mx);
+        // scale = max(fp16(max - min), fp16(1e-5)) / 15 ; zero = -min   (each step one fp16 rounding)
+        f16 rng = (f16)(mx - mn);
+        const f16 floor_ = (f16)1e-5f;
+        rng = rng < floor_ ? floor_ : rng;
+        const f16 sc = (f16)(float)((double)(float)rng / 15.0);
+        const f16 zp = (f16)(-mn);
+        const float s = (float)sc, z = (float)zp;
+        const float rs = 1.0f / s;                       // s >= fp16(1e-5)/15 > 0, finite
+        u32 out = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sh = (float)(f16)(v[e] + z);
+            const float q0 = sh * rs;
+            const float er = __builtin_fmaf(-q0, s, sh);
+            const float q1 = __builtin_fabsf(q0) < __builtin_inff() ? __builtin_fmaf(er, rs, q0) : q0;
+            const float r = __builtin_rintf((float)(f16)q1);
+            int code = (int)r;
+            code = code < 0 ? 0 : (code > 15 ? 15 : code);
+            code = (r != r) ? 0 : code;
+            out |= (u32)code << (4 * e);
+        }
+        if (live) {
+            q[c] = out;
+            if ((lane & ((1 << LG) - 1)) == 0) {
+                scale[c >> LG] = sc;
+                zero[c >> LG] = zp;
+            }
+        }
+    }
+}
+
+template <int LG>
+__global__ __launch_bounds__(KT) void kv_dequant_kernel(const u32* __restrict__ q, const f16* __restrict__ scale,
+                                                        const f16* __restrict__ zero, int64_t nchunks,
+                                                        u32x4* __restrict__ y) {
+    const int64_t stride = (int64_t)gridDim.x * KT;
+    for (int64_t c = (int64_t)blockIdx.x * KT + threadIdx.x; c < nchunks; c += stride) {
+        const u32 w = __builtin_nontemporal_load(q + c);
+        const f16 sc = scale[c >> LG], zp = zero[c >> LG];
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f16 a = (f16)((f16)(float)((w >> (8 * i)) & 0xfu) * sc) - zp;
+            const f16 b = (f16)((f16)(float)((w >> (8 * i + 4)) & 0xfu) * sc) - zp;
+            o[i] = (u32)f16_bits(a) | ((u32)f16_bits(b) << 16);
+        }
+        __builtin_nontemporal_store(o, y + c);
+    }
+}
+
+int log2_dim(int dim) {
+    for (int l = 4; l <= 8; ++l)
+        if ((1 << l) == dim) return l;
+    return -1;
+}
+
+unsigned grid_for(int64_t nchunks) {
+    int64_t b = (nchunks + KT - 1) / KT;
+    const int64_t cap = 256 * 32;
+    return (unsigned)(b < cap ? b : cap);
+}
+
+}  // namespace
+
+extern "C" int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int had_mode, void* q, void* scale,
+                                  void* zero, void* stream) {
+    if (vectors < 0) return QR_E_SHAPE;
+    const int l2 = log2_dim(dim);
+    if (l2 < 0) return dim > 0 ? QR_E_UNSUPPORTED : QR_E_SHAPE;
+    if (had_mode != 0 && had_mode != 1) return QR_E_DTYPE;
+    if (vectors == 0) return QR_OK;
+    if (!x || !q || !scale || !zero) return QR_E_NULL;
+    if (((uintptr_t)x & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
+    const int64_t nchunks = vectors * (dim / 8);
+    const float hs = (float)(1.0 / __builtin_sqrt((double)dim));
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(grid_for(nchunks)), block(KT);
+#define QR_KV(LG)                                                                                                     \
+    case LG + 3:                                                                                                      \
+        if (had_mode)                                                                                                 \
+            kv_quant_kernel<LG, true><<<grid, block, 0, st>>>((const u32x4*)x, nchunks, hs, (u32*)q, (f16*)scale,     \
+                                                              (f16*)zero);                                            \
+        else                                                                                                          \
+            kv_quant_kernel<LG, false><<<grid, block, 0, st>>>((const u32x4*)x, nchunks, hs, (u32*)q, (f16*)scale,    \
+                                                               (f16*)zero);                                           \
+        break;
+    switch (l2) {
+        QR_KV(1) QR_KV(2) QR_KV(3) QR_KV(4) QR_KV(5)
+    }
+#undef QR_KV
+    return qr_launch_status();
+}
+
+extern "C" int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void* zero, int64_t vectors, int dim,
+                                    void* y, void* stream) {
+    if (vectors < 0) return QR_E_SHAPE;
+    const int l2 = log2_dim(dim);
+    if (l2 < 0) return dim > 0 ? QR_E_UNSUPPORTED : QR_E_SHAPE;
+    if (vectors == 0) return QR_OK;
+    if (!q || !scale || !zero || !y) return QR_E_NULL;
+    if (((uintptr_t)y & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
+    const int64_t nchunks = vectors * (dim / 8);
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(grid_for(nchunks)), block(KT);
+    switch (l2 - 3) {
+        case 1: kv_dequant_kernel<1><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
+        case 2: kv_dequant_kernel<2><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
+        case 3: kv_dequant_kernel<3><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
+        case 4: kv_dequant_kernel<4><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
+        case 5: kv_dequant_kernel<5><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
+    }
+    return qr_launch_status();
+}

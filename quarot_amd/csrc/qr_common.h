@@ -1,0 +1,106 @@
+// Shared device helpers for the gfx950 kernels of libquarot_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/quarot_hip.h"
+
+typedef _Float16 f16;
+typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int u32;
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+#define QR_WAVE 64
+
+static inline int qr_launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? QR_OK : (int)e;
+}
+
+// fp16 bit helpers ---------------------------------------------------------------------------
+__device__ __forceinline__ f16 f16_from_bits(unsigned short b) { return __builtin_bit_cast(f16, b); }
+__device__ __forceinline__ unsigned short f16_bits(f16 h) { return __builtin_bit_cast(unsigned short, h); }
+
+// max over |x| for the 8 halves held in a uint4, as raw magnitudes (sign bit cleared).  Comparing
+// magnitudes as unsigned integers orders finite values and inf correctly and lets a NaN win, which
+// is how torch.max propagates it.
+__device__ __forceinline__ u32 absmax_bits8(u32x4 v) {
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        u32 w = v[i] & 0x7fff7fffu;
+        u32 lo = w & 0xffffu, hi = w >> 16;
+        m = m > lo ? m : lo;
+        m = m > hi ? m : hi;
+    }
+    return m;
+}
+
+__device__ __forceinline__ u32 wave_max_u32(u32 v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        u32 o = (u32)__shfl_xor((int)v, off, QR_WAVE);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+// Quantiser scale: fp16( float(fp16(amax / 7)) * clip ), each step correctly rounded.  The fp32
+// quotient of an fp16 by 7 rounds to fp16 like the exact quotient does (24 >= 2*11 + 2); it is
+// formed in double so no fast-division lowering can touch it.
+__device__ __forceinline__ f16 quantizer_scale(f16 amax, float clip) {
+    f16 s = (f16)(float)((double)(float)amax / 7.0);
+    return (f16)((float)s * clip);
+}
+
+// One code: clamp(round_half_even(fp16(x / s)), -8, 7) with x / s a single correctly rounded fp16
+// division.  `rs` = 1.0f / s (IEEE).  q1 below is x / s to within a fraction of a float ulp
+// (reciprocal, one Newton correction with exact residual); the exact quotient of two fp16 numbers
+// is either an fp16 rounding boundary itself (then q1 is exact, the quotient having <= 12
+// significant bits) or at least 2^-23 away from one in relative terms, more than q1's error, so
+// rounding q1 to fp16 gives the correctly rounded quotient.  s == 0 and non-finite cases take the
+// IEEE division directly.  NaN converts to 0, +-inf saturates and is clamped.
+__device__ __forceinline__ int sym_code(f16 x, float s, float rs, bool fast_ok) {
+    float xf = (float)x;
+    float q;
+    if (fast_ok) {
+        float q0 = xf * rs;
+        float e = __builtin_fmaf(-q0, s, xf);
+        float q1 = __builtin_fmaf(e, rs, q0);
+        q = __builtin_fabsf(q0) < __builtin_inff() ? q1 : q0;   // x = +-inf: keep the infinity
+    } else {
+        q = xf / s;
+    }
+    f16 d = (f16)q;
+    float r = __builtin_rintf((float)d);
+    int c = (int)r;              // v_cvt_i32_f32: NaN -> 0, saturating
+    c = c < -8 ? -8 : c;
+    c = c > 7 ? 7 : c;
+    return (r != r) ? 0 : c;
+}
+
+// 8 fp16 (one 16-byte chunk) -> 8 nibbles in one 32-bit word, element 0 in the lowest nibble.
+__device__ __forceinline__ u32 sym_codes8(u32x4 v, float s, float rs, bool fast_ok) {
+    u32 out = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f16 a = f16_from_bits((unsigned short)(v[i] & 0xffffu));
+        f16 b = f16_from_bits((unsigned short)(v[i] >> 16));
+        u32 ca = (u32)sym_code(a, s, rs, fast_ok) & 0xfu;
+        u32 cb = (u32)sym_code(b, s, rs, fast_ok) & 0xfu;
+        out |= (ca | (cb << 4)) << (8 * i);
+    }
+    return out;
+}
+
+// The reciprocal path is valid when s is a finite non-zero fp16 (then 1/s is a finite float).
+__device__ __forceinline__ bool scale_fast_ok(float s) {
+    float a = __builtin_fabsf(s);
+    return a > 0.0f && a < __builtin_inff();
+}

@@ -1,0 +1,178 @@
+// Symmetric per-token int4 quantiser and the int32 -> fp16 dequantiser (HBM-bound kernels).
+#include "qr_common.h"
+
+namespace {
+
+constexpr int QT = 256;           // threads per workgroup
+
+// One workgroup per row.  NV = 16-byte chunks (8 halves) each thread keeps in registers, so a row
+// of up to 256 * 8 * NV columns is read from HBM exactly once.  GIVEN_SCALE: scale[row] is an
+// input (sym_quant); otherwise it is derived from the row abs-max and written out (Quantizer).
+template <int NV, bool GIVEN_SCALE>
+__global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict__ x, const f16* __restrict__ scale_in,
+                                                        float clip, int cols8, u32* __restrict__ q,
+                                                        f16* __restrict__ scale_out) {
+    __shared__ u32 red[QT / QR_WAVE];
+    const int64_t row = blockIdx.x;
+    const u32x4* xr = x + row * (int64_t)cols8;
+    u32x4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        int c = threadIdx.x + i * QT;
+        v[i] = c < cols8 ? __builtin_nontemporal_load(xr + c) : u32x4{0, 0, 0, 0};
+    }
+    float s;
+    if (GIVEN_SCALE) {
+        s = (float)scale_in[row];
+    } else {
+        u32 m = 0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            u32 mi = absmax_bits8(v[i]);
+            m = m > mi ? m : mi;
+        }
+        m = wave_max_u32(m);
+        if ((threadIdx.x & (QR_WAVE - 1)) == 0) red[threadIdx.x / QR_WAVE] = m;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
+        f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
+        if (threadIdx.x == 0) scale_out[row] = sh;
+        s = (float)sh;
+    }
+    const bool fast = scale_fast_ok(s);
+    const float rs = fast ? 1.0f / s : 0.0f;
+    u32* qr = q + row * (int64_t)cols8;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        int c = threadIdx.x + i * QT;
+        if (c < cols8) qr[c] = sym_codes8(v[i], s, rs, fast);
+    }
+}
+
+// Any column count (odd included), any alignment: one workgroup per row, scalar accesses, the row
+// is read twice when the scale has to be derived.  Used only when the vector kernel's
+// preconditions (cols % 8 == 0, cols <= 32768, 16-byte aligned x, 4-byte aligned q) do not hold.
+template <bool GIVEN_SCALE>
+__global__ __launch_bounds__(QT) void quant_rows_generic_kernel(const f16* __restrict__ x, const f16* __restrict__ scale_in,
+                                                                float clip, int64_t cols, uint8_t* __restrict__ q,
+                                                                f16* __restrict__ scale_out) {
+    __shared__ u32 red[QT / QR_WAVE];
+    const int64_t row = blockIdx.x;
+    const f16* xr = x + row * cols;
+    const int64_t cols_dst = (cols + 1) / 2;
+    float s;
+    if (GIVEN_SCALE) {
+        s = (float)scale_in[row];
+    } else {
+        u32 m = 0;
+        for (int64_t c = threadIdx.x; c < cols; c += QT) {
+            u32 b = f16_bits(xr[c]) & 0x7fffu;
+            m = m > b ? m : b;
+        }
+        m = wave_max_u32(m);
+        if ((threadIdx.x & (QR_WAVE - 1)) == 0) red[threadIdx.x / QR_WAVE] = m;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
+        f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
+        if (threadIdx.x == 0) scale_out[row] = sh;
+        s = (float)sh;
+    }
+    const bool fast = scale_fast_ok(s);
+    const float rs = fast ? 1.0f / s : 0.0f;
+    for (int64_t j = threadIdx.x; j < cols_dst; j += QT) {
+        u32 lo = (u32)sym_code(xr[2 * j], s, rs, fast) & 0xfu;
+        u32 hi = (2 * j + 1 < cols) ? ((u32)sym_code(xr[2 * j + 1], s, rs, fast) & 0xfu) : 0u;
+        q[row * cols_dst + j] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+// y = fp16(fp16(sr * sc) * fp16_rn(q)): 8 columns per thread (two 16-byte loads, one 16-byte store).
+__global__ __launch_bounds__(QT) void dequant_i32_f16_kernel(const int32_t* __restrict__ q, const f16* __restrict__ sr,
+                                                             const f16* __restrict__ sc, int64_t rows, int64_t cols,
+                                                             f16* __restrict__ y, bool vec_ok) {
+    const int64_t cols8 = (cols + 7) / 8;
+    const int64_t total = rows * cols8;
+    for (int64_t idx = (int64_t)blockIdx.x * QT + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * QT) {
+        const int64_t r = idx / cols8;
+        const int64_t c0 = (idx - r * cols8) * 8;
+        const f16 a = sr[r];
+        const int32_t* qp = q + r * cols + c0;
+        f16* yp = y + r * cols + c0;
+        if (vec_ok && c0 + 8 <= cols) {
+            i32x4 q0 = __builtin_nontemporal_load((const i32x4*)qp);
+            i32x4 q1 = __builtin_nontemporal_load((const i32x4*)qp + 1);
+            f16x8 b = *(const f16x8*)(sc + c0);
+            f16x8 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                o[i] = (f16)(a * b[i]) * (f16)(float)q0[i];
+                o[i + 4] = (f16)(a * b[i + 4]) * (f16)(float)q1[i];
+            }
+            __builtin_nontemporal_store(o, (f16x8*)yp);
+        } else {
+            for (int i = 0; i < 8 && c0 + i < cols; ++i) yp[i] = (f16)(a * sc[c0 + i]) * (f16)(float)qp[i];
+        }
+    }
+}
+
+template <bool GIVEN>
+int launch_quant(const void* x, const void* scale_in, float clip, int64_t rows, int64_t cols, void* q, void* scale_out,
+                 hipStream_t st) {
+    if (rows == 0 || cols == 0) return QR_OK;
+    const bool vec = (cols % 8 == 0) && cols <= 32768 && (((uintptr_t)x & 15) == 0) && (((uintptr_t)q & 3) == 0);
+    dim3 grid((unsigned)rows), block(QT);
+    if (rows > 0x7fffffffLL) return QR_E_SHAPE;
+    if (!vec) {
+        quant_rows_generic_kernel<GIVEN><<<grid, block, 0, st>>>((const f16*)x, (const f16*)scale_in, clip, cols,
+                                                                  (uint8_t*)q, (f16*)scale_out);
+        return qr_launch_status();
+    }
+    const int cols8 = (int)(cols / 8);
+    const int nv = (cols8 + QT - 1) / QT;
+#define QR_LAUNCH(NV)                                                                                                  \
+    quant_rows_kernel<NV, GIVEN><<<grid, block, 0, st>>>((const u32x4*)x, (const f16*)scale_in, clip, cols8, (u32*)q, \
+                                                         (f16*)scale_out)
+    if (nv <= 1) QR_LAUNCH(1);
+    else if (nv <= 2) QR_LAUNCH(2);
+    else if (nv <= 4) QR_LAUNCH(4);
+    else if (nv <= 6) QR_LAUNCH(6);
+    else if (nv <= 8) QR_LAUNCH(8);
+    else QR_LAUNCH(16);
+#undef QR_LAUNCH
+    return qr_launch_status();
+}
+
+}  // namespace
+
+extern "C" int qr_sym_quant_f16_i4(const void* x, const void* scale, int64_t rows, int64_t cols, void* q, void* stream) {
+    if (rows < 0 || cols < 0) return QR_E_SHAPE;
+    if (rows == 0 || cols == 0) return QR_OK;
+    if (!x || !scale || !q) return QR_E_NULL;
+    return launch_quant<true>(x, scale, 1.0f, rows, cols, q, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, int64_t cols, void* q, void* scales,
+                                       void* stream) {
+    if (rows < 0 || cols < 0) return QR_E_SHAPE;
+    if (rows == 0) return QR_OK;
+    if (cols == 0) return QR_E_SHAPE;   // torch.max over an empty axis raises in the reference
+    if (!x || !q || !scales) return QR_E_NULL;
+    return launch_quant<false>(x, nullptr, clip, rows, cols, q, scales, (hipStream_t)stream);
+}
+
+extern "C" int qr_sym_dequant_i32_f16(const void* q, const void* scale_row, const void* scale_col, int64_t rows,
+                                      int64_t cols, void* y, void* stream) {
+    if (rows < 0 || cols < 0) return QR_E_SHAPE;
+    if (rows == 0 || cols == 0) return QR_OK;
+    if (!q || !scale_row || !scale_col || !y) return QR_E_NULL;
+    const bool vec_ok = (cols % 8 == 0) && (((uintptr_t)q & 15) == 0) && (((uintptr_t)y & 15) == 0) &&
+                        (((uintptr_t)scale_col & 15) == 0);
+    const int64_t total = rows * ((cols + 7) / 8);
+    int64_t blocks = (total + QT - 1) / QT;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    dequant_i32_f16_kernel<<<dim3((unsigned)blocks), dim3(QT), 0, (hipStream_t)stream>>>(
+        (const int32_t*)q, (const f16*)scale_row, (const f16*)scale_col, rows, cols, (f16*)y, vec_ok);
+    return qr_launch_status();
+}

@@ -1,0 +1,46 @@
+import torch
+
+import quarot_amd
+
+
+class OnlineHadamard(torch.nn.Module):
+    """Online Hadamard over the last axis (quarot/nn/hadamard.py:5-23): buffer `had_rem_dim` holds
+    the non-power-of-two factor (fp16 unless force_fp32), None for power-of-two widths."""
+
+    def __init__(self, hadamard_dim, force_fp32=False):
+        super().__init__()
+        self.fp32_had = force_fp32
+        had_rem_dim, self.rem_dim = quarot_amd.functional.hadamard.get_hadK(hadamard_dim)
+        if had_rem_dim is not None:
+            self.register_buffer("had_rem_dim", had_rem_dim)
+            if not self.fp32_had:
+                self.had_rem_dim = self.had_rem_dim.to(torch.float16)
+        else:
+            self.had_rem_dim = None
+
+    def forward(self, x):
+        x_dtype = x.dtype
+        if self.fp32_had:
+            x = x.float()
+        x = quarot_amd.functional.matmul_hadU_cuda(x, self.had_rem_dim, self.rem_dim)
+        return x.to(x_dtype)
+
+
+class OnlineHadamardQuantizer(torch.nn.Module):
+    """Sequential(OnlineHadamard(dim, force_fp32), Quantizer(clip)) in one kernel: same codes and
+    scales, without the transformed fp16 tensor going through HBM.  Same buffer name, so a
+    state-dict written for the two-module form loads."""
+
+    def __init__(self, hadamard_dim, force_fp32=False, input_clip_ratio=1.0):
+        super().__init__()
+        self.fp32_had = force_fp32
+        self.input_clip_ratio = input_clip_ratio
+        had_rem_dim, self.rem_dim = quarot_amd.functional.hadamard.get_hadK(hadamard_dim)
+        if had_rem_dim is not None:
+            self.register_buffer("had_rem_dim", had_rem_dim if force_fp32 else had_rem_dim.to(torch.float16))
+        else:
+            self.had_rem_dim = None
+
+    def forward(self, x):
+        return quarot_amd.hadamard_quantize(x, self.had_rem_dim, self.rem_dim, self.input_clip_ratio,
+                                            force_fp32=self.fp32_had)
