@@ -9,11 +9,13 @@
 // 256 * (the int4 dot product); an arithmetic shift by 8 at the end restores it.  Even and odd k
 // go to different MFMA issues; that permutation of k is the same for A and B, so dot products are
 // unchanged.  |acc| <= 256 * 64 * K requires K < 131072.
+//
+// The MFMA's first operand is the W (B-matrix) fragment and its second the X (A-matrix) fragment,
+// so in the 32x32 accumulator a lane owns one token (m = lane % 32) and runs of 4 consecutive
+// output features n: stores are 8 bytes (fp16) or 16 bytes (int32) per lane.
 #include "qr_common.h"
 
 namespace {
-
-constexpr int GT = 256;     // threads per workgroup (4 waves)
 
 // LDS holds, per stage, (BM + BN) rows of 64 packed bytes (128 k values) as four 16-byte chunks.
 // The chunk position is XOR-swizzled with bits 2..3 of the row so that the 16 rows a quarter-wave
@@ -21,16 +23,15 @@ constexpr int GT = 256;     // threads per workgroup (4 waves)
 __device__ __forceinline__ int lds_slot(int row, int chunk) { return row * 4 + (chunk ^ ((row >> 2) & 3)); }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
-__global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
-                                                     int M, int N, int Kb, int32_t* __restrict__ C,
-                                                     f16* __restrict__ Y, const f16* __restrict__ sA,
-                                                     const f16* __restrict__ sB, const f16* __restrict__ bias,
-                                                     int tiles_m, int tiles_n) {
-    static_assert(WAVES_M * WAVES_N == GT / QR_WAVE, "four waves");
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
+    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
+    int tiles_m, int tiles_n) {
+    constexpr int NT = 64 * WAVES_M * WAVES_N;              // threads per workgroup
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;     // per-wave output tile
     constexpr int IM = TM / 32, JN = TN / 32;               // 32x32 MFMA tiles per wave
     constexpr int CH = (BM + BN) * 4;                       // 16-byte chunks per stage
-    constexpr int NL = (CH + GT - 1) / GT;                  // chunks each thread moves per stage
+    constexpr int NL = (CH + NT - 1) / NT;                  // chunks each thread moves per stage
     static_assert(TM % 32 == 0 && TN % 32 == 0, "tile shape");
     __shared__ u32x4 lds[2][CH];
 
@@ -53,15 +54,14 @@ __global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-    // Global -> LDS staging: chunk id = tid + i * GT; 4 consecutive threads fetch one row's 64 bytes.
+    // Global -> LDS staging: chunk id = tid + i * NT; 4 consecutive threads fetch one row's 64 bytes.
     // Rows beyond M (or N) are clamped to the last valid row: they are read but never stored.
     const uint8_t* src[NL];
     int dst[NL];
-    int coff[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        int qid = tid + i * GT;
-        if (qid >= CH) qid = CH - 1;        // (BM + BN) * 4 not a multiple of 256: the tail repeats the last chunk
+        int qid = tid + i * NT;
+        if (qid >= CH) qid = CH - 1;        // CH not a multiple of NT: the tail repeats the last chunk
         const int row = qid >> 2, c = qid & 3;
         if (row < BM) {
             int gr = m0 + row;
@@ -72,7 +72,6 @@ __global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__
             gr = gr < N ? gr : N - 1;
             src[i] = B + (int64_t)gr * Kb + c * 16;
         }
-        coff[i] = c * 16;
         dst[i] = lds_slot(row, c);
     }
 
@@ -84,81 +83,123 @@ __global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
-    const int ksteps = (Kb + 63) / 64;
-    u32x4 pre[NL];
-#pragma unroll
-    for (int i = 0; i < NL; ++i)
-        pre[i] = (coff[i] < Kb) ? *(const u32x4*)(src[i]) : u32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < NL; ++i) lds[0][dst[i]] = pre[i];
-    __syncthreads();
-
     const int arow = wm * TM + (lane & 31);
     const int brow = BM + wn * TN + (lane & 31);
     const int khalf = lane >> 5;
 
-    for (int ks = 0; ks < ksteps; ++ks) {
-        const bool more = ks + 1 < ksteps;
-        if (more) {
-            const int kb = (ks + 1) * 64;
-#pragma unroll
-            for (int i = 0; i < NL; ++i)
-                pre[i] = (kb + coff[i] < Kb) ? *(const u32x4*)(src[i] + kb) : u32x4{0, 0, 0, 0};
-        }
-        const u32x4* buf = lds[ks & 1];
+    // One stage = 64 packed bytes per row = two sub-steps of 64 k values (two MFMA issues each).
+    auto compute = [&](const u32x4* buf, int nsub) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
+            if (s < nsub) {
+                i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
 #pragma unroll
-            for (int i = 0; i < IM; ++i) {
-                u32x4 p = buf[lds_slot(arow + i * 32, s * 2 + khalf)];
-                alo[i] = (i32x4)((p << 4) & 0xF0F0F0F0u);
-                ahi[i] = (i32x4)(p & 0xF0F0F0F0u);
-            }
-#pragma unroll
-            for (int j = 0; j < JN; ++j) {
-                u32x4 p = buf[lds_slot(brow + j * 32, s * 2 + khalf)];
-                blo[j] = (i32x4)((p << 4) & 0xF0F0F0F0u);
-                bhi[j] = (i32x4)(p & 0xF0F0F0F0u);
-            }
-#pragma unroll
-            for (int i = 0; i < IM; ++i)
+                for (int i = 0; i < IM; ++i) {
+                    u32x4 p = buf[lds_slot(arow + i * 32, s * 2 + khalf)];
+                    alo[i] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+                    ahi[i] = (i32x4)(p & 0xF0F0F0F0u);
+                }
 #pragma unroll
                 for (int j = 0; j < JN; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo[i], blo[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi[i], bhi[j], acc[i][j], 0, 0, 0);
+                    u32x4 p = buf[lds_slot(brow + j * 32, s * 2 + khalf)];
+                    blo[j] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+                    bhi[j] = (i32x4)(p & 0xF0F0F0F0u);
                 }
+#pragma unroll
+                for (int i = 0; i < IM; ++i)
+#pragma unroll
+                    for (int j = 0; j < JN; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo[j], alo[i], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bhi[j], ahi[i], acc[i][j], 0, 0, 0);
+                    }
+            }
         }
+    };
+
+    // K % 64 == 0, so a row is a whole number of 32-byte half-stages: `full` whole stages, then
+    // possibly one half stage (chunks 0 and 1 only).
+    const int full = Kb / 64;
+    const bool half_tail = (Kb & 63) != 0;
+    u32x4 pre[NL];
+    if (full > 0) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) pre[i] = *(const u32x4*)(src[i]);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) lds[0][dst[i]] = pre[i];
+    }
+    __syncthreads();
+    for (int ks = 0; ks < full; ++ks) {
+        const bool more = ks + 1 < full;
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                src[i] += 64;
+                pre[i] = *(const u32x4*)(src[i]);
+            }
+        }
+        compute(lds[ks & 1], 2);
         if (more) {
 #pragma unroll
             for (int i = 0; i < NL; ++i) lds[(ks + 1) & 1][dst[i]] = pre[i];
         }
         __syncthreads();
     }
-
-    // Epilogue.  32x32 accumulator layout: lane l, register v -> row (v/4)*8 + (l/32)*4 + v%4, column l%32.
+    if (half_tail) {
+        // chunks 2 and 3 of this last stage lie beyond the row: only chunks 0/1 are fetched and used
 #pragma unroll
-    for (int j = 0; j < JN; ++j) {
-        const int col = n0 + wn * TN + j * 32 + (lane & 31);
-        if (col >= N) continue;
-        f16 sb = (f16)0, bb = (f16)0;
-        if (DEQ) {
-            sb = sB[col];
-            if (bias) bb = bias[col];
+        for (int i = 0; i < NL; ++i) {
+            int qid = tid + i * NT;
+            if (qid >= CH) qid = CH - 1;
+            if ((qid & 3) < 2) lds[0][dst[i]] = *(const u32x4*)(src[i] + (full > 0 ? 64 : 0));
         }
+        __syncthreads();
+        compute(lds[0], 1);
+    }
+
+    // Epilogue.  Accumulator layout (first operand = W rows, second = X rows): lane l, register v ->
+    // n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
 #pragma unroll
-        for (int i = 0; i < IM; ++i) {
+    for (int i = 0; i < IM; ++i) {
+        const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (row >= M) continue;
+        f16 sa = (f16)0;
+        if (DEQ) sa = sA[row];
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = m0 + wm * TM + i * 32 + (v >> 2) * 8 + khalf * 4 + (v & 3);
-                if (row >= M) continue;
-                const int val = acc[i][j][v] >> 8;
+        for (int j = 0; j < JN; ++j) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
+                if (col >= N) continue;
+                int v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
+                const bool whole = (col + 4 <= N) && ((N & 3) == 0);
                 if (DEQ) {
-                    f16 yv = (f16)(sA[row] * sb) * (f16)(float)val;
-                    if (bias) yv = yv + bb;
-                    Y[(int64_t)row * N + col] = yv;
+                    f16 o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int cc = col + e < N ? col + e : N - 1;
+                        f16 yv = (f16)(sa * sB[cc]) * (f16)(float)v4[e];
+                        if (bias) yv = yv + bias[cc];
+                        o[e] = yv;
+                    }
+                    f16* yp = Y + (int64_t)row * N + col;
+                    if (whole) {
+                        *(f16x4*)yp = f16x4{o[0], o[1], o[2], o[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < N) yp[e] = o[e];
+                    }
                 } else {
-                    C[(int64_t)row * N + col] = val;
+                    int32_t* cp = C + (int64_t)row * N + col;
+                    if (whole) {
+                        *(i32x4*)cp = i32x4{v4[0], v4[1], v4[2], v4[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < N) cp[e] = v4[e];
+                    }
                 }
             }
         }
@@ -168,16 +209,17 @@ __global__ __launch_bounds__(GT) void gemm_i4_kernel(const uint8_t* __restrict__
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st) {
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     if (Y)
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(GT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, (const f16*)sA, (const f16*)sB,
             (const f16*)bias, tiles_m, tiles_n);
     else
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(GT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr, nullptr, nullptr, nullptr, tiles_m,
             tiles_n);
     return qr_launch_status();
@@ -190,13 +232,14 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (K == 0 || K % 64 != 0 || K > 131008 || M > 0x7fffffff || N > 0x7fffffff) return QR_E_SHAPE;
     if (!A || !B || (!C && !Y)) return QR_E_NULL;
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return QR_E_ALIGN;
+    if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     if (M <= 32) return launch_cfg<32, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     if (M <= 64) return launch_cfg<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    if (t256 >= 512) return launch_cfg<256, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 256) return launch_cfg<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t128x256 >= 256) return launch_cfg<128, 256, 2, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
 

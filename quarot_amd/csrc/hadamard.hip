@@ -76,7 +76,7 @@ __device__ __forceinline__ u32x4 to_f16x8(const float (&v)[8]) {
     u32x4 o;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-        o[i] = (u32)f16_bits((f16)v[2 * i]) | ((u32)f16_bits((f16)v[2 * i + 1]) << 16);
+        o[i] = (u32)f16_bits(narrow_f16(v[2 * i])) | ((u32)f16_bits(narrow_f16(v[2 * i + 1])) << 16);
     return o;
 }
 
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(HT) void hadamard_kernel(const IO* __restrict__ x, 
                         const int k = ks * 32 + kq * 8 + j;
                         float t = 0.f;
                         if (ks < ksteps && k < K && rin) t = buf[k * m + r] * scale;
-                        f16 hi = (f16)t;
+                        f16 hi = narrow_f16(t);
                         bh[ks][j] = hi;
                         if (MODE32) bl[ks][j] = (f16)(t - (float)hi);
                     }

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
             if (LG > 3) kv_butterfly<8>(v, lane);
             if (LG > 4) kv_butterfly<16>(v, lane);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (float)(f16)(v[e] * hscale);   // the transform's fp16 output
+            for (int e = 0; e < 8; ++e) v[e] = (float)narrow_f16(v[e] * hscale);   // the transform's fp16 output
         }
         float mn = v[0], mx = v[0];
 #pragma unroll

@@ -27,6 +27,15 @@ static inline int qr_launch_status() {
 __device__ __forceinline__ f16 f16_from_bits(unsigned short b) { return __builtin_bit_cast(f16, b); }
 __device__ __forceinline__ unsigned short f16_bits(f16 h) { return __builtin_bit_cast(unsigned short, h); }
 
+// Narrow a value that must FIRST be rounded to fp32 (the reference multiplies in fp32, then casts).
+// The empty asm hides the producer from the optimiser, which otherwise folds "multiply, then
+// convert" into v_fma_mixlo_f16: that instruction rounds the exact product once, and differs from
+// the two-step result in rare double-rounding cases.
+__device__ __forceinline__ f16 narrow_f16(float v) {
+    asm("" : "+v"(v));
+    return (f16)v;
+}
+
 // max over |x| for the 8 halves held in a uint4, as raw magnitudes (sign bit cleared).  Comparing
 // magnitudes as unsigned integers orders finite values and inf correctly and lets a NaN win, which
 // is how torch.max propagates it.
@@ -56,7 +65,7 @@ __device__ __forceinline__ u32 wave_max_u32(u32 v) {
 // formed in double so no fast-division lowering can touch it.
 __device__ __forceinline__ f16 quantizer_scale(f16 amax, float clip) {
     f16 s = (f16)(float)((double)(float)amax / 7.0);
-    return (f16)((float)s * clip);
+    return narrow_f16((float)s * clip);
 }
 
 // One code: clamp(round_half_even(fp16(x / s)), -8, 7) with x / s a single correctly rounded fp16

@@ -1,0 +1,79 @@
+"""The C ABI: the shared library loads and exports exactly what include/quarot_hip.h declares.
+No kernel is launched here; argument errors are returned before any launch."""
+import ctypes
+import pathlib
+import re
+
+import pytest
+
+from quarot_amd import _lib
+
+ROOT = pathlib.Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "quarot_hip.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not _lib.LIB_PATH.exists():          # built beforehand normally; build only if nothing is there
+        from quarot_amd import build
+        build.build(verbose=False)
+    return _lib.lib()
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(qr_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    syms = declared_symbols()
+    for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
+                 "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
+                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in declared_symbols():
+        assert hasattr(raw, name), name
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+
+
+def test_version_and_error_text(lib):
+    assert lib.qr_version() >= 100
+    assert lib.qr_strerror(0) == b"success"
+    for code in (-1, -2, -3, -4, -5):
+        assert len(lib.qr_strerror(code)) > 5
+    assert b"unknown" in lib.qr_strerror(-99)
+
+
+def test_argument_errors_are_returned_before_any_launch(lib):
+    one = ctypes.c_void_p(16)       # never dereferenced: every call below must fail validation first
+    assert lib.qr_matmul_i4_i32(one, one, 4, 4, 100, one, None) == -2          # K % 64 != 0
+    assert lib.qr_matmul_i4_i32(one, one, 4, 4, 1 << 18, one, None) == -2      # accumulator would overflow
+    assert lib.qr_matmul_i4_i32(None, one, 4, 4, 64, one, None) == -1
+    assert lib.qr_matmul_i4_i32(ctypes.c_void_p(8), one, 4, 4, 64, one, None) == -4
+    assert lib.qr_matmul_i4_i32(one, one, 0, 4, 64, None, None) == 0           # empty: nothing to do
+    assert lib.qr_matmul_i4_i32(one, one, -1, 4, 64, one, None) == -2
+    assert lib.qr_linear_i4_f16(one, None, one, one, None, 4, 4, 64, one, None) == -1
+    assert lib.qr_sym_quant_f16_i4(None, one, 3, 8, one, None) == -1
+    assert lib.qr_sym_quant_f16_i4(one, one, 0, 8, one, None) == 0
+    assert lib.qr_quantize_rows_f16_i4(one, 1.0, 3, 0, one, one, None) == -2   # max over an empty axis
+    assert lib.qr_sym_dequant_i32_f16(one, one, None, 2, 2, one, None) == -1
+    assert lib.qr_hadamard(one, one, 2, 100, 1, None, 0, 1.0, None) == -2      # not a power of two
+    assert lib.qr_hadamard(one, one, 2, 172 * 3, 172, one, 0, 1.0, None) == -2
+    assert lib.qr_hadamard(one, one, 2, 1 << 16, 1, None, 0, 1.0, None) == -3  # longer than one workgroup's LDS
+    assert lib.qr_hadamard(one, one, 2, 64, 1, None, 7, 1.0, None) == -5
+    assert lib.qr_hadamard(one, one, 2, 11008, 172, None, 0, 1.0, None) == -1  # hadK missing
+    assert lib.qr_hadamard_quantize_f16_i4(one, 2, 64, 1, None, 0, 1.0, 1.0, None, one, None, None) == -1
+    assert lib.qr_kv_quant_f16_i4(one, 4, 100, 0, one, one, one, None) == -3
+    assert lib.qr_kv_quant_f16_i4(one, 4, 128, 3, one, one, one, None) == -5
+    assert lib.qr_kv_dequant_i4_f16(one, one, one, 0, 128, one, None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()

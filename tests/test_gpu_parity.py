@@ -1,0 +1,402 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI (ctypes) and the Python mirror
+of the reference interface.  Bars: int4 codes, scales, int32 accumulators and fp16 dequantised
+values BIT-EXACT; Hadamard outputs within rtol 1e-3 / atol 1e-3 of the oracle."""
+import numpy as np
+import pytest
+import torch
+
+import quarot_amd
+from oracle import quarot_oracle as o
+from quarot_amd import _lib
+from quarot_amd.transformers import kv_cache as kv
+
+pytestmark = pytest.mark.gpu
+F16, F32 = np.float16, np.float32
+RTOL = ATOL = 1e-3
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def gpu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev())
+
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint16)
+
+
+def synth_x(m, k, seed=0, outliers=True):
+    """Activations of the benchmark configs: N(0,1) with 1 % of channels scaled by 20."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g)
+    if outliers:
+        idx = torch.randperm(k, generator=g)[: -(-k // 100)]
+        x[:, idx] *= 20
+    return x.half().numpy()
+
+
+def synth_w(n, k, seed=1):
+    """Weights: N(0, 0.02), per-row fp16 scale amax/7, round-to-nearest codes, packed."""
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(n, k, generator=g) * 0.02).half().numpy()
+    s = (np.max(np.abs(w), axis=1, keepdims=True).astype(F32) / F32(7)).astype(F16)
+    codes = np.clip(np.rint((w.astype(F32) / s.astype(F32)).astype(F16).astype(F32)), -8, 7).astype(np.int8)
+    return o.pack_i4(codes), s
+
+
+# ------------------------------------------------------------------------------ quantiser
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (5, 64), (33, 4096), (16, 11008), (7, 28672), (4, 32768), (2048, 4096),
+                                       (9, 37), (3, 7), (2, 1), (6, 40000), (5, 12)])
+def test_quantizer_codes_and_scales_bit_exact(rows, cols):
+    x = synth_x(rows, cols, seed=rows * 7 + cols) * F16(1.7)
+    for clip in (1.0, 0.9):
+        q, s = quarot_amd.quantize_rows(gpu(x), clip)
+        wq, ws = o.quantizer(x, clip)
+        assert q.shape == (rows, (cols + 1) // 2) and s.shape == (rows, 1)
+        assert np.array_equal(s.cpu().numpy().reshape(-1), ws)
+        assert np.array_equal(q.cpu().numpy(), wq)
+
+
+def test_quantizer_module_shapes_follow_reference_quirk():
+    x = gpu(synth_x(6 * 5, 64).reshape(6, 5, 64))
+    p = quarot_amd.nn.Quantizer()(x)
+    assert p.quantized_x.shape == (6, 5, 32)
+    assert p.scales_x.shape == (6, 1, 5)            # max(dim=-1)[0].unsqueeze(1) on a 3-D input
+    wq, ws = o.quantizer(x.cpu().numpy().reshape(30, 64))
+    assert np.array_equal(p.quantized_x.cpu().numpy().reshape(30, 32), wq)
+    assert np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+
+
+def test_quantizer_zero_rows_and_extremes():
+    x = np.zeros((4, 64), F16)
+    x[1, 3] = 65504
+    x[2, :] = -65504
+    x[3, 0] = 6e-8          # smallest subnormal: scale rounds to 0 -> division by zero -> +inf -> 7
+    q, s = quarot_amd.quantize_rows(gpu(x))
+    wq, ws = o.quantizer(x)
+    assert np.array_equal(s.cpu().numpy().reshape(-1), ws) and np.array_equal(q.cpu().numpy(), wq)
+    assert not q.cpu().numpy()[0].any()
+
+
+def test_scale_for_every_finite_fp16_amax():
+    v = np.arange(65536, dtype=np.uint16).view(F16)
+    v = v[np.isfinite(v)]
+    x = np.zeros((v.size, 8), F16)
+    x[:, 5] = v
+    for clip in (1.0, 0.85):
+        _, s = quarot_amd.quantize_rows(gpu(x), clip)
+        assert np.array_equal(s.cpu().numpy().reshape(-1), o.quantizer_scales(x, clip))
+
+
+def test_sym_quant_every_fp16_value_times_many_scales():
+    """Brute force of the division + rounding: all finite fp16 x against 240 scales (ties, values
+    that round up into a tie, subnormal quotients, overflow), plus zero / inf / NaN scales."""
+    v = np.arange(65536, dtype=np.uint16).view(F16)
+    v = v[np.isfinite(v)].reshape(2, -1)                                   # 2 x 31744
+    rng = np.random.default_rng(0)
+    scales = np.concatenate([
+        np.abs(rng.standard_normal(100)).astype(F16) + F16(1e-3),
+        (2.0 ** rng.integers(-14, 12, 40)).astype(F16),
+        rng.integers(1, 65536, 80).astype(np.uint16).view(F16),           # arbitrary bit patterns
+        np.array([0.0, -0.0, np.inf, -np.inf, 6e-8, 65504, -1.5, 1 / 3, 7.0, 1 / 7, np.nan, 0.3, 3e-5, -2e-4, 1e-3,
+                  0.1, 0.7, 1.1, 13.0, 100.0], F16)])
+    x = np.tile(v, (scales.size, 1))
+    s = np.repeat(scales, 2)
+    got = quarot_amd.sym_quant(gpu(x), gpu(s)).cpu().numpy()
+    finite_scale = np.isfinite(s) | np.isinf(s)
+    want = o.pack_i4(o.sym_quant_codes(x, s))
+    assert np.array_equal(got[finite_scale], want[finite_scale])
+    # NaN scale: every quotient is NaN -> code 0
+    assert not got[~finite_scale].any()
+
+
+def test_sym_quant_odd_columns_and_views():
+    x = synth_x(11, 75, seed=3)
+    s = o.quantizer_scales(x)
+    got = quarot_amd.sym_quant(gpu(x), gpu(s).view(11, 1))
+    assert got.shape == (11, 38)
+    assert np.array_equal(got.cpu().numpy(), o.pack_i4(o.sym_quant_codes(x, s)))
+    x3 = gpu(x[:10, :64].copy()).view(2, 5, 64)
+    got3 = quarot_amd.sym_quant(x3, gpu(s[:10]).view(2, 5))
+    assert got3.shape == (2, 5, 32)
+    with pytest.raises(RuntimeError):
+        quarot_amd.sym_quant(gpu(x), gpu(s[:5]))                            # scale size mismatch
+    with pytest.raises(RuntimeError):
+        quarot_amd.sym_quant(gpu(x).t().contiguous().t(), gpu(s))           # not contiguous -> view fails
+
+
+# ------------------------------------------------------------------------------ GEMM / dequant / linear
+
+GEMM_SHAPES = [(1, 1, 64), (32, 32, 64), (33, 65, 128), (64, 64, 192), (100, 200, 192), (128, 128, 256), (1, 256, 4096),
+               (8, 300, 1024), (40, 512, 512), (64, 1000, 2048), (65, 256, 320), (129, 257, 448), (256, 512, 4096),
+               (300, 700, 11008), (512, 1024, 2048), (1000, 3000, 1024), (2048, 4096, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_matmul_int32_bit_exact(m, n, k):
+    rng = np.random.default_rng(m * 31 + n * 7 + k)
+    a = o.pack_i4(rng.integers(-8, 8, (m, k)))
+    b = o.pack_i4(rng.integers(-8, 8, (n, k)))
+    c = quarot_amd.matmul(gpu(a), gpu(b))
+    assert c.dtype == torch.int32 and c.shape == (m, n)
+    assert np.array_equal(c.cpu().numpy(), o.int4_matmul(a, b))
+
+
+def test_matmul_known_answers_and_leading_dims():
+    k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
+    a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
+    b = np.full((5, k // 2), 0x88, np.uint8)
+    assert (quarot_amd.matmul(gpu(a), gpu(b)).cpu().numpy() == 64 * k).all()
+    b7 = np.full((5, k // 2), 0x77, np.uint8)      # all 7
+    assert (quarot_amd.matmul(gpu(a), gpu(b7)).cpu().numpy() == -56 * k).all()
+    rng = np.random.default_rng(1)
+    a3 = o.pack_i4(rng.integers(-8, 8, (6, 128))).reshape(2, 3, 64)
+    b2 = o.pack_i4(rng.integers(-8, 8, (7, 128)))
+    c = quarot_amd.matmul(gpu(a3), gpu(b2))
+    assert c.shape == (2, 3, 7)
+    assert np.array_equal(c.cpu().numpy().reshape(6, 7), o.int4_matmul(a3.reshape(6, 64), b2))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 13), (64, 64), (100, 4096), (33, 1000), (2048, 4096)])
+def test_sym_dequant_bit_exact(rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    q = rng.integers(-70000, 70000, (rows, cols)).astype(np.int32)          # crosses 2048 (11-bit) and 65520 (inf)
+    q.reshape(-1)[:4] = [2049, 65519, 65520, -(1 << 30)][: min(4, q.size)]
+    sr = (np.abs(rng.standard_normal(rows)) * 0.1).astype(F16)
+    sc = (np.abs(rng.standard_normal(cols)) * 0.01).astype(F16)
+    y = quarot_amd.sym_dequant(gpu(q), gpu(sr).view(rows, 1), gpu(sc).view(cols, 1))
+    assert y.dtype == torch.float16 and y.shape == (rows, cols)
+    assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(q, sr, sc)))
+    with pytest.raises(RuntimeError, match="Unsupported"):
+        quarot_amd.sym_dequant(gpu(q), gpu(sr), gpu(sc), bits=8)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (33, 65, 128), (64, 512, 1024), (100, 200, 192), (300, 700, 11008),
+                                   (512, 1024, 2048), (2048, 4096, 4096)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_linear_fused_equals_staged_reference_ops(m, n, k, with_bias):
+    rng = np.random.default_rng(m + n + k)
+    a = o.pack_i4(rng.integers(-8, 8, (m, k)))
+    w = o.pack_i4(rng.integers(-8, 8, (n, k)))
+    sa = (np.abs(rng.standard_normal(m)) * 0.2).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01).astype(F16)
+    bias = rng.standard_normal(n).astype(F16) if with_bias else None
+    y = quarot_amd.linear_i4(gpu(a), gpu(sa).view(m, 1), gpu(w), gpu(sw).view(n, 1), None if bias is None else gpu(bias))
+    want = o.linear4bit(a, sa, w, sw, bias)
+    assert np.array_equal(bits(y.cpu().numpy()), bits(want))
+    # and equals the staged calls of the reference API
+    staged = quarot_amd.sym_dequant(quarot_amd.matmul(gpu(a), gpu(w)), gpu(sa), gpu(sw).view(n, 1))
+    if bias is not None:
+        staged = staged + gpu(bias)
+    assert torch.equal(staged, y)
+
+
+def test_linear4bit_module_from_float_and_state_dict():
+    w = (torch.randn(96, 128, generator=torch.Generator().manual_seed(4)) * 0.02).half()
+    s = (w.abs().amax(dim=1, keepdim=True) / 7).half()
+    lin = torch.nn.Linear(128, 96, bias=True).half()
+    lin.weight.data = w
+    lin.bias.data = torch.randn(96, generator=torch.Generator().manual_seed(5)).half()
+    q4 = quarot_amd.nn.Linear4bit.from_float(lin, weight_scales=s).cuda()
+    assert np.array_equal(q4.weight.cpu().numpy(), o.weight_codes_from_float(w.numpy(), s.numpy()))
+    x = gpu(synth_x(10, 128, seed=6))
+    seq = torch.nn.Sequential(quarot_amd.nn.Quantizer(), q4)
+    y = seq(x)
+    xq, xs = o.quantizer(x.cpu().numpy())
+    want = o.linear4bit(xq, xs, q4.weight.cpu().numpy(), s.numpy(), lin.bias.data.numpy())
+    assert np.array_equal(bits(y.cpu().numpy()), bits(want))
+    clone = quarot_amd.nn.Linear4bit(128, 96, bias=True).half().cuda()   # buffers are fp32 until cast, as in the reference
+    clone.load_state_dict(q4.state_dict())
+    assert torch.equal(clone(quarot_amd.nn.Quantizer()(x)), y)
+
+
+# ------------------------------------------------------------------------------ Hadamard
+
+HAD_SIZES = [8, 64, 128, 512, 1024, 4096, 8192, 32768, 96, 224, 320, 1376, 5120, 11008, 13824, 14336, 28672]
+
+
+def close(got, want):
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    return np.all(np.abs(g - w) <= ATOL + RTOL * np.abs(w))
+
+
+@pytest.mark.parametrize("n", HAD_SIZES)
+@pytest.mark.parametrize("dtype", [F16, F32])
+def test_hadamard_within_tolerance(n, dtype):
+    x = (synth_x(6, n, seed=n) if dtype == F16 else synth_x(6, n, seed=n).astype(F32) * F32(1.001))
+    hadk, k = quarot_amd.functional.hadamard.get_hadK(n)
+    y = quarot_amd.functional.matmul_hadU_cuda(gpu(x), None if hadk is None else hadk.cuda(), k)
+    assert y.dtype == (torch.float16 if dtype == F16 else torch.float32) and y.shape == (6, n)
+    ho, ko = o.get_hadK(n)
+    got = y.cpu().numpy()
+    assert close(got, o.hadamard_staged(x, ho, ko, dtype))
+    # float64 closed form: the transform itself (kron orientation, natural order, scale)
+    cf = o.hadamard_closed_form(x.astype(np.float64))
+    tol = 3e-3 if dtype == F16 else 1e-5
+    assert np.all(np.abs(got - cf) <= tol * (1 + np.abs(cf)))
+
+
+@pytest.mark.parametrize("n", [64, 4096, 8192, 224, 11008, 28672, 13824])
+@pytest.mark.parametrize("fp32", [False, True])
+def test_fused_hadamard_quantize_equals_staged(n, fp32):
+    x = gpu(synth_x(9, n, seed=n + 1))
+    had = quarot_amd.nn.OnlineHadamard(n, force_fp32=fp32).cuda()
+    fused = quarot_amd.nn.OnlineHadamardQuantizer(n, force_fp32=fp32, input_clip_ratio=0.95).cuda()
+    y = had(x)                                                     # the kernel's own fp16 Hadamard output
+    p = fused(x)
+    wq, ws = o.quantizer(y.cpu().numpy(), 0.95)                    # oracle quantiser on that output
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    assert np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+    staged = quarot_amd.nn.Quantizer(0.95)(y)
+    assert torch.equal(staged.quantized_x, p.quantized_x) and torch.equal(staged.scales_x, p.scales_x)
+    p2, y2 = quarot_amd.hadamard_quantize(x, fused.had_rem_dim, fused.rem_dim, 0.95, force_fp32=fp32, return_transformed=True)
+    assert torch.equal(y2, y) and torch.equal(p2.quantized_x, p.quantized_x)
+    ho, ko = o.get_hadK(n)
+    assert close(y.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
+
+
+def test_hadamard_full_size_properties():
+    """Benchmark-size rows (2048 x 11008 and 2048 x 4096): norm preservation, linearity in a row
+    scaling by 2 (exact in floating point), power-of-two transform is an involution."""
+    for n in (11008, 4096):
+        x = gpu(synth_x(2048, n, seed=0))
+        had = quarot_amd.nn.OnlineHadamard(n).cuda()
+        y = had(x)
+        nx, ny = x.float().norm(dim=1), y.float().norm(dim=1)
+        assert torch.allclose(nx, ny, rtol=2e-3)
+        # doubling the input doubles the output, except where an fp16 subnormal or a rounding boundary
+        # is crossed (then by one fp16 ulp)
+        y2 = had(x * 2)
+        assert float((y2 == y * 2).float().mean()) > 0.999
+        assert torch.allclose(y2.float(), 2 * y.float(), rtol=1e-3, atol=1e-4)
+        sub = o.online_hadamard(x[::257].cpu().numpy())
+        assert close(y[::257].cpu().numpy(), sub)
+    x = gpu(synth_x(512, 4096, seed=2, outliers=False))
+    had = quarot_amd.nn.OnlineHadamard(4096).cuda()
+    assert torch.allclose(had(had(x)).float(), x.float(), atol=4e-3, rtol=4e-3)
+
+
+def test_hadamard_in_place_and_leading_dims():
+    n = 1024
+    x = gpu(synth_x(12, n, seed=9)).view(3, 4, n)
+    y = quarot_amd.functional.hadamard.hadamard_transform(x, scale=1 / 32)
+    assert y.shape == (3, 4, n)
+    flat = x.clone().view(12, n)
+    rc = _lib.lib().qr_hadamard(flat.data_ptr(), flat.data_ptr(), 12, n, 1, None, 0, 1 / 32,
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(flat.view(3, 4, n), y)
+
+
+# ------------------------------------------------------------------------------ KV cache
+
+@pytest.mark.parametrize("dim", [16, 64, 128, 256])
+@pytest.mark.parametrize("hadamard", [False, True])
+def test_kv_quant_dequant_bit_exact(dim, hadamard):
+    rng = np.random.default_rng(dim)
+    v = 1500
+    x = rng.standard_normal((v, dim))
+    x[rng.random((v, dim)) < 0.005] *= 15
+    x[3], x[4] = 0.5, 0.0                                          # constant vectors: range clamps to fp16(1e-5)
+    x = x.astype(F16).reshape(3, 500, dim)
+    q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=hadamard)
+    assert q.shape == (3, 500, dim // 2) and s.shape == (3, 500, 1) and z.shape == (3, 500, 1)
+    xin = x
+    if hadamard:        # codes are judged on the kernel's own Hadamard output (same arithmetic as matmul_had_cuda)
+        xh = kv.matmul_had_cuda(gpu(x), torch.float16)
+        assert close(xh.cpu().numpy(), o.kv_hadamard(x))
+        xin = xh.cpu().numpy()
+    wq, ws, wz = o.kv_asym_quant(xin)
+    assert np.array_equal(q.cpu().numpy(), wq)
+    assert np.array_equal(bits(s.cpu().numpy()), bits(ws)) and np.array_equal(bits(z.cpu().numpy()), bits(wz))
+    y = kv.unpack_i4_and_asym_dequantize(q, s, z)
+    assert np.array_equal(bits(y.cpu().numpy()), bits(o.kv_asym_dequant(wq, ws, wz)))
+    err = (y.float() - gpu(xin).float()).abs()
+    # half a step plus the fp16 roundings of x + zero, q * scale and the final subtraction
+    assert bool((err <= s.float() / 2 + 0.004 * (15 * s.float() + z.float().abs()) + 1e-3).all())
+
+
+def test_kv_full_size_round_trip():
+    """The benchmark tensor [32, 4096, 8, 128]: codes in range, extremes hit, error bound, and a
+    strided sample against the oracle."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(32, 4096, 8, 128, generator=g)
+    mask = torch.rand(x.shape, generator=torch.Generator().manual_seed(5)) < 0.005
+    x[mask] *= 15
+    x = x.half()
+    xd = x.to(dev())
+    q, s, z = kv.asym_quantize_and_pack_i4(xd)
+    y = kv.unpack_i4_and_asym_dequantize(q, s, z)
+    assert bool(((y.float() - xd.float()).abs() <= s.float() / 2 + 0.004 * (15 * s.float() + z.float().abs()) + 1e-3).all())
+    lo, hi = q & 0xF, q >> 4
+    assert int(torch.minimum(lo.amin(-1), hi.amin(-1)).max()) == 0 and int(torch.maximum(lo.amax(-1), hi.amax(-1)).min()) == 15
+    sub = x[::7, ::211].numpy()
+    wq, ws, wz = o.kv_asym_quant(sub)
+    assert np.array_equal(q[::7, ::211].cpu().numpy(), wq) and np.array_equal(bits(s[::7, ::211].cpu().numpy()), bits(ws))
+
+
+# ------------------------------------------------------------------------------ benchmark-size configs
+
+def check_rows_against_oracle(y, a, sa, w, sw, rows):
+    want = o.linear4bit(a[rows], sa[rows], w, sw)
+    assert np.array_equal(bits(y[rows].cpu().numpy()), bits(want))
+
+
+def test_config_down_proj_2048x11008x4096_end_to_end():
+    """Config 2 at full size: fused Hadamard+quantise then fused GEMM+dequant.  Codes are checked
+    against the oracle quantiser on the kernel's Hadamard output for every row; the linear output
+    is checked bit-exactly on a strided sample of rows (all 4096 columns)."""
+    m, k, n = 2048, 11008, 4096
+    x = gpu(synth_x(m, k, seed=0))
+    w, sw = synth_w(n, k, seed=1)
+    fused = quarot_amd.nn.OnlineHadamardQuantizer(k).cuda()
+    p, y_h = quarot_amd.hadamard_quantize(x, fused.had_rem_dim, fused.rem_dim, return_transformed=True)
+    wq, ws = o.quantizer(y_h.cpu().numpy())
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq) and np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+    rows = np.arange(0, m, 37)
+    assert close(y_h[rows].cpu().numpy(), o.online_hadamard(x[rows].cpu().numpy()))
+    lin = quarot_amd.nn.Linear4bit(k, n).half().cuda()
+    lin.weight.copy_(gpu(w))
+    lin.weight_scales.copy_(gpu(sw))
+    y = lin(p)
+    check_rows_against_oracle(y, wq, ws, w, sw.reshape(-1), rows)
+
+
+@pytest.mark.parametrize("m,k,n", [(32768, 4096, 4096), (8192, 4096, 12288), (4096, 11008, 4096)])
+def test_prefill_shapes_sampled_rows(m, k, n):
+    rng = np.random.default_rng(m + n)
+    a = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    w = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    sa = (np.abs(rng.standard_normal(m)) * 0.2).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01).astype(F16)
+    y = quarot_amd.linear_i4(gpu(a), gpu(sa), gpu(w), gpu(sw))
+    rows = np.concatenate([np.arange(0, m, 509), [m - 1]])
+    check_rows_against_oracle(y, a, sa, w, sw, rows)
+    c = quarot_amd.matmul(gpu(a), gpu(w))
+    assert np.array_equal(c[rows].cpu().numpy(), o.int4_matmul(a[rows], w))
+
+
+@pytest.mark.parametrize("m", [1, 8, 32, 64])
+@pytest.mark.parametrize("k,n", [(8192, 57344), (28672, 8192)])
+def test_decode_shapes_bit_exact(m, k, n):
+    rng = np.random.default_rng(m + n)
+    a = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    w = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    sa = (np.abs(rng.standard_normal(m)) * 0.2).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01).astype(F16)
+    y = quarot_amd.linear_i4(gpu(a), gpu(sa), gpu(w), gpu(sw))
+    cols = np.arange(0, n, 3)
+    want = o.linear4bit(a, sa, w[cols], sw[cols])
+    assert np.array_equal(bits(y[:, cols].cpu().numpy()), bits(want))
+
+
+def test_runs_on_the_current_stream():
+    s = torch.cuda.Stream()
+    x = gpu(synth_x(64, 4096, seed=8))
+    with torch.cuda.stream(s):
+        q, sc = quarot_amd.quantize_rows(x)
+    s.synchronize()
+    wq, ws = o.quantizer(x.cpu().numpy())
+    assert np.array_equal(q.cpu().numpy(), wq)

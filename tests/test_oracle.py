@@ -337,3 +337,22 @@ def test_kv_asym_exact_rational_spot():
             assert nib[r, c] == max(0, min(15, q))
             back = round_fraction_to_f16(Fraction(float(round_fraction_to_f16(int(nib[r, c]) * Fraction(float(sc))))) + mn)
             assert back == o.kv_asym_dequant(p, s, z)[r, c]
+
+
+def test_cpu_baseline_port_agrees_with_oracle():
+    """The torch chain timed as the CPU baseline computes what the oracle computes (Hadamard to
+    tolerance; given the same Hadamard output, identical codes and identical fp16 outputs)."""
+    import torch
+    from oracle import cpu_baseline as cb
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((8, 688)).astype(F16)
+    wq = rng.integers(-8, 8, (24, 688))
+    ws = (np.abs(rng.standard_normal(24)) * 0.01).astype(F16)
+    xh = cb.matmul_hadU(torch.from_numpy(x).float())
+    np.testing.assert_allclose(xh.numpy(), o.hadamard_closed_form(x.astype(np.float64)), rtol=1e-4, atol=1e-4)
+    xh16 = xh.half()
+    q, sx = cb.quantize(xh16)
+    assert np.array_equal(q.numpy(), o.sym_quant_codes(xh16.numpy(), o.quantizer_scales(xh16.numpy())))
+    y = cb.linear4bit_path(torch.from_numpy(x), torch.from_numpy(wq.astype(np.int32)), torch.from_numpy(ws))
+    want = o.linear4bit(o.pack_i4(q.numpy()), sx.numpy().reshape(-1), o.pack_i4(wq), ws)
+    assert np.array_equal(y.numpy().view(np.uint16), want.view(np.uint16))
