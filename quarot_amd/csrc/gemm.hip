@@ -13,6 +13,14 @@
 // The MFMA's first operand is the W (B-matrix) fragment and its second the X (A-matrix) fragment,
 // so in the 32x32 accumulator a lane owns one token (m = lane % 32) and runs of 4 consecutive
 // output features n: stores are 8 bytes (fp16) or 16 bytes (int32) per lane.
+//
+// Issue budget: a 32x32x32 int8 MFMA occupies the matrix pipe for 32 cycles and a wave's VALU op
+// takes 4; measured on MI355X, up to ~5 VALU ops per MFMA are hidden.  Unpacking costs 3 VALU ops per
+// packed dword, i.e. 6 (IM + JN) / (IM JN) per MFMA for a wave tile of IM x JN MFMA tiles: 64x128 per
+// wave (4.5) is the smallest tile that fits.  To still run two waves per SIMD on a 128x256 workgroup
+// tile (one tile per CU at M = 2048, N = 4096), eight waves are arranged as 2 (M) x 2 (N) x 2 (K): the
+// two K-groups take alternate 64-k sub-steps of every stage and exchange half of their accumulators
+// through LDS at the end.
 #include "qr_common.h"
 
 namespace {
@@ -22,18 +30,24 @@ namespace {
 // reads in one ds_read_b128 beat fall in 16 different 16-byte bank groups.
 __device__ __forceinline__ int lds_slot(int row, int chunk) { return row * 4 + (chunk ^ ((row >> 2) & 3)); }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
+template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT, bool DEQ>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
     int tiles_m, int tiles_n) {
-    constexpr int NT = 64 * WAVES_M * WAVES_N;              // threads per workgroup
+    constexpr int NT = 64 * WAVES_M * WAVES_N * KSPLIT;     // threads per workgroup
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;     // per-wave output tile
     constexpr int IM = TM / 32, JN = TN / 32;               // 32x32 MFMA tiles per wave
     constexpr int CH = (BM + BN) * 4;                       // 16-byte chunks per stage
     constexpr int NL = (CH + NT - 1) / NT;                  // chunks each thread moves per stage
     static_assert(TM % 32 == 0 && TN % 32 == 0, "tile shape");
-    __shared__ u32x4 lds[2][CH];
+    static_assert(KSPLIT == 1 || (KSPLIT == 2 && JN % 2 == 0), "K split");
+    // stage buffers; with KSPLIT == 2 the same memory later carries the accumulator exchange
+    // (per round: every wave sends JN/2 tiles of 4 KB)
+    constexpr int XCH = KSPLIT == 2 ? WAVES_M * WAVES_N * 2 * (JN / 2) * 256 : 0;
+    constexpr int LDS_ELEMS = 2 * CH > XCH ? 2 * CH : XCH;
+    __shared__ u32x4 lds_raw[LDS_ELEMS];
+    u32x4(*lds)[CH] = (u32x4(*)[CH])lds_raw;
 
     // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Give every XCD a
     // contiguous range of tile ids, and walk tiles in groups of GROUP_M rows so that the tiles in
@@ -52,7 +66,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int kg = wave / (WAVES_M * WAVES_N);              // K-group of this wave
+    const int wxy = wave % (WAVES_M * WAVES_N);
+    const int wm = wxy / WAVES_N, wn = wxy % WAVES_N;
 
     // Global -> LDS staging: chunk id = tid + i * NT; 4 consecutive threads fetch one row's 64 bytes.
     // Rows beyond M (or N) are clamped to the last valid row: they are read but never stored.
@@ -91,7 +107,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     auto compute = [&](const u32x4* buf, int nsub) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            if (s < nsub) {
+            if (s < nsub && (KSPLIT == 1 || s == kg)) {
                 i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
 #pragma unroll
                 for (int i = 0; i < IM; ++i) {
@@ -120,30 +136,44 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     // possibly one half stage (chunks 0 and 1 only).
     const int full = Kb / 64;
     const bool half_tail = (Kb & 63) != 0;
-    u32x4 pre[NL];
+    // Global loads run TWO stages ahead of the MFMAs (HBM/L2 latency exceeds one stage of compute):
+    // stage ks+2 is requested into one register set at the top of iteration ks, while the other
+    // set (stage ks+1, requested an iteration earlier) is written to LDS at the bottom.
+    u32x4 preA[NL], preB[NL];
     if (full > 0) {
 #pragma unroll
-        for (int i = 0; i < NL; ++i) pre[i] = *(const u32x4*)(src[i]);
+        for (int i = 0; i < NL; ++i) preA[i] = *(const u32x4*)(src[i]);
 #pragma unroll
-        for (int i = 0; i < NL; ++i) lds[0][dst[i]] = pre[i];
+        for (int i = 0; i < NL; ++i) lds[0][dst[i]] = preA[i];
+    }
+    if (full > 1) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) preA[i] = *(const u32x4*)(src[i] + 64);      // stage 1
     }
     __syncthreads();
-    for (int ks = 0; ks < full; ++ks) {
-        const bool more = ks + 1 < full;
-        if (more) {
+    auto iteration = [&](int ks, u32x4(&cur)[NL], u32x4(&nxt)[NL]) {
+        // `cur` holds stage ks+1 (in flight or landed); `nxt` receives stage ks+2
+        if (ks + 2 < full) {
 #pragma unroll
-            for (int i = 0; i < NL; ++i) {
-                src[i] += 64;
-                pre[i] = *(const u32x4*)(src[i]);
-            }
+            for (int i = 0; i < NL; ++i) nxt[i] = *(const u32x4*)(src[i] + (int64_t)(ks + 2) * 64);
         }
         compute(lds[ks & 1], 2);
-        if (more) {
+        if (ks + 1 < full) {
 #pragma unroll
-            for (int i = 0; i < NL; ++i) lds[(ks + 1) & 1][dst[i]] = pre[i];
+            for (int i = 0; i < NL; ++i) lds[(ks + 1) & 1][dst[i]] = cur[i];
         }
         __syncthreads();
+    };
+    {
+        int ks = 0;
+        for (; ks + 1 < full; ks += 2) {
+            iteration(ks, preA, preB);
+            iteration(ks + 1, preB, preA);
+        }
+        if (ks < full) iteration(ks, preA, preB);
     }
+#pragma unroll
+    for (int i = 0; i < NL; ++i) src[i] += (int64_t)(full > 0 ? full - 1 : 0) * 64;   // last full stage
     if (half_tail) {
         // chunks 2 and 3 of this last stage lie beyond the row: only chunks 0/1 are fetched and used
 #pragma unroll
@@ -156,6 +186,54 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
         compute(lds[0], 1);
     }
 
+    // K-split: the two K-groups hold partial sums of the same wave tile.  Group 0 finalises the
+    // lower half of the j tiles and group 1 the upper half; each sends the other half across, one
+    // row of MFMA tiles (i) per round.  A tile travels as four 16-byte pieces per lane, lane-contiguous.
+    constexpr int JH = KSPLIT == 2 ? JN / 2 : JN;
+    const int j_first = KSPLIT == 2 ? kg * JH : 0;
+    if constexpr (KSPLIT == 2) {
+        u32x4* xbuf = lds_raw;
+        const int send0 = (1 - kg) * JH;            // first j tile this wave gives away
+        for (int i = 0; i < IM; ++i) {
+            __syncthreads();                        // stage buffers / previous round no longer read
+#pragma unroll
+            for (int jj = 0; jj < JH; ++jj)
+#pragma unroll
+                for (int qv = 0; qv < 4; ++qv) {
+                    // slot owned by the RECEIVER (wxy, 1 - kg)
+                    const int slot = (((wxy * 2 + (1 - kg)) * JH + jj) * 4 + qv) * 64 + lane;
+                    i32x4 piece;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        int val = 0;
+#pragma unroll
+                        for (int ii = 0; ii < IM; ++ii)
+#pragma unroll
+                            for (int jx = 0; jx < JN; ++jx)
+                                if (ii == i && jx == send0 + jj) val = acc[ii][jx][qv * 4 + e];
+                        piece[e] = val;
+                    }
+                    xbuf[slot] = (u32x4)piece;
+                }
+            __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < JH; ++jj)
+#pragma unroll
+                for (int qv = 0; qv < 4; ++qv) {
+                    const int slot = (((wxy * 2 + kg) * JH + jj) * 4 + qv) * 64 + lane;
+                    const i32x4 piece = (i32x4)xbuf[slot];
+#pragma unroll
+                    for (int ii = 0; ii < IM; ++ii)
+#pragma unroll
+                        for (int jx = 0; jx < JN; ++jx)
+                            if (ii == i && jx == j_first + jj) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[ii][jx][qv * 4 + e] += piece[e];
+                            }
+                }
+        }
+    }
+
     // Epilogue.  Accumulator layout (first operand = W rows, second = X rows): lane l, register v ->
     // n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
 #pragma unroll
@@ -166,6 +244,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
         if (DEQ) sa = sA[row];
 #pragma unroll
         for (int j = 0; j < JN; ++j) {
+            if (j < j_first || j >= j_first + JH) continue;     // the other K-group stores this tile
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
                 const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
@@ -206,20 +285,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT>
 int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st) {
-    constexpr int NT = 64 * WAVES_M * WAVES_N;
+    constexpr int NT = 64 * WAVES_M * WAVES_N * KSPLIT;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     if (Y)
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(NT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, KSPLIT, true><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, (const f16*)sA, (const f16*)sB,
             (const f16*)bias, tiles_m, tiles_n);
     else
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(NT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, KSPLIT, false><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr, nullptr, nullptr, nullptr, tiles_m,
             tiles_n);
     return qr_launch_status();
@@ -235,12 +314,12 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M <= 32) return launch_cfg<32, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    if (M <= 64) return launch_cfg<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 32) return launch_cfg<32, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 64) return launch_cfg<64, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t256 >= 512) return launch_cfg<256, 256, 4, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 256) return launch_cfg<128, 256, 2, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t128x256 >= 128) return launch_cfg<128, 256, 2, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    return launch_cfg<128, 128, 2, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
 
 }  // namespace

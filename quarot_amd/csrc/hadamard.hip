@@ -141,26 +141,35 @@ __global__ __launch_bounds__(HT) void hadamard_kernel(const IO* __restrict__ x, 
     for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
         const IO* xr = x + row * (int64_t)n;
         __syncthreads();        // previous row's phase 4 (and the hadK staging) done before buf is overwritten
-        // ---- phase 1
-        for (int c0 = 0; c0 < nchunks; c0 += HT) {
-            const int c = c0 + tid;             // whole waves share the predicate: nchunks % 64 may be != 0 only
-            float v[8];                         // when m < 512, and then exchanges stay inside a segment's lanes
-            const bool live = c < nchunks;
-            if (live) load8(xr + (int64_t)c * 8, v);
-            else {
+        // ---- phase 1 (loads issued four chunks ahead of their use)
+        for (int c0 = 0; c0 < nchunks; c0 += 4 * HT) {
+            float v[4][8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = 0.f;
+            for (int u = 0; u < 4; ++u) {
+                const int c = c0 + u * HT + tid;
+                if (c < nchunks) load8(xr + (int64_t)c * 8, v[u]);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[u][e] = 0.f;
+                }
             }
-            reg_fwht8(v);
-            if (lane_stages > 0) lane_stage<1>(v, lane);
-            if (lane_stages > 1) lane_stage<2>(v, lane);
-            if (lane_stages > 2) lane_stage<4>(v, lane);
-            if (lane_stages > 3) lane_stage<8>(v, lane);
-            if (lane_stages > 4) lane_stage<16>(v, lane);
-            if (lane_stages > 5) lane_stage<32>(v, lane);
-            if (live) {
-                *(f32x4*)(buf + c * 8) = f32x4{v[0], v[1], v[2], v[3]};
-                *(f32x4*)(buf + c * 8 + 4) = f32x4{v[4], v[5], v[6], v[7]};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                // whole waves share `live`: nchunks % 64 != 0 only when m < 512, and then the
+                // exchanges stay inside a segment's lanes, which are all live or all dead
+                const int c = c0 + u * HT + tid;
+                if (c0 + u * HT >= nchunks) break;
+                reg_fwht8(v[u]);
+                if (lane_stages > 0) lane_stage<1>(v[u], lane);
+                if (lane_stages > 1) lane_stage<2>(v[u], lane);
+                if (lane_stages > 2) lane_stage<4>(v[u], lane);
+                if (lane_stages > 3) lane_stage<8>(v[u], lane);
+                if (lane_stages > 4) lane_stage<16>(v[u], lane);
+                if (lane_stages > 5) lane_stage<32>(v[u], lane);
+                if (c < nchunks) {
+                    *(f32x4*)(buf + c * 8) = f32x4{v[u][0], v[u][1], v[u][2], v[u][3]};
+                    *(f32x4*)(buf + c * 8 + 4) = f32x4{v[u][4], v[u][5], v[u][6], v[u][7]};
+                }
             }
         }
         __syncthreads();
@@ -261,6 +270,211 @@ __global__ __launch_bounds__(HT) void hadamard_kernel(const IO* __restrict__ x, 
     }
 }
 
+// ---- K > 1 with a short power-of-two factor (16 <= m <= 256), fp16 I/O -------------------------
+// The butterflies need no LDS (a segment spans at most 32 lanes); hadK lives in REGISTERS as MFMA
+// A-fragments (each wave owns every fourth 16-row tile), which leaves LDS for two small fp16
+// arrays -- the transposed, scaled, fp16-rounded T (so a B-fragment is one 16-byte read) and the
+// result -- and lets several workgroups share a CU.  The next row's global loads are issued before
+// the matrix stage of the current one.
+constexpr int RT_W = 3;          // 16-row tiles per wave: hadK order <= 192
+
+template <bool MODE32, bool QUANT, int NCH>
+__global__ __launch_bounds__(HT) void hadamard_km_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
+                                                         int n, int K, int log2m, const void* __restrict__ hadK,
+                                                         float scale, float clip, u32* __restrict__ q,
+                                                         f16* __restrict__ scales) {
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[HT / QR_WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m = 1 << log2m;
+    const int nchunks = n >> 3;
+    const int Kc = (K + 31) & ~31;
+    const int TS = Kc + 8;                       // halves per row of Tt (row = one column r of T)
+    const int YS = m + 8;                        // halves per row of Yl (row = one output k')
+    const int ksteps = Kc >> 5;
+    const int row_tiles = (K + 15) >> 4;
+    f16* Tt = (f16*)smem_raw;                    // [m][TS]; 8-half blocks XOR-swizzled by (r >> 3) & 3
+    f16* Tlo = Tt + m * TS;                      // second plane, fp32 mode only
+    f16* Yl = Tt + (MODE32 ? 2 : 1) * m * TS;    // [K][YS]
+    const int kq = lane >> 4;
+
+    // hadK -> A-fragments in registers (zero padded)
+    f16x8 hf[RT_W][KS_MAX];
+#pragma unroll
+    for (int t = 0; t < RT_W; ++t) {
+        const int hr = (wave + 4 * t) * 16 + (lane & 15);
+#pragma unroll
+        for (int ks = 0; ks < KS_MAX; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int hc = ks * 32 + kq * 8 + j;
+                f16 h = (f16)0;
+                if (hr < K && hc < K)
+                    h = MODE32 ? (f16)((const float*)hadK)[hr * K + hc] : ((const f16*)hadK)[hr * K + hc];
+                hf[t][ks][j] = h;
+            }
+    }
+    // the padding of Tt (k >= K) is never written afterwards: clear everything once
+    for (int i = tid; i < ((MODE32 ? 2 : 1) * m * TS) / 8; i += HT) ((u32x4*)Tt)[i] = u32x4{0, 0, 0, 0};
+
+    const int lane_stages = log2m - 3;
+    u32x4 raw[NCH];
+    int64_t row = blockIdx.x;
+    if (row < rows) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * HT;
+            raw[i] = c < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + row * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
+        }
+    }
+    __syncthreads();
+    for (; row < rows; row += gridDim.x) {
+        // ---- phase 1: butterflies in registers and across lanes, scatter to Tt
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * HT;
+            if (i * HT >= nchunks) break;
+            float v[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                v[2 * w] = (float)f16_from_bits((unsigned short)(raw[i][w] & 0xffffu));
+                v[2 * w + 1] = (float)f16_from_bits((unsigned short)(raw[i][w] >> 16));
+            }
+            reg_fwht8(v);
+            if (lane_stages > 0) lane_stage<1>(v, lane);
+            if (lane_stages > 1) lane_stage<2>(v, lane);
+            if (lane_stages > 2) lane_stage<4>(v, lane);
+            if (lane_stages > 3) lane_stage<8>(v, lane);
+            if (lane_stages > 4) lane_stage<16>(v, lane);
+            if (c < nchunks) {
+                const int k = (c * 8) >> log2m;
+                const int r0 = (c * 8) & (m - 1);
+                const int pb = (k >> 3) ^ ((r0 >> 3) & 3);
+                f16* dst = Tt + r0 * TS + pb * 8 + (k & 7);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float t = v[e] * scale;
+                    const f16 hi = narrow_f16(t);
+                    dst[e * TS] = hi;
+                    if (MODE32) dst[e * TS + m * TS] = (f16)(t - (float)hi);
+                }
+            }
+        }
+        // next row's loads fly during the matrix stage
+        const int64_t nrow = row + gridDim.x;
+        if (nrow < rows) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int c = tid + i * HT;
+                raw[i] = c < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + nrow * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
+            }
+        }
+        __syncthreads();
+        // ---- phase 3: Y[K, m] = hadK . T on the matrix cores
+        for (int ct = 0; ct < (m >> 4); ++ct) {
+            const int r = ct * 16 + (lane & 15);
+            const int sw = (r >> 3) & 3;
+            f16x8 bh[KS_MAX], bl[KS_MAX];
+#pragma unroll
+            for (int ks = 0; ks < KS_MAX; ++ks)
+                if (ks < ksteps) {
+                    const int off = r * TS + (((ks << 2) + kq) ^ sw) * 8;
+                    bh[ks] = *(const f16x8*)(Tt + off);
+                    if (MODE32) bl[ks] = *(const f16x8*)(Tlo + off);
+                }
+#pragma unroll
+            for (int t = 0; t < RT_W; ++t) {
+                const int rt = wave + 4 * t;
+                if (rt < row_tiles) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS_MAX; ++ks)
+                        if (ks < ksteps) {
+                            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(hf[t][ks], bh[ks], acc, 0, 0, 0);
+                            if (MODE32) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(hf[t][ks], bl[ks], acc, 0, 0, 0);
+                        }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int kp = rt * 16 + kq * 4 + v;
+                        if (kp < K) Yl[kp * YS + r] = (f16)acc[v];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // ---- phase 4: Yl -> global (and the quantiser)
+        if (QUANT) {
+            u32 mx = 0;
+            for (int c = tid; c < nchunks; c += HT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> log2m) * YS + ((c * 8) & (m - 1)));
+                const u32 mc = absmax_bits8(h);
+                mx = mx > mc ? mx : mc;
+            }
+            mx = wave_max_u32(mx);
+            if (lane == 0) red[wave] = mx;
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+            const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+            if (tid == 0) scales[row] = sh;
+            const float s = (float)sh;
+            const bool fast = scale_fast_ok(s);
+            const float rs = fast ? 1.0f / s : 0.0f;
+            for (int c = tid; c < nchunks; c += HT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> log2m) * YS + ((c * 8) & (m - 1)));
+                q[row * (int64_t)nchunks + c] = sym_codes8(h, s, rs, fast);
+                if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            }
+        } else {
+            for (int c = tid; c < nchunks; c += HT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> log2m) * YS + ((c * 8) & (m - 1)));
+                __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            }
+        }
+        // red[] and Yl are next written after the barrier that follows the next phase 1
+    }
+}
+
+template <bool MODE32, bool QUANT>
+int launch_hadamard_km(const void* x, void* y, int64_t rows, int n, int K, int log2m, const void* hadK, float scale,
+                       float clip, void* q, void* scales, hipStream_t st) {
+    const int m = 1 << log2m;
+    const int Kc = (K + 31) & ~31;
+    const size_t lds = (size_t)(MODE32 ? 2 : 1) * m * (Kc + 8) * 2 + (size_t)K * (m + 8) * 2;
+    const int nch = ((n >> 3) + HT - 1) / HT;
+    int per_cu = (int)((160 * 1024) / (lds + 1024));
+    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
+    const int64_t cap = 256LL * per_cu;
+    const unsigned grid = (unsigned)(rows < cap ? rows : cap);
+#define QR_KM(NCH)                                                                                                    \
+    do {                                                                                                              \
+        auto kern = hadamard_km_kernel<MODE32, QUANT, NCH>;                                                           \
+        if (lds > 48 * 1024) {                                                                                        \
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) return (int)e;                                                                       \
+        }                                                                                                             \
+        kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, log2m, hadK, scale, clip, (u32*)q, \
+                                                (f16*)scales);                                                        \
+    } while (0)
+    if (nch <= 2) QR_KM(2);
+    else if (nch <= 4) QR_KM(4);
+    else if (nch <= 6) QR_KM(6);
+    else if (nch <= 8) QR_KM(8);
+    else QR_KM(16);
+#undef QR_KM
+    return qr_launch_status();
+}
+
+// true when the register-resident-hadK kernel applies
+bool km_applies(int n, int K, bool mode32) {
+    if (K <= 1) return false;
+    const int m = n / K;
+    if (m < 16 || m > 256) return false;
+    const int Kc = (K + 31) & ~31;
+    const size_t lds = (size_t)(mode32 ? 2 : 1) * m * (Kc + 8) * 2 + (size_t)K * (m + 8) * 2;
+    return lds <= 150 * 1024 && (n >> 3) <= 16 * HT;
+}
+
 template <typename IO, bool MODE32, bool QUANT>
 int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
                     void* q, void* scales, hipStream_t st) {
@@ -306,6 +520,11 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == QR_DTYPE_F16 && km_applies(n, K, false)) {
+        int log2m = 0;
+        while ((1 << log2m) < n / K) ++log2m;
+        return launch_hadamard_km<false, false>(x, y, rows, n, K, log2m, hadK, scale, 1.f, nullptr, nullptr, st);
+    }
     if (dtype == QR_DTYPE_F16) return launch_hadamard<f16, false, false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F32) return launch_hadamard<float, true, false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     return QR_E_DTYPE;
@@ -320,6 +539,13 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (!x || !q || !scales || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (km_applies(n, K, mode == QR_DTYPE_F32)) {
+        int log2m = 0;
+        while ((1 << log2m) < n / K) ++log2m;
+        if (mode == QR_DTYPE_F16) return launch_hadamard_km<false, true>(x, y_or_null, rows, n, K, log2m, hadK, scale, clip, q, scales, st);
+        return launch_hadamard_km<true, true>(x, y_or_null, rows, n, K, log2m, hadK, scale, clip, q, scales, st);
+    }
     if (mode == QR_DTYPE_F16) return launch_hadamard<f16, false, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     if (mode == QR_DTYPE_F32) return launch_hadamard<f16, true, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     return QR_E_DTYPE;
