@@ -243,6 +243,8 @@ __global__ __launch_bounds__(HT) void hadamard_kernel(const IO* __restrict__ x, 
             const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
             if (tid == 0) scales[row] = sh;
             const float s = (float)sh;
+            const bool lean = fast_quant_ok(mx, s);
+            const FastRecip fr = make_fast_recip(lean ? s : 1.0f);
             const bool fast = scale_fast_ok(s);
             const float rs = fast ? 1.0f / s : 0.0f;
             for (int c = tid; c < nchunks; c += HT) {
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(HT) void hadamard_kernel(const IO* __restrict__ x, 
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = buf[c * 8 + e] * osc;
                 u32x4 h = to_f16x8(v);
-                q[row * (int64_t)nchunks + c] = sym_codes8(h, s, rs, fast);
+                q[row * (int64_t)nchunks + c] = lean ? sym_codes8_fast(h, fr) : sym_codes8(h, s, rs, fast);
                 if (y) __builtin_nontemporal_store(h, (u32x4*)((f16*)y + row * (int64_t)n) + c);
             }
         } else {
@@ -418,11 +420,13 @@ __global__ __launch_bounds__(HT) void hadamard_km_kernel(const f16* __restrict__
             const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
             if (tid == 0) scales[row] = sh;
             const float s = (float)sh;
+            const bool lean = fast_quant_ok(mx, s);
+            const FastRecip fr = make_fast_recip(lean ? s : 1.0f);
             const bool fast = scale_fast_ok(s);
             const float rs = fast ? 1.0f / s : 0.0f;
             for (int c = tid; c < nchunks; c += HT) {
                 const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> log2m) * YS + ((c * 8) & (m - 1)));
-                q[row * (int64_t)nchunks + c] = sym_codes8(h, s, rs, fast);
+                q[row * (int64_t)nchunks + c] = lean ? sym_codes8_fast(h, fr) : sym_codes8(h, s, rs, fast);
                 if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
             }
         } else {
@@ -475,6 +479,268 @@ bool km_applies(int n, int K, bool mode32) {
     return lds <= 150 * 1024 && (n >> 3) <= 16 * HT;
 }
 
+// ---- K > 1, m = 64 or 128, fp16 I/O: both factors on the matrix cores ---------------------------
+// Per row (token), with X viewed as [K, m]:
+//   stage 1   T = X . H_m            A-fragments straight from global memory (a lane's 8 consecutive
+//                                    r of one k are 16 contiguous bytes), H_m fragments generated in
+//                                    registers from popcount parity.  The accumulator of two 16-row
+//                                    tiles, scaled and rounded to fp16, IS one 32-deep fragment of T
+//                                    for stage 2 when the contraction index is taken in the order
+//                                    k = 32 s + 16 (j / 4) + 4 (lane / 16) + j % 4 -- no transposition;
+//                                    it goes to LDS as one 16-byte write per lane.
+//   stage 2   Y^T = T^T . hadK^T     hadK fragments (same k order) live in registers, each wave owns
+//                                    every fourth 16-row tile of hadK and reads all of T from LDS;
+//                                    a lane ends with 4 consecutive r of one output k: 8-byte writes
+//                                    into the fp16 result row in LDS.
+//   stage 3   result row -> global, with the quantiser when fused.
+template <bool MODE32, bool QUANT, int LOG2M, int KS2>
+__global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
+                                                         int n, int K, const void* __restrict__ hadK, float scale,
+                                                         float clip, u32* __restrict__ q, f16* __restrict__ scales) {
+    constexpr int M_ = 1 << LOG2M;
+    constexpr int KS1 = M_ / 32;                 // contraction steps of stage 1
+    constexpr int CT = M_ / 16;                  // 16-column tiles of T / Y
+    constexpr int NCT = CT / 4;                  // column tiles per wave in stage 1
+    constexpr int YS = M_ + 8;                   // halves per row of Yl
+    // Rows of m = 64: a whole row of stage-1 fragments (KS2 tile pairs) is kept in registers and
+    // each pair is re-requested for the NEXT row as soon as it has been consumed, so global loads
+    // run one full row ahead.  m = 128 would need twice the registers: one pair ahead only.
+    constexpr bool FULL_ROW = (M_ == 64);
+    constexpr int SLOTS = FULL_ROW ? KS2 : 2;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[HT / QR_WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int nchunks = n >> 3;
+    const int row_tiles = (K + 15) >> 4;
+    u32x4* Tl = (u32x4*)smem_raw;                              // [CT][KS2][64 lanes] fragments of T (hi plane)
+    u32x4* Tlo = Tl + CT * KS2 * 64;                           // lo plane (fp32 mode)
+    f16* Yl = (f16*)(Tl + (MODE32 ? 2 : 1) * CT * KS2 * 64);   // [K][YS]
+
+    // hadK fragments, contraction index in the stage-1 accumulator order: for each (step, half) a
+    // lane needs 4 consecutive k -- one 8-byte (fp16) or 16-byte (fp32) load (every order is a
+    // multiple of 4, so a group of 4 is inside or outside the matrix as a whole)
+    f16x8 hf[RT_W][KS2];
+#pragma unroll
+    for (int t = 0; t < RT_W; ++t) {
+        const int hr = (wave + 4 * t) * 16 + l16;
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int hc = ks * 32 + hh * 16 + g * 4;
+                f16x4 v = {(f16)0, (f16)0, (f16)0, (f16)0};
+                if (hr < K && hc < K) {
+                    if (MODE32) {
+                        const f32x4 w = *(const f32x4*)((const float*)hadK + hr * K + hc);
+                        v = f16x4{(f16)w[0], (f16)w[1], (f16)w[2], (f16)w[3]};
+                    } else {
+                        v = *(const f16x4*)((const f16*)hadK + hr * K + hc);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hf[t][ks][hh * 4 + e] = v[e];
+            }
+    }
+    // Sylvester fragments: H_m[r][r'] = (-1)^popcount(r & r')
+    f16x8 b1[NCT][KS1];
+#pragma unroll
+    for (int c = 0; c < NCT; ++c)
+#pragma unroll
+        for (int ks = 0; ks < KS1; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int rp = (wave + 4 * c) * 16 + l16;
+                const int r = ks * 32 + g * 8 + j;
+                b1[c][ks][j] = (__builtin_popcount(r & rp) & 1) ? (f16)-1.0f : (f16)1.0f;
+            }
+
+    // stage-1 A-fragments for the tile pair s2 of a row: [2 tiles][KS1] 16-byte loads
+    auto load_pair = [&](const f16* xr, int s2, u32x4(&dst)[2][KS1]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = (2 * s2 + h) * 16 + l16;
+#pragma unroll
+            for (int ks = 0; ks < KS1; ++ks)
+                dst[h][ks] = k < K ? __builtin_nontemporal_load((const u32x4*)(xr + k * M_ + ks * 32 + g * 8)) : u32x4{0, 0, 0, 0};
+        }
+    };
+    // one tile pair through stage 1: T fragments for this wave's column tile(s) -> LDS
+    auto stage1 = [&](int s2, const u32x4(&cur)[2][KS1]) {
+#pragma unroll
+        for (int c = 0; c < NCT; ++c) {
+            f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS1; ++ks) {
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, cur[0][ks]), b1[c][ks], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, cur[1][ks]), b1[c][ks], a1, 0, 0, 0);
+            }
+            float t[8];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                t[e] = a0[e] * scale;
+                t[e + 4] = a1[e] * scale;
+            }
+            u32x4 hi, lo;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const f16 h0 = narrow_f16(t[2 * e]), h1 = narrow_f16(t[2 * e + 1]);
+                hi[e] = (u32)f16_bits(h0) | ((u32)f16_bits(h1) << 16);
+                if (MODE32)
+                    lo[e] = (u32)f16_bits((f16)(t[2 * e] - (float)h0)) | ((u32)f16_bits((f16)(t[2 * e + 1] - (float)h1)) << 16);
+            }
+            const int slot = ((wave + 4 * c) * KS2 + s2) * 64 + lane;
+            Tl[slot] = hi;
+            if (MODE32) Tlo[slot] = lo;
+        }
+    };
+
+    u32x4 fr[SLOTS][2][KS1];
+    int64_t row = blockIdx.x;
+    if (row < rows) {
+        if (FULL_ROW) {
+#pragma unroll
+            for (int s2 = 0; s2 < KS2; ++s2) load_pair(x + row * (int64_t)n, s2, fr[s2 % SLOTS]);
+        } else {
+            load_pair(x + row * (int64_t)n, 0, fr[0]);
+        }
+    }
+    for (; row < rows; row += gridDim.x) {
+        const f16* xr = x + row * (int64_t)n;
+        const int64_t nrow = row + gridDim.x;
+        // ---- stage 1
+#pragma unroll
+        for (int s2 = 0; s2 < KS2; ++s2) {
+            if (FULL_ROW) {
+                stage1(s2, fr[s2 % SLOTS]);
+                if (nrow < rows) load_pair(x + nrow * (int64_t)n, s2, fr[s2 % SLOTS]);
+            } else {
+                // slot parity alternates per pair; with an odd KS2 the next row starts on the other slot,
+                // so the last pair's successor (next row, pair 0) is copied into slot 0 below
+                if (s2 + 1 < KS2) load_pair(xr, s2 + 1, fr[(s2 + 1) % SLOTS]);
+                else if (nrow < rows) load_pair(x + nrow * (int64_t)n, 0, fr[(s2 + 1) % SLOTS]);
+                stage1(s2, fr[s2 % SLOTS]);
+            }
+        }
+        if (!FULL_ROW && (KS2 % 2) == 1) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int ks = 0; ks < KS1; ++ks) fr[0][h][ks] = fr[1][h][ks];
+        }
+        __syncthreads();
+        // ---- stage 2
+        for (int ct = 0; ct < CT; ++ct) {
+            f16x8 th[KS2], tl[KS2];
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                th[ks] = __builtin_bit_cast(f16x8, Tl[(ct * KS2 + ks) * 64 + lane]);
+                if (MODE32) tl[ks] = __builtin_bit_cast(f16x8, Tlo[(ct * KS2 + ks) * 64 + lane]);
+            }
+#pragma unroll
+            for (int t = 0; t < RT_W; ++t) {
+                const int rt = wave + 4 * t;
+                if (rt < row_tiles) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS2; ++ks) {
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(th[ks], hf[t][ks], acc, 0, 0, 0);
+                        if (MODE32) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(tl[ks], hf[t][ks], acc, 0, 0, 0);
+                    }
+                    const int kp = rt * 16 + l16;
+                    if (kp < K) {
+                        u32x2 o;
+                        o[0] = (u32)f16_bits((f16)acc[0]) | ((u32)f16_bits((f16)acc[1]) << 16);
+                        o[1] = (u32)f16_bits((f16)acc[2]) | ((u32)f16_bits((f16)acc[3]) << 16);
+                        *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // ---- stage 3
+        if (QUANT) {
+            u32 mx = 0;
+            for (int c = tid; c < nchunks; c += HT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                const u32 mc = absmax_bits8(h);
+                mx = mx > mc ? mx : mc;
+            }
+            mx = wave_max_u32(mx);
+            if (lane == 0) red[wave] = mx;
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+            const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+            if (tid == 0) scales[row] = sh;
+            const float s = (float)sh;
+            if (fast_quant_ok(mx, s)) {
+                const FastRecip fq = make_fast_recip(s);
+                for (int c = tid; c < nchunks; c += HT) {
+                    const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                    q[row * (int64_t)nchunks + c] = sym_codes8_fast(h, fq);
+                    if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+                }
+            } else {
+                const bool fast = scale_fast_ok(s);
+                const float rs = fast ? 1.0f / s : 0.0f;
+                for (int c = tid; c < nchunks; c += HT) {
+                    const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                    q[row * (int64_t)nchunks + c] = sym_codes8(h, s, rs, fast);
+                    if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+                }
+            }
+        } else {
+            for (int c = tid; c < nchunks; c += HT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            }
+        }
+    }
+}
+
+bool mm_applies(int n, int K) {
+    if (K <= 1 || K > 32 * KS_MAX) return false;
+    const int m = n / K;
+    return m == 64 || m == 128;
+}
+
+template <bool MODE32, bool QUANT>
+int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
+                       void* q, void* scales, hipStream_t st) {
+    const int m = n / K;
+    const int KS2 = ((K + 31) & ~31) >> 5;
+    const size_t lds = (size_t)(MODE32 ? 2 : 1) * (m / 16) * KS2 * 64 * 16 + (size_t)K * (m + 8) * 2;
+    int per_cu = (int)((160 * 1024) / (lds + 1024));
+    per_cu = per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu);
+    const int64_t cap = 256LL * per_cu;
+    const unsigned grid = (unsigned)(rows < cap ? rows : cap);
+#define QR_MM(L2M, KS)                                                                                                 \
+    do {                                                                                                               \
+        auto kern = hadamard_mm_kernel<MODE32, QUANT, L2M, KS>;                                                        \
+        if (lds > 48 * 1024) {                                                                                         \
+            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            if (e != hipSuccess) return (int)e;                                                                        \
+        }                                                                                                              \
+        kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
+                                                (f16*)scales);                                                         \
+    } while (0)
+#define QR_MM_K(L2M)                     \
+    switch (KS2) {                       \
+        case 1: QR_MM(L2M, 1); break;    \
+        case 2: QR_MM(L2M, 2); break;    \
+        case 3: QR_MM(L2M, 3); break;    \
+        case 4: QR_MM(L2M, 4); break;    \
+        case 5: QR_MM(L2M, 5); break;    \
+        default: QR_MM(L2M, 6); break;   \
+    }
+    if (m == 64) { QR_MM_K(6) }
+    else { QR_MM_K(7) }
+#undef QR_MM_K
+#undef QR_MM
+    return qr_launch_status();
+}
+
 template <typename IO, bool MODE32, bool QUANT>
 int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
                     void* q, void* scales, hipStream_t st) {
@@ -520,6 +786,8 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == QR_DTYPE_F16 && mm_applies(n, K))
+        return launch_hadamard_mm<false, false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && km_applies(n, K, false)) {
         int log2m = 0;
         while ((1 << log2m) < n / K) ++log2m;
@@ -540,6 +808,10 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (mm_applies(n, K)) {
+        if (mode == QR_DTYPE_F16) return launch_hadamard_mm<false, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
+        return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
+    }
     if (km_applies(n, K, mode == QR_DTYPE_F32)) {
         int log2m = 0;
         while ((1 << log2m) < n / K) ++log2m;

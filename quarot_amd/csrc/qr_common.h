@@ -108,6 +108,49 @@ __device__ __forceinline__ u32 sym_codes8(u32x4 v, float s, float rs, bool fast_
     return out;
 }
 
+// ---- lean quantiser for rows known to be all-finite with a finite non-zero scale ------------------
+// 1/s is held as rh + rl with rh cut to 13 significant bits, so x * rh is EXACT in fp32 (x has 11)
+// and q = fma(x, rl, x * rh) is the correctly rounded fp32 quotient x / s up to a 2^-36 relative
+// perturbation: far inside the 2^-23 margin that separates a quotient of two fp16 numbers from an
+// fp16 rounding boundary (see sym_code), so (f16)q is the correctly rounded fp16 division.
+// Clamping to [-8, 7] before that conversion commutes with it (rounding is monotone and -8, 7 are
+// representable).  Adding 1536 (ulp 1 in [1024, 2048)) in fp16 then rounds to the nearest integer,
+// ties to even, and leaves the two's-complement code in the low four mantissa bits.
+struct FastRecip {
+    float rh, rl;
+};
+__device__ __forceinline__ FastRecip make_fast_recip(float s) {
+    const double r = 1.0 / (double)s;
+    FastRecip f;
+    f.rh = __builtin_bit_cast(float, __builtin_bit_cast(u32, (float)r) & 0xFFFFF800u);
+    f.rl = (float)(r - (double)f.rh);
+    return f;
+}
+__device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
+    u32 b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float x0 = (float)f16_from_bits((unsigned short)(v[i] & 0xffffu));
+        const float x1 = (float)f16_from_bits((unsigned short)(v[i] >> 16));
+        float q0 = __builtin_fmaf(x0, f.rl, x0 * f.rh);
+        float q1 = __builtin_fmaf(x1, f.rl, x1 * f.rh);
+        q0 = __builtin_amdgcn_fmed3f(q0, -8.0f, 7.0f);
+        q1 = __builtin_amdgcn_fmed3f(q1, -8.0f, 7.0f);
+        f16x2 h = {(f16)q0, (f16)q1};
+        h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
+        const u32 w = __builtin_bit_cast(u32, h);
+        b[i] = (w & 0xFu) | ((w >> 12) & ~0xFu);    // low byte: code0 | code1 << 4 (upper bytes: don't care)
+    }
+    const u32 t01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+    const u32 t23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
+    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+}
+// amax bits below 0x7c00 <=> every element of the row is finite
+__device__ __forceinline__ bool fast_quant_ok(u32 amax_bits, float s) {
+    const float a = __builtin_fabsf(s);
+    return amax_bits < 0x7c00u && a > 0.0f && a < __builtin_inff();
+}
+
 // The reciprocal path is valid when s is a finite non-zero fp16 (then 1/s is a finite float).
 __device__ __forceinline__ bool scale_fast_ok(float s) {
     float a = __builtin_fabsf(s);

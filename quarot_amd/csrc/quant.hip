@@ -22,10 +22,11 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
         v[i] = c < cols8 ? __builtin_nontemporal_load(xr + c) : u32x4{0, 0, 0, 0};
     }
     float s;
+    u32 m = 0x7c00u;                 // "not known to be finite" unless the abs-max says otherwise
     if (GIVEN_SCALE) {
         s = (float)scale_in[row];
     } else {
-        u32 m = 0;
+        m = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             u32 mi = absmax_bits8(v[i]);
@@ -40,9 +41,18 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
         if (threadIdx.x == 0) scale_out[row] = sh;
         s = (float)sh;
     }
+    u32* qr = q + row * (int64_t)cols8;
+    if (fast_quant_ok(m, s)) {       // workgroup-uniform
+        const FastRecip fr = make_fast_recip(s);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            int c = threadIdx.x + i * QT;
+            if (c < cols8) qr[c] = sym_codes8_fast(v[i], fr);
+        }
+        return;
+    }
     const bool fast = scale_fast_ok(s);
     const float rs = fast ? 1.0f / s : 0.0f;
-    u32* qr = q + row * (int64_t)cols8;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         int c = threadIdx.x + i * QT;
