@@ -121,13 +121,17 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
                     blo[j] = (i32x4)((p << 4) & 0xF0F0F0F0u);
                     bhi[j] = (i32x4)(p & 0xF0F0F0F0u);
                 }
+                // all even-k issues first, then all odd-k ones: consecutive MFMAs never share an accumulator
 #pragma unroll
                 for (int i = 0; i < IM; ++i)
 #pragma unroll
-                    for (int j = 0; j < JN; ++j) {
+                    for (int j = 0; j < JN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(blo[j], alo[i], acc[i][j], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < IM; ++i)
+#pragma unroll
+                    for (int j = 0; j < JN; ++j)
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bhi[j], ahi[i], acc[i][j], 0, 0, 0);
-                    }
             }
         }
     };
@@ -236,6 +240,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
 
     // Epilogue.  Accumulator layout (first operand = W rows, second = X rows): lane l, register v ->
     // n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    // column scales (and bias) of this lane's 4-column groups, fetched up front as 8-byte vectors
+    f16x4 sb4[JN][4], bi4[JN][4];
+    if (DEQ) {
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
+                if (col + 4 <= N && (N & 3) == 0) {
+                    sb4[j][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bi4[j][gq] = *(const f16x4*)(bias + col);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int cc = col + e < N ? col + e : N - 1;
+                        sb4[j][gq][e] = sB[cc];
+                        if (bias) bi4[j][gq][e] = bias[cc];
+                    }
+                }
+            }
+    }
 #pragma unroll
     for (int i = 0; i < IM; ++i) {
         const int row = m0 + wm * TM + i * 32 + (lane & 31);
@@ -257,9 +282,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
                     f16 o[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int cc = col + e < N ? col + e : N - 1;
-                        f16 yv = (f16)(sa * sB[cc]) * (f16)(float)v4[e];
-                        if (bias) yv = yv + bias[cc];
+                        f16 yv = (f16)(sa * sb4[j][gq][e]) * (f16)(float)v4[e];
+                        if (bias) yv = yv + bi4[j][gq][e];
                         o[e] = yv;
                     }
                     f16* yp = Y + (int64_t)row * N + col;
@@ -283,6 +307,324 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
             }
         }
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Compute-bound shapes (M > 64): 128x256 workgroup tile, eight waves as 2 (M) x 2 (N) x 2 (K).
+//
+// Both K-groups own the same 64x128 wave tiles and split every 128-k stage between them (group g
+// takes the 64-k sub-step g); they exchange half of their accumulators through LDS at the end.
+// The two waves that share a SIMD belong to different K-groups and run half an iteration out of
+// phase: group 0 reads and unpacks its fragments and then multiplies, group 1 first multiplies the
+// operands it unpacked during the previous iteration and then reads and unpacks the next ones.  So
+// on every SIMD one wave's unpacking (VALU) runs under the other wave's MFMAs instead of both
+// unpacking, then both multiplying.  A stage is 256 k (a full 128-byte line per row, so every line
+// fetched from L2 is used whole); three LDS stages rotate (group 1 reads one stage ahead of group
+// 0), global loads run one more stage ahead through registers, one barrier per stage.
+// (A variant in which half the waves only unpacked into int8 planes in LDS for the other half was
+// measured LDS-bound: twice the LDS bytes at ~128 B/clk/CU exceed the MFMA time.)
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
+__global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
+    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
+    int tiles_m, int tiles_n) {
+    constexpr int NT = 128 * WAVES_M * WAVES_N;
+    constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
+    constexpr int IM = TM / 32, JN = TN / 32;
+    // A stage is 128 packed bytes (256 k) per row = one full cache line, eight 16-byte chunks,
+    // four 64-k sub-steps; K-group g multiplies sub-steps 2g and 2g+1.
+    constexpr int CH = (BM + BN) * 8;
+    constexpr int NL = CH / NT;
+    constexpr int NBUF = 3;
+    constexpr int JH = JN / 2;
+    static_assert(CH % NT == 0 && JN % 2 == 0, "tile shape");
+    extern __shared__ u32x4 ks_lds[];                       // [NBUF][CH]; later the accumulator exchange
+
+    const int nxcd = 8;
+    const int per_xcd = gridDim.x / nxcd;
+    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (tile >= tiles_m * tiles_n) return;
+    constexpr int GROUP_M = 8;
+    const int group_sz = GROUP_M * tiles_n;
+    const int g = tile / group_sz;
+    const int gm0 = g * GROUP_M;
+    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
+    const int tm = gm0 + (tile - g * group_sz) % gh;
+    const int tn = (tile - g * group_sz) / gh;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = wave / (WAVES_M * WAVES_N);
+    const int wxy = wave % (WAVES_M * WAVES_N);
+    const int wm = wxy / WAVES_N, wn = wxy % WAVES_N;
+    const int khalf = lane >> 5;
+    const int stages = (Kb + 127) / 128;
+    // chunk position within a row is XOR-swizzled with (row >> 1) & 7: the 16 rows a quarter-wave
+    // reads at one logical chunk cover all sixteen 16-byte bank groups (row parity picks the half)
+    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
+
+    // ---- staging (all threads): chunk id = tid + i * NT, eight consecutive threads fetch one row's line.
+    // Thread-invariant parts are kept out of registers: the rows of a thread's chunks differ by
+    // multiples of 64 (same swizzle), so LDS slots differ by compile-time constants.
+    static_assert(NT == 512 && BM % 64 == 0 && BN % 64 == 0, "staging layout");
+    const int srow = tid >> 3;
+    const int scoff = (tid & 7) * 16;
+    const int dst0 = slot8(srow, tid & 7);
+    u32 goff[NL];                                           // byte offset of the row from A (i < BM/64) or B
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int row = srow + i * 64;
+        int gr = row < BM ? m0 + row : n0 + row - BM;
+        const int lim = row < BM ? M - 1 : N - 1;
+        gr = gr < lim ? gr : lim;
+        goff[i] = (u32)gr * (u32)Kb;
+    }
+    // branch-free loads: a stage past the end repeats the last one; chunks beyond the row end of a
+    // partly filled last stage re-read the stage's first chunk and are zeroed when written to LDS
+    const bool ragged = (Kb & 127) != 0;
+    auto fetch = [&](int st, u32x4(&r)[NL]) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        const u32 off = (u32)((kb + scoff < Kb) ? kb + scoff : kb);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const uint8_t* base = (i * 64 < BM) ? A : B;
+            r[i] = *(const u32x4*)(base + (size_t)(goff[i] + off));
+        }
+    };
+    auto deposit = [&](int st, int buf, u32x4(&r)[NL]) {
+        if (st < stages) {
+            if (ragged && st == stages - 1 && st * 128 + scoff >= Kb) {
+#pragma unroll
+                for (int i = 0; i < NL; ++i) r[i] = u32x4{0, 0, 0, 0};
+            }
+            u32x4* base = ks_lds + buf * CH + dst0;
+#pragma unroll
+            for (int i = 0; i < NL; ++i) base[i * 64 * 8] = r[i];
+        }
+    };
+
+    i32x16 acc[IM][JN];
+#pragma unroll
+    for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    // this wave's fragment slots for its two sub-steps (u = 0, 1): logical chunk (2 kg + u) * 2 + khalf;
+    // tile rows differ by multiples of 32 (same swizzle): compile-time offsets
+    int aslot[2], bslot[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        aslot[u] = slot8(wm * TM + (lane & 31), (2 * kg + u) * 2 + khalf);
+        bslot[u] = slot8(BM + wn * TN + (lane & 31), (2 * kg + u) * 2 + khalf);
+    }
+    struct Ops {
+        i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
+    };
+    auto load_ops = [&](int buf, int u, Ops& o) {
+        const u32x4* pa = ks_lds + buf * CH + (u ? aslot[1] : aslot[0]);
+        const u32x4* pb = ks_lds + buf * CH + (u ? bslot[1] : bslot[0]);
+#pragma unroll
+        for (int i = 0; i < IM; ++i) {
+            const u32x4 p = pa[i * 32 * 8];
+            o.alo[i] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+            o.ahi[i] = (i32x4)(p & 0xF0F0F0F0u);
+        }
+#pragma unroll
+        for (int j = 0; j < JN; ++j) {
+            const u32x4 p = pb[j * 32 * 8];
+            o.blo[j] = (i32x4)((p << 4) & 0xF0F0F0F0u);
+            o.bhi[j] = (i32x4)(p & 0xF0F0F0F0u);
+        }
+    };
+    auto multiply = [&](const Ops& o) {
+        // all even-k issues first, then all odd-k ones: consecutive MFMAs never share an accumulator
+#pragma unroll
+        for (int i = 0; i < IM; ++i)
+#pragma unroll
+            for (int j = 0; j < JN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.blo[j], o.alo[i], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < IM; ++i)
+#pragma unroll
+            for (int j = 0; j < JN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.bhi[j], o.ahi[i], acc[i][j], 0, 0, 0);
+    };
+
+    // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during iteration
+    // ks from registers requested at the end of iteration ks-1 (a second register set would spill).
+    u32x4 regs[NL];
+    fetch(0, regs);
+    deposit(0, 0, regs);
+    fetch(1, regs);
+    deposit(1, 1, regs);
+    fetch(2, regs);
+    __syncthreads();                                        // stages 0 and 1 visible
+    Ops ops;
+    if (kg == 1) load_ops(0, 0, ops);                       // group 1 starts one unpack ahead
+    int bcur = 0;
+    for (int ks = 0; ks < stages; ++ks) {
+        const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+        const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
+        if (kg == 0) {
+            load_ops(bcur, 0, ops);
+            multiply(ops);
+            load_ops(bcur, 1, ops);
+            multiply(ops);
+        } else {
+            multiply(ops);                                  // sub-step 2 of this stage (unpacked earlier)
+            load_ops(bcur, 1, ops);
+            multiply(ops);                                  // sub-step 3
+            if (ks + 1 < stages) load_ops(bnext, 0, ops);   // next stage's sub-step 2
+        }
+        deposit(ks + 2, bfill, regs);
+        fetch(ks + 3, regs);
+        __syncthreads();
+        bcur = bnext;
+    }
+
+    // K-split: group 0 finalises the lower half of the j tiles and group 1 the upper half; each sends
+    // the other half across, one row of MFMA tiles (i) per round, four 16-byte pieces per lane.
+    const int j_first = kg * JH;
+    {
+        u32x4* xbuf = ks_lds;
+        const int send0 = (1 - kg) * JH;
+        for (int i = 0; i < IM; ++i) {
+            __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < JH; ++jj)
+#pragma unroll
+                for (int qv = 0; qv < 4; ++qv) {
+                    const int slot = (((wxy * 2 + (1 - kg)) * JH + jj) * 4 + qv) * 64 + lane;
+                    i32x4 piece;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        int val = 0;
+#pragma unroll
+                        for (int ii = 0; ii < IM; ++ii)
+#pragma unroll
+                            for (int jx = 0; jx < JN; ++jx)
+                                if (ii == i && jx == send0 + jj) val = acc[ii][jx][qv * 4 + e];
+                        piece[e] = val;
+                    }
+                    xbuf[slot] = (u32x4)piece;
+                }
+            __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < JH; ++jj)
+#pragma unroll
+                for (int qv = 0; qv < 4; ++qv) {
+                    const int slot = (((wxy * 2 + kg) * JH + jj) * 4 + qv) * 64 + lane;
+                    const i32x4 piece = (i32x4)xbuf[slot];
+#pragma unroll
+                    for (int ii = 0; ii < IM; ++ii)
+#pragma unroll
+                        for (int jx = 0; jx < JN; ++jx)
+                            if (ii == i && jx == j_first + jj) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[ii][jx][qv * 4 + e] += piece[e];
+                            }
+                }
+        }
+    }
+
+    // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    // column scales (and bias) of this lane's 4-column groups, fetched up front as 8-byte vectors
+    f16x4 sb4[JH][4], bi4[JH][4];                          // only the j tiles this K-group stores
+    if (DEQ) {
+#pragma unroll
+        for (int jj = 0; jj < JH; ++jj)
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + (j_first + jj) * 32 + gq * 8 + khalf * 4;
+                if (col + 4 <= N && (N & 3) == 0) {
+                    sb4[jj][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bi4[jj][gq] = *(const f16x4*)(bias + col);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int cc = col + e < N ? col + e : N - 1;
+                        sb4[jj][gq][e] = sB[cc];
+                        if (bias) bi4[jj][gq][e] = bias[cc];
+                    }
+                }
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < IM; ++i) {
+        const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (row >= M) continue;
+        f16 sa = (f16)0;
+        if (DEQ) sa = sA[row];
+#pragma unroll
+        for (int j = 0; j < JN; ++j) {
+            if (j < j_first || j >= j_first + JH) continue;     // the other K-group stores this tile
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
+                if (col >= N) continue;
+                int v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
+                const bool whole = (col + 4 <= N) && ((N & 3) == 0);
+                if (DEQ) {
+                    f16 o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        f16 yv = (f16)(sa * sb4[j % JH][gq][e]) * (f16)(float)v4[e];
+                        if (bias) yv = yv + bi4[j % JH][gq][e];
+                        o[e] = yv;
+                    }
+                    f16* yp = Y + (int64_t)row * N + col;
+                    if (whole) {
+                        *(f16x4*)yp = f16x4{o[0], o[1], o[2], o[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < N) yp[e] = o[e];
+                    }
+                } else {
+                    int32_t* cp = C + (int64_t)row * N + col;
+                    if (whole) {
+                        *(i32x4*)cp = i32x4{v4[0], v4[1], v4[2], v4[3]};
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < N) cp[e] = v4[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+              const void* bias, hipStream_t st) {
+    constexpr int NT = 128 * WAVES_M * WAVES_N;
+    constexpr size_t STAGES = (size_t)3 * (BM + BN) * 8 * 16;
+    constexpr size_t XCH = (size_t)WAVES_M * WAVES_N * 2 * (BN / WAVES_N / 64) * 256 * 16;
+    constexpr size_t LDS = STAGES > XCH ? STAGES : XCH;
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles > 0x3fffffff) return QR_E_SHAPE;
+    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    hipError_t e;
+    if (Y) {
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, true>;
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
+                                                (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+    } else {
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
+                                                nullptr, nullptr, nullptr, tiles_m, tiles_n);
+    }
+    return qr_launch_status();
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT>
@@ -316,9 +658,8 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     if (M <= 32) return launch_cfg<32, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     if (M <= 64) return launch_cfg<64, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    if (t256 >= 512) return launch_cfg<256, 256, 4, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 128) return launch_cfg<128, 256, 2, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t128x256 >= 128) return launch_ks<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
 
