@@ -599,6 +599,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
               const void* bias, hipStream_t st) {
@@ -624,6 +625,304 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
     }
+    return qr_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode (M <= 64): the weights are streamed once from HBM and nothing is reused, so no LDS
+// staging.  A workgroup of eight waves owns 32 weight rows; the waves split K into eight contiguous
+// ranges, each wave loads its W fragments (16 bytes per lane, straight into registers) and the
+// matching X fragments (small, L2-resident), unpacks and multiplies; the eight partial 32 x M tiles
+// are summed through LDS and dequantised.  Loads run PF steps ahead in a register ring.
+template <int MT, bool DEQ>
+__global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                        int M, int N, int Kb, int32_t* __restrict__ C,
+                                                        f16* __restrict__ Y, const f16* __restrict__ sA,
+                                                        const f16* __restrict__ sB, const f16* __restrict__ bias) {
+    constexpr int PF = 4;                                   // steps in flight; a step = 64 packed bytes (128 k) per row
+    __shared__ i32x4 red[8 * MT * 4 * 64];                  // [wave][m tile][4-register group][lane]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * 32;
+    const int steps = (Kb + 63) / 64;
+    const int s_begin = (int)((int64_t)steps * wave / 8), s_end = (int)((int64_t)steps * (wave + 1) / 8);
+
+    int nr = n0 + r;
+    nr = nr < N ? nr : N - 1;
+    const uint8_t* wp = B + (int64_t)nr * Kb + h * 32;
+    const uint8_t* xp[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        int mr = t * 32 + r;
+        mr = mr < M ? mr : M - 1;
+        xp[t] = A + (int64_t)mr * Kb + h * 32;
+    }
+    // in a half-full last step (K % 128 == 64) the upper 32 bytes lie beyond the row: those lanes
+    // re-read the lower half and their fragments are zeroed
+    const bool half_tail = (Kb & 63) != 0;
+    struct Step {
+        u32x4 w[2], x[MT][2];
+    };
+    auto fetch = [&](int sidx, Step& st) {
+        const int sc = sidx < steps ? sidx : steps - 1;
+        const bool dead = half_tail && sc == steps - 1 && h == 1;
+        const int off = sc * 64 - (dead ? 32 : 0);
+        st.w[0] = __builtin_nontemporal_load((const u32x4*)(wp + off));
+        st.w[1] = __builtin_nontemporal_load((const u32x4*)(wp + off + 16));
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            st.x[t][0] = *(const u32x4*)(xp[t] + off);
+            st.x[t][1] = *(const u32x4*)(xp[t] + off + 16);
+        }
+    };
+    i32x16 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0;
+    auto consume = [&](int sidx, const Step& st) {
+        const bool dead = half_tail && sidx == steps - 1 && h == 1;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const u32x4 wq = dead ? u32x4{0, 0, 0, 0} : st.w[c];
+            const i32x4 wlo = (i32x4)((wq << 4) & 0xF0F0F0F0u), whi = (i32x4)(wq & 0xF0F0F0F0u);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const i32x4 xlo = (i32x4)((st.x[t][c] << 4) & 0xF0F0F0F0u), xhi = (i32x4)(st.x[t][c] & 0xF0F0F0F0u);
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, xlo, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, xhi, acc[t], 0, 0, 0);
+            }
+        }
+    };
+    Step ring[PF];
+#pragma unroll
+    for (int p = 0; p < PF; ++p) fetch(s_begin + p, ring[p]);
+    for (int s = s_begin; s < s_end; s += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; ++p) {
+            if (s + p < s_end) {
+                consume(s + p, ring[p]);
+                fetch(s + p + PF, ring[p]);                 // indices past the end re-read the last step (unused)
+            }
+        }
+    }
+    // ---- sum the eight partial tiles
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq)
+            red[((wave * MT + t) * 4 + gq) * 64 + lane] = i32x4{acc[t][gq * 4], acc[t][gq * 4 + 1], acc[t][gq * 4 + 2], acc[t][gq * 4 + 3]};
+    __syncthreads();
+    // unit u = (m tile, register group): one wave each
+    if (wave < MT * 4) {
+        const int t = wave >> 2, gq = wave & 3;
+        i32x4 sum = {0, 0, 0, 0};
+#pragma unroll
+        for (int w = 0; w < 8; ++w) sum += red[((w * MT + t) * 4 + gq) * 64 + lane];
+        const int row = t * 32 + r;
+        const int col = n0 + gq * 8 + h * 4;
+        if (row < M && col < N) {
+            const bool whole = (col + 4 <= N) && ((N & 3) == 0);
+            if (DEQ) {
+                const f16 sa = sA[row];
+                f16 o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int cc = col + e < N ? col + e : N - 1;
+                    f16 yv = (f16)(sa * sB[cc]) * (f16)(float)(sum[e] >> 8);
+                    if (bias) yv = yv + bias[cc];
+                    o[e] = yv;
+                }
+                f16* yp = Y + (int64_t)row * N + col;
+                if (whole) {
+                    *(f16x4*)yp = f16x4{o[0], o[1], o[2], o[3]};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) yp[e] = o[e];
+                }
+            } else {
+                int32_t* cp = C + (int64_t)row * N + col;
+                if (whole) {
+                    *(i32x4*)cp = i32x4{sum[0] >> 8, sum[1] >> 8, sum[2] >> 8, sum[3] >> 8};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) cp[e] = sum[e] >> 8;
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode with very few tokens (M <= 8): a matrix-vector style kernel on the native int4 dot product
+// (v_dot8_i32_i4: eight signed 4-bit products per lane and instruction, no unpacking).  A wave owns
+// groups of four weight rows and walks K in 1 KB segments: lane l loads bytes [l*16, l*16+16) of
+// each row's segment -- every load instruction reads 1 KB of contiguous weight bytes -- and the
+// matching 16 bytes of each token's codes (shared by the four rows, L1/L2 resident).  A wave takes
+// `ng` consecutive row groups as one flattened sequence of segments, so the loads of the next group
+// are already in flight while the current one finishes.  The 64 partial sums of each (row, token)
+// pair are added across the wave by a halving exchange (each step gives away half of the values a
+// lane still holds), which costs one cross-lane move per value instead of six.
+template <int MB, bool DEQ>
+__global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                      int M, int N, int Kb, int ng, int32_t* __restrict__ C,
+                                                      f16* __restrict__ Y, const f16* __restrict__ sA,
+                                                      const f16* __restrict__ sB, const f16* __restrict__ bias) {
+    constexpr int R = 4;                                    // rows per group
+    constexpr int NV = R * MB;                              // sums per group
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g0 = (blockIdx.x * 4 + wave) * ng;            // first row group of this wave
+    const int groups = (N + R - 1) / R;
+    if (g0 >= groups) return;
+    const int gcount = groups - g0 < ng ? groups - g0 : ng;
+    const int nseg = (Kb + 1023) / 1024;
+    const int total = gcount * nseg;                        // flattened (group, segment) items
+    const uint8_t* xp[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+        const int mr = m < M ? m : M - 1;
+        xp[m] = A + (int64_t)mr * Kb + lane * 16;
+    }
+    struct Seg {
+        u32x4 w[R], x[MB];
+    };
+    // fetch side: position (fg, fs) runs ahead of the consume side
+    int fg = 0, fs = 0;
+    auto fetch = [&](Seg& g) {
+        // a lane whose 16 bytes lie beyond the row end re-reads the row start and contributes nothing;
+        // items past the end of the sequence re-read the last one
+        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int nr = (g0 + fg) * R + r;
+            nr = nr < N ? nr : N - 1;
+            g.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
+        }
+#pragma unroll
+        for (int m = 0; m < MB; ++m) g.x[m] = *(const u32x4*)(xp[m] - lane * 16 + off);
+        if (fs + 1 < nseg) ++fs;
+        else if (fg + 1 < gcount) { ++fg; fs = 0; }
+    };
+    int acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = 0;
+    int cg = 0, cs = 0;
+    auto consume = [&](const Seg& g) {
+        if (cs * 1024 + lane * 16 < Kb) {
+#pragma unroll
+            for (int m = 0; m < MB; ++m)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                        acc[m * R + r] = __builtin_amdgcn_sdot8((int)g.w[r][d], (int)g.x[m][d], acc[m * R + r], false);
+        }
+        if (++cs < nseg) return;
+        // ---- end of a row group: halving exchange.  After the steps with offsets 32, 16, ... a lane
+        // holds the sum of value index (bits of its lane id, most significant first) over the lanes
+        // that agree with it on those bits; the remaining offsets finish the sum.
+        int vals[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) vals[v] = acc[v];
+        int off = 32;
+#pragma unroll
+        for (int cur = NV; cur > 1; cur >>= 1) {
+            const bool upper = (lane & off) != 0;
+#pragma unroll
+            for (int i = 0; i < cur / 2; ++i) {
+                const int give = upper ? vals[i] : vals[i + cur / 2];
+                const int keep = upper ? vals[i + cur / 2] : vals[i];
+                vals[i] = keep + __shfl_xor(give, off, QR_WAVE);
+            }
+            off >>= 1;
+        }
+        int sum = vals[0];
+        for (; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
+        // which value this lane ended up with: log2(NV) lane bits from bit 5 downwards
+        constexpr int LV = NV == 4 ? 2 : NV == 8 ? 3 : NV == 16 ? 4 : 5;
+        const int vidx = lane >> (6 - LV);
+        if ((lane & ((1 << (6 - LV)) - 1)) == 0) {
+            const int m = vidx / R, r = vidx % R;
+            const int col = (g0 + cg) * R + r;
+            if (m < M && col < N) {
+                if (DEQ) {
+                    f16 yv = (f16)(sA[m] * sB[col]) * (f16)(float)sum;
+                    if (bias) yv = yv + bias[col];
+                    Y[(int64_t)m * N + col] = yv;
+                } else {
+                    C[(int64_t)m * N + col] = sum;
+                }
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] = 0;
+        cs = 0;
+        ++cg;
+    };
+    Seg ga, gb, gc;
+    fetch(ga);
+    fetch(gb);
+    fetch(gc);
+    for (int it = 0; it < total; it += 3) {
+        consume(ga);
+        fetch(ga);
+        if (it + 1 < total) {
+            consume(gb);
+            fetch(gb);
+        }
+        if (it + 2 < total) {
+            consume(gc);
+            fetch(gc);
+        }
+    }
+}
+
+int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+                const void* bias, hipStream_t st) {
+    const int groups = (N + 3) / 4;
+    // row groups per wave: at least ~64 KB of weights per wave, but keep >= 2048 waves when N allows
+    int ng = (65536 + 4 * Kb - 1) / (4 * Kb);
+    while (ng > 1 && groups / ng < 2048) --ng;
+    const int waves = (groups + ng - 1) / ng;
+    const unsigned grid = (unsigned)((waves + 3) / 4);
+#define QR_GEMV(MB)                                                                                                   \
+    do {                                                                                                              \
+        if (Y)                                                                                                        \
+            gemv_i4_kernel<MB, true><<<dim3(grid), dim3(256), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, \
+                                                                       ng, nullptr, (f16*)Y, (const f16*)sA,          \
+                                                                       (const f16*)sB, (const f16*)bias);             \
+        else                                                                                                          \
+            gemv_i4_kernel<MB, false><<<dim3(grid), dim3(256), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N,   \
+                                                                        Kb, ng, (int32_t*)C, nullptr, nullptr,        \
+                                                                        nullptr, nullptr);                            \
+    } while (0)
+    if (M <= 1) QR_GEMV(1);
+    else if (M <= 2) QR_GEMV(2);
+    else if (M <= 4) QR_GEMV(4);
+    else QR_GEMV(8);
+#undef QR_GEMV
+    return qr_launch_status();
+}
+
+int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+                  const void* bias, hipStream_t st) {
+    const unsigned grid = (unsigned)((N + 31) / 32);
+#define QR_DEC(MT)                                                                                                    \
+    do {                                                                                                              \
+        if (Y)                                                                                                        \
+            decode_i4_kernel<MT, true><<<dim3(grid), dim3(512), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N,  \
+                                                                         Kb, nullptr, (f16*)Y, (const f16*)sA,        \
+                                                                         (const f16*)sB, (const f16*)bias);           \
+        else                                                                                                          \
+            decode_i4_kernel<MT, false><<<dim3(grid), dim3(512), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, \
+                                                                          Kb, (int32_t*)C, nullptr, nullptr, nullptr, \
+                                                                          nullptr);                                   \
+    } while (0)
+    if (M <= 32) QR_DEC(1);
+    else QR_DEC(2);
+#undef QR_DEC
     return qr_launch_status();
 }
 
@@ -656,8 +955,17 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M <= 32) return launch_cfg<32, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    if (M <= 64) return launch_cfg<64, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 8) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 64) {
+        // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
+        // once per tile); otherwise eight waves split K over 32 rows
+        if ((N + 255) / 256 >= 128) {
+            if (M <= 32) return launch_cfg<32, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+            return launch_cfg<64, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        }
+        return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    }
+    if (t256 >= 512) return launch_cfg<256, 256, 4, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
     if (t128x256 >= 128) return launch_ks<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
