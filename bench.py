@@ -11,6 +11,9 @@ outlier channels that motivate the Hadamard):
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
     c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
     c4  down_proj 70B decode  X [64, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28
+        (c4m1, c4m8: 1 / 8 tokens; c4g1, c4g8, c4g64: gate_up W int4 [57344, 8192])
+Decode workloads (M <= 64) rotate among several copies of the weights so that they are streamed from
+HBM rather than from the 256 MB last-level cache.
 Prints ONE JSON line on stdout (metric = TOPS of the whole step, 2.M.N.K / t).
 """
 import argparse
@@ -31,7 +34,12 @@ WORKLOADS = {
     "c1": (2048, 4096, 4096, False),
     "c2": (2048, 11008, 4096, True),
     "c3d": (32768, 11008, 4096, True),
-    "c4": (64, 28672, 8192, True),
+    "c4": (64, 28672, 8192, True),          # decode, 70B down_proj
+    "c4m1": (1, 28672, 8192, True),
+    "c4m8": (8, 28672, 8192, True),
+    "c4g1": (1, 8192, 57344, False),        # decode, 70B gate_up (input already quantised upstream: no Hadamard)
+    "c4g8": (8, 8192, 57344, False),
+    "c4g64": (64, 8192, 57344, False),
 }
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 HBM_PEAK_GBS = 8000.0
@@ -107,12 +115,20 @@ def main():
     lin.weight.copy_(w_cpu.to(dev))
     lin.weight_scales.copy_(sw_cpu.to(dev))
     front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if hadamard else quarot_amd.nn.Quantizer()).to(dev)
+    # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
+    copies = [lin.weight]
+    if m <= 64:
+        while sum(c.numel() for c in copies) < 640 * 1024 * 1024:
+            copies.append(lin.weight.clone())
+    state = {"i": 0}
 
     def step(ev=None):
         p = front(x)
         if ev is not None:
             ev[0].record()
-        y = lin(p)
+        w = copies[state["i"] % len(copies)]
+        state["i"] += 1
+        y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, w, lin.weight_scales, lin.bias)
         if ev is not None:
             ev[1].record()
         return y
@@ -153,7 +169,9 @@ def main():
         roof = {"bound": "mfma", "achieved": round(ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
                 "unit": "TFLOP/s", "traffic": None}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = "gemm_i4_kernel (int4 GEMM + dequant epilogue)"
+    roof["kernel"] = ("gemv_i4_kernel" if m <= 8 else "decode_i4_kernel / gemm_i4_kernel" if decode else
+                      "gemm_ks_kernel" if ((m + 255) // 256) * ((n + 255) // 256) < 512 else "gemm_i4_kernel<256,256>")
+    roof["kernel"] += " (int4 GEMM + dequant epilogue)"
     roof["kernel_ms"] = round(gemm_ms, 4)
 
     out = {

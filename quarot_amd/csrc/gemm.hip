@@ -614,13 +614,13 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
     hipError_t e;
     if (Y) {
         auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, true>;
-        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
     } else {
         auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
-        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);

@@ -454,7 +454,7 @@ int launch_hadamard_km(const void* x, void* y, int64_t rows, int n, int K, int l
     do {                                                                                                              \
         auto kern = hadamard_km_kernel<MODE32, QUANT, NCH>;                                                           \
         if (lds > 48 * 1024) {                                                                                        \
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
             if (e != hipSuccess) return (int)e;                                                                       \
         }                                                                                                             \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, log2m, hadK, scale, clip, (u32*)q, \
@@ -719,7 +719,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
     do {                                                                                                               \
         auto kern = hadamard_mm_kernel<MODE32, QUANT, L2M, KS>;                                                        \
         if (lds > 48 * 1024) {                                                                                         \
-            hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+            hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
             if (e != hipSuccess) return (int)e;                                                                        \
         }                                                                                                              \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
@@ -741,6 +741,193 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
     return qr_launch_status();
 }
 
+// ---- K > 1 with a long power-of-two factor (m = 512 or 1024), fp16 I/O ---------------------------
+// Decode-sized inputs have few rows, so the row itself must supply the parallelism: 1024 threads per
+// row.  A wave transforms whole segments in registers (8 values per chunk, 64 lanes, CPL chunks per
+// lane: 3 + 6 + log2(CPL) butterfly levels, no LDS), scatters the scaled fp16 results into LDS in
+// MFMA-fragment order, and the hadK factor then runs on the matrix cores as in hadamard_mm_kernel
+// (T^T as first operand, hadK fragments in registers, 8-byte result writes).  All of a row's loads are
+// issued at once and the next row's are requested before the matrix stage.
+template <bool QUANT, int CPL>
+__global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
+                                                           int n, int K, const f16* __restrict__ hadK, float scale,
+                                                           float clip, u32* __restrict__ q, f16* __restrict__ scales) {
+    constexpr int BT = 1024, NW = 16;
+    constexpr int M_ = 512 * CPL, LOG2M = CPL == 1 ? 9 : 10;
+    constexpr int CT = M_ / 16;                  // 16-column tiles
+    constexpr int SPW = 4 / CPL;                 // segments per wave (K <= 16 * SPW)
+    constexpr int KS2 = CPL == 1 ? 2 : 1;        // contraction steps of 32
+    constexpr int RT = SPW;                      // 16-row tiles of hadK
+    constexpr int TS = 17;                       // u32x4 units per (step, k-group, column tile): 16 + 1 pad
+    constexpr int YS = M_ + 8;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[NW];
+    u32x4* Tl = (u32x4*)smem_raw;                // [KS2][4][CT][TS]
+    f16* Yl = (f16*)(Tl + KS2 * 4 * CT * TS);    // [K][YS]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int nchunks = n >> 3;
+
+    // hadK fragments (second MFMA operand): column k' = rt*16 + l16, contraction k = ks*32 + g*8 + j
+    f16x8 hf[RT][KS2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int hr = rt * 16 + l16, hc = ks * 32 + g * 8 + hh * 4;
+                f16x4 v = {(f16)0, (f16)0, (f16)0, (f16)0};
+                if (hr < K && hc < K) v = *(const f16x4*)(hadK + hr * K + hc);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hf[rt][ks][hh * 4 + e] = v[e];
+            }
+    // slots of T for k >= K are never written afterwards: clear once
+    for (int i = tid; i < KS2 * 4 * CT * TS; i += BT) Tl[i] = u32x4{0, 0, 0, 0};
+
+    u32x4 raw[SPW][CPL];
+    auto request = [&](int64_t row) {
+#pragma unroll
+        for (int sg = 0; sg < SPW; ++sg) {
+            const int k = wave + NW * sg;
+#pragma unroll
+            for (int i = 0; i < CPL; ++i)
+                raw[sg][i] = k < K ? __builtin_nontemporal_load((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
+                                   : u32x4{0, 0, 0, 0};
+        }
+    };
+    int64_t row = blockIdx.x;
+    if (row < rows) request(row);
+    __syncthreads();
+    for (; row < rows; row += gridDim.x) {
+        // ---- phase 1: per-segment transform in registers, scatter to fragment order
+#pragma unroll
+        for (int sg = 0; sg < SPW; ++sg) {
+            const int k = wave + NW * sg;
+            if (k < K) {
+                float v[CPL][8];
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        v[i][2 * w] = (float)f16_from_bits((unsigned short)(raw[sg][i][w] & 0xffffu));
+                        v[i][2 * w + 1] = (float)f16_from_bits((unsigned short)(raw[sg][i][w] >> 16));
+                    }
+                    reg_fwht8(v[i]);
+                    lane_stage<1>(v[i], lane);
+                    lane_stage<2>(v[i], lane);
+                    lane_stage<4>(v[i], lane);
+                    lane_stage<8>(v[i], lane);
+                    lane_stage<16>(v[i], lane);
+                    lane_stage<32>(v[i], lane);
+                }
+                if (CPL == 2) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float a = v[0][e], b = v[CPL - 1][e];
+                        v[0][e] = a + b;
+                        v[CPL - 1][e] = a - b;
+                    }
+                }
+                const int ks = k >> 5, kgp = (k & 31) >> 3, kj = k & 7;
+#pragma unroll
+                for (int i = 0; i < CPL; ++i) {
+                    const int r0 = (i * 64 + lane) * 8;
+                    f16* dst = (f16*)(Tl + ((ks * 4 + kgp) * CT + (r0 >> 4)) * TS + (r0 & 8)) + kj;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) dst[e * 8] = narrow_f16(v[i][e] * scale);
+                }
+            }
+        }
+        const int64_t nrow = row + gridDim.x;
+        if (nrow < rows) request(nrow);
+        __syncthreads();
+        // ---- stage 2: Y^T = T^T . hadK^T
+        for (int ct = wave * (CT / NW); ct < (wave + 1) * (CT / NW); ++ct) {
+            f16x8 th[KS2];
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) th[ks] = __builtin_bit_cast(f16x8, Tl[((ks * 4 + g) * CT + ct) * TS + l16]);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                if (rt * 16 < K) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS2; ++ks)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(th[ks], hf[rt][ks], acc, 0, 0, 0);
+                    const int kp = rt * 16 + l16;
+                    if (kp < K) {
+                        u32x2 o;
+                        o[0] = (u32)f16_bits((f16)acc[0]) | ((u32)f16_bits((f16)acc[1]) << 16);
+                        o[1] = (u32)f16_bits((f16)acc[2]) | ((u32)f16_bits((f16)acc[3]) << 16);
+                        *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        // ---- stage 3
+        if (QUANT) {
+            u32 mx = 0;
+            for (int c = tid; c < nchunks; c += BT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                const u32 mc = absmax_bits8(h);
+                mx = mx > mc ? mx : mc;
+            }
+            mx = wave_max_u32(mx);
+            if (lane == 0) red[wave] = mx;
+            __syncthreads();
+#pragma unroll
+            for (int w = 0; w < NW; ++w) mx = mx > red[w] ? mx : red[w];
+            const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+            if (tid == 0) scales[row] = sh;
+            const float s = (float)sh;
+            const bool lean = fast_quant_ok(mx, s);
+            const FastRecip fq = make_fast_recip(lean ? s : 1.0f);
+            const bool fast = scale_fast_ok(s);
+            const float rs = fast ? 1.0f / s : 0.0f;
+            for (int c = tid; c < nchunks; c += BT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                q[row * (int64_t)nchunks + c] = lean ? sym_codes8_fast(h, fq) : sym_codes8(h, s, rs, fast);
+                if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            }
+        } else {
+            for (int c = tid; c < nchunks; c += BT) {
+                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            }
+        }
+        // the next row's phase 1 writes Tl (last read before the barrier above) and its stage 2 writes
+        // Yl only after the barrier that follows that phase 1
+    }
+}
+
+bool bm_applies(int n, int K) {
+    if (K <= 1) return false;
+    const int m = n / K;
+    return (m == 512 && K <= 64) || (m == 1024 && K <= 32);
+}
+
+template <bool QUANT>
+int launch_hadamard_bm(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
+                       void* q, void* scales, hipStream_t st) {
+    const int m = n / K;
+    const int cpl = m / 512;
+    const size_t lds = (size_t)(cpl == 1 ? 2 : 1) * 4 * (m / 16) * 17 * 16 + (size_t)K * (m + 8) * 2;
+    const unsigned grid = (unsigned)(rows < 256 ? rows : 256);
+#define QR_BM(CPL)                                                                                                     \
+    do {                                                                                                               \
+        auto kern = hadamard_bm_kernel<QUANT, CPL>;                                                                    \
+        hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);   \
+        if (e != hipSuccess) return (int)e;                                                                            \
+        kern<<<dim3(grid), dim3(1024), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, (const f16*)hadK, scale, clip,   \
+                                                  (u32*)q, (f16*)scales);                                              \
+    } while (0)
+    if (cpl == 1) QR_BM(1);
+    else QR_BM(2);
+#undef QR_BM
+    return qr_launch_status();
+}
+
 template <typename IO, bool MODE32, bool QUANT>
 int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
                     void* q, void* scales, hipStream_t st) {
@@ -753,7 +940,7 @@ int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const vo
     if (lds > 160 * 1024 - 64) return QR_E_UNSUPPORTED;
     auto kern = hadamard_kernel<IO, MODE32, QUANT>;
     if (lds > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);
         if (e != hipSuccess) return (int)e;
     }
     // persistent workgroups: as many as fit the CUs' LDS at once (256 CUs, 160 KB each), so that the
@@ -786,6 +973,8 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == QR_DTYPE_F16 && bm_applies(n, K))
+        return launch_hadamard_bm<false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && mm_applies(n, K))
         return launch_hadamard_mm<false, false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && km_applies(n, K, false)) {
@@ -808,6 +997,8 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (mode == QR_DTYPE_F16 && bm_applies(n, K))
+        return launch_hadamard_bm<true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     if (mm_applies(n, K)) {
         if (mode == QR_DTYPE_F16) return launch_hadamard_mm<false, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
         return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);

@@ -18,6 +18,26 @@ typedef u32 u32x4 __attribute__((ext_vector_type(4)));
 
 #define QR_WAVE 64
 
+// Raise a kernel's dynamic-LDS limit, once per (kernel, device, size): the runtime call costs host
+// time on every launch otherwise.  A benign race at first use only repeats the call.
+static inline hipError_t qr_allow_dynamic_lds(const void* kernel, size_t bytes) {
+    struct Entry {
+        const void* fn;
+        int dev;
+        size_t bytes;
+    };
+    static Entry table[64];
+    static int used = 0;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    for (int i = 0; i < used; ++i)
+        if (table[i].fn == kernel && table[i].dev == dev && table[i].bytes >= bytes) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess && used < 64) table[used++] = Entry{kernel, dev, bytes};
+    return e;
+}
+
 static inline int qr_launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? QR_OK : (int)e;
