@@ -446,10 +446,6 @@ int launch_hadamard_km(const void* x, void* y, int64_t rows, int n, int K, int l
     const int Kc = (K + 31) & ~31;
     const size_t lds = (size_t)(MODE32 ? 2 : 1) * m * (Kc + 8) * 2 + (size_t)K * (m + 8) * 2;
     const int nch = ((n >> 3) + HT - 1) / HT;
-    int per_cu = (int)((160 * 1024) / (lds + 1024));
-    per_cu = per_cu < 1 ? 1 : (per_cu > 4 ? 4 : per_cu);
-    const int64_t cap = 256LL * per_cu;
-    const unsigned grid = (unsigned)(rows < cap ? rows : cap);
 #define QR_KM(NCH)                                                                                                    \
     do {                                                                                                              \
         auto kern = hadamard_km_kernel<MODE32, QUANT, NCH>;                                                           \
@@ -457,6 +453,8 @@ int launch_hadamard_km(const void* x, void* y, int64_t rows, int n, int K, int l
             hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
             if (e != hipSuccess) return (int)e;                                                                       \
         }                                                                                                             \
+        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);                                     \
+        const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                    \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, log2m, hadK, scale, clip, (u32*)q, \
                                                 (f16*)scales);                                                        \
     } while (0)
@@ -531,7 +529,11 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
                 const int hc = ks * 32 + hh * 16 + g * 4;
                 f16x4 v = {(f16)0, (f16)0, (f16)0, (f16)0};
                 if (hr < K && hc < K) {
-                    if (MODE32) {
+                    if (hadK == nullptr) {
+                        // power-of-two row: the outer factor is the Sylvester matrix of order K itself
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (__builtin_popcount(hr & (hc + e)) & 1) ? (f16)-1.0f : (f16)1.0f;
+                    } else if (MODE32) {
                         const f32x4 w = *(const f32x4*)((const float*)hadK + hr * K + hc);
                         v = f16x4{(f16)w[0], (f16)w[1], (f16)w[2], (f16)w[3]};
                     } else {
@@ -699,6 +701,14 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
     }
 }
 
+// A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
+// kernel applies with a generated outer factor, in its fp32-precision mode so that the result is
+// rounded to fp16 once, like a plain fp32 transform.  Returns the outer order (0: not applicable).
+int pow2_split(int n) {
+    if (n < 1024 || n > 16384 || (n & (n - 1)) != 0) return 0;
+    return n <= 8192 ? n / 64 : n / 128;
+}
+
 bool mm_applies(int n, int K) {
     if (K <= 1 || K > 32 * KS_MAX) return false;
     const int m = n / K;
@@ -711,10 +721,6 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
     const size_t lds = (size_t)(MODE32 ? 2 : 1) * (m / 16) * KS2 * 64 * 16 + (size_t)K * (m + 8) * 2;
-    int per_cu = (int)((160 * 1024) / (lds + 1024));
-    per_cu = per_cu < 1 ? 1 : (per_cu > 2 ? 2 : per_cu);
-    const int64_t cap = 256LL * per_cu;
-    const unsigned grid = (unsigned)(rows < cap ? rows : cap);
 #define QR_MM(L2M, KS)                                                                                                 \
     do {                                                                                                               \
         auto kern = hadamard_mm_kernel<MODE32, QUANT, L2M, KS>;                                                        \
@@ -722,6 +728,8 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
             hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
             if (e != hipSuccess) return (int)e;                                                                        \
         }                                                                                                              \
+        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);                                      \
+        const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
                                                 (f16*)scales);                                                         \
     } while (0)
@@ -945,9 +953,7 @@ int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const vo
     }
     // persistent workgroups: as many as fit the CUs' LDS at once (256 CUs, 160 KB each), so that the
     // hadK staging is paid once per resident workgroup
-    int per_cu = (int)((160 * 1024) / (lds + 1024));
-    per_cu = per_cu < 1 ? 1 : (per_cu > 8 ? 8 : per_cu);
-    const int64_t cap = 256LL * per_cu;
+    const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);
     const int64_t grid = rows < cap ? rows : cap;
     kern<<<dim3((unsigned)grid), dim3(HT), lds, st>>>((const IO*)x, (IO*)y, rows, n, K, log2m, hadK, scale, clip,
                                                       (u32*)q, (f16*)scales, hs_stride);
@@ -973,6 +979,8 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == QR_DTYPE_F16 && K == 1 && pow2_split(n))
+        return launch_hadamard_mm<true, false>(x, y, rows, n, pow2_split(n), nullptr, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && bm_applies(n, K))
         return launch_hadamard_bm<false>(x, y, rows, n, K, hadK, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && mm_applies(n, K))
@@ -997,6 +1005,8 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (K == 1 && pow2_split(n))
+        return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, pow2_split(n), nullptr, scale, clip, q, scales, st);
     if (mode == QR_DTYPE_F16 && bm_applies(n, K))
         return launch_hadamard_bm<true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     if (mm_applies(n, K)) {

@@ -38,6 +38,28 @@ static inline hipError_t qr_allow_dynamic_lds(const void* kernel, size_t bytes) 
     return e;
 }
 
+// Resident workgroups per CU for a kernel at a given block size and dynamic LDS size (cached; used
+// to size the grid of persistent kernels so that every workgroup is resident at once).
+static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) {
+    struct Entry {
+        const void* fn;
+        int dev, threads;
+        size_t lds;
+        int blocks;
+    };
+    static Entry table[64];
+    static int used = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 1;
+    for (int i = 0; i < used; ++i)
+        if (table[i].fn == kernel && table[i].dev == dev && table[i].threads == threads && table[i].lds == lds)
+            return table[i].blocks;
+    int blocks = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, threads, lds) != hipSuccess || blocks < 1) blocks = 1;
+    if (used < 64) table[used++] = Entry{kernel, dev, threads, lds, blocks};
+    return blocks;
+}
+
 static inline int qr_launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? QR_OK : (int)e;
