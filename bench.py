@@ -94,6 +94,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=64)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="instead of a workload, run a plain 256 MiB device copy 20 times (known traffic: 256 MiB read, "
+                         "256 MiB written per launch) for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path is data-parallel over tokens with no exchange; "
@@ -107,6 +110,14 @@ def main():
         build.build(verbose=False)
     _lib.lib()
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.randint(0, 255, (256 * 1024 * 1024,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": {"launches": 20, "read_bytes": src.numel(), "written_bytes": src.numel()}}))
+        return
     m, k, n, hadamard = WORKLOADS[args.workload]
     x_cpu = synth_x(m, k, seed=0, outliers=True)
     w_cpu, sw_cpu = synth_w(n, k, seed=1)

@@ -30,23 +30,55 @@ namespace {
 // reads in one ds_read_b128 beat fall in 16 different 16-byte bank groups.
 __device__ __forceinline__ int lds_slot(int row, int chunk) { return row * 4 + (chunk ^ ((row >> 2) & 3)); }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT, bool DEQ>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kernel(
+// Row-contiguous output of one wave's 32 x (32 NJ) fp16 slab.  In the accumulator layout a lane owns
+// 4 consecutive columns of one row, so a direct store instruction would write 16-byte pieces of 32
+// different rows and leave every 128-byte line to be assembled from eight partial writes in L2
+// (measured: 2.6x the output bytes written to memory on outputs larger than L2).  Instead the slab
+// goes through a wave-private LDS region and leaves as 16 bytes per lane with NJ*4 consecutive lanes
+// covering one row segment, i.e. whole lines per instruction.
+//   o[jj][gq] = this lane's columns jj*32 + gq*8 + (lane/32)*4 .. +3 of row lane%32.
+//   region: 32 * NJ * 8 slots of 8 bytes; the 8-byte slot index within a row is XORed with a key made
+//   from the row so that the 32 rows written by one instruction spread over all banks.
+template <int NJ>
+__device__ __forceinline__ void store_slab_rows(u32x2* region, const f16x4 (&o)[NJ][4], int lane, f16* ybase, int N) {
+    constexpr int U = NJ * 8;                   // 8-byte slots per row
+    constexpr int LPR = U / 2;                  // lanes (16 bytes each) per row on the way out
+    constexpr int RPP = 64 / LPR;               // rows per store instruction
+    const int r = lane & 31, khalf = lane >> 5;
+#pragma unroll
+    for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            const int u = jj * 8 + gq * 2 + khalf;
+            region[r * U + (u ^ ((r * U / 32) & (U - 1)))] = __builtin_bit_cast(u32x2, o[jj][gq]);
+        }
+    const u32x4* region16 = (const u32x4*)region;
+    const int s = lane % LPR;
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; ++pass) {
+        const int rr = lane / LPR + pass * RPP;
+        const int key = (rr * U / 32) & (U - 1);
+        u32x4 v = region16[rr * LPR + (s ^ (key >> 1))];
+        if (key & 1) v = u32x4{v[2], v[3], v[0], v[1]};
+        *(u32x4*)(ybase + (int64_t)rr * N + s * 8) = v;
+    }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
     int tiles_m, int tiles_n) {
-    constexpr int NT = 64 * WAVES_M * WAVES_N * KSPLIT;     // threads per workgroup
+    constexpr int NT = 64 * WAVES_M * WAVES_N;              // threads per workgroup
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;     // per-wave output tile
     constexpr int IM = TM / 32, JN = TN / 32;               // 32x32 MFMA tiles per wave
     constexpr int CH = (BM + BN) * 4;                       // 16-byte chunks per stage
     constexpr int NL = (CH + NT - 1) / NT;                  // chunks each thread moves per stage
     static_assert(TM % 32 == 0 && TN % 32 == 0, "tile shape");
-    static_assert(KSPLIT == 1 || (KSPLIT == 2 && JN % 2 == 0), "K split");
-    // stage buffers; with KSPLIT == 2 the same memory later carries the accumulator exchange
-    // (per round: every wave sends JN/2 tiles of 4 KB)
-    constexpr int XCH = KSPLIT == 2 ? WAVES_M * WAVES_N * 2 * (JN / 2) * 256 : 0;
-    constexpr int LDS_ELEMS = 2 * CH > XCH ? 2 * CH : XCH;
-    __shared__ u32x4 lds_raw[LDS_ELEMS];
+    // two stage buffers; the same memory later stages the fp16 output slabs (one per wave)
+    constexpr int SLAB = 32 * 64 * 2 / 16;                  // 16-byte units of a 32-row x 64-column fp16 slab
+    static_assert(2 * CH >= WAVES_M * WAVES_N * SLAB, "output slabs must fit in the stage buffers");
+    __shared__ u32x4 lds_raw[2 * CH];
     u32x4(*lds)[CH] = (u32x4(*)[CH])lds_raw;
 
     // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Give every XCD a
@@ -66,9 +98,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kg = wave / (WAVES_M * WAVES_N);              // K-group of this wave
-    const int wxy = wave % (WAVES_M * WAVES_N);
-    const int wm = wxy / WAVES_N, wn = wxy % WAVES_N;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     // Global -> LDS staging: chunk id = tid + i * NT; 4 consecutive threads fetch one row's 64 bytes.
     // Rows beyond M (or N) are clamped to the last valid row: they are read but never stored.
@@ -107,7 +137,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
     auto compute = [&](const u32x4* buf, int nsub) {
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            if (s < nsub && (KSPLIT == 1 || s == kg)) {
+            if (s < nsub) {
                 i32x4 alo[IM], ahi[IM], blo[JN], bhi[JN];
 #pragma unroll
                 for (int i = 0; i < IM; ++i) {
@@ -190,56 +220,44 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
         compute(lds[0], 1);
     }
 
-    // K-split: the two K-groups hold partial sums of the same wave tile.  Group 0 finalises the
-    // lower half of the j tiles and group 1 the upper half; each sends the other half across, one
-    // row of MFMA tiles (i) per round.  A tile travels as four 16-byte pieces per lane, lane-contiguous.
-    constexpr int JH = KSPLIT == 2 ? JN / 2 : JN;
-    const int j_first = KSPLIT == 2 ? kg * JH : 0;
-    if constexpr (KSPLIT == 2) {
-        u32x4* xbuf = lds_raw;
-        const int send0 = (1 - kg) * JH;            // first j tile this wave gives away
-        for (int i = 0; i < IM; ++i) {
-            __syncthreads();                        // stage buffers / previous round no longer read
-#pragma unroll
-            for (int jj = 0; jj < JH; ++jj)
-#pragma unroll
-                for (int qv = 0; qv < 4; ++qv) {
-                    // slot owned by the RECEIVER (wxy, 1 - kg)
-                    const int slot = (((wxy * 2 + (1 - kg)) * JH + jj) * 4 + qv) * 64 + lane;
-                    i32x4 piece;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        int val = 0;
-#pragma unroll
-                        for (int ii = 0; ii < IM; ++ii)
-#pragma unroll
-                            for (int jx = 0; jx < JN; ++jx)
-                                if (ii == i && jx == send0 + jj) val = acc[ii][jx][qv * 4 + e];
-                        piece[e] = val;
-                    }
-                    xbuf[slot] = (u32x4)piece;
-                }
-            __syncthreads();
-#pragma unroll
-            for (int jj = 0; jj < JH; ++jj)
-#pragma unroll
-                for (int qv = 0; qv < 4; ++qv) {
-                    const int slot = (((wxy * 2 + kg) * JH + jj) * 4 + qv) * 64 + lane;
-                    const i32x4 piece = (i32x4)xbuf[slot];
-#pragma unroll
-                    for (int ii = 0; ii < IM; ++ii)
-#pragma unroll
-                        for (int jx = 0; jx < JN; ++jx)
-                            if (ii == i && jx == j_first + jj) {
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) acc[ii][jx][qv * 4 + e] += piece[e];
-                            }
-                }
-        }
-    }
-
     // Epilogue.  Accumulator layout (first operand = W rows, second = X rows): lane l, register v ->
     // n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    // Whole tiles of an fp16 output leave as full rows through LDS, 64 columns (one line) at a time.
+    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    if (DEQ && by_rows) {
+        constexpr int NJ = JN > 2 ? 2 : JN;                 // MFMA tiles per slab
+        __syncthreads();                                    // every wave is done with the stage buffers
+#pragma unroll
+        for (int jb = 0; jb < JN; jb += NJ) {
+            f16x4 sbh[NJ][4], bih[NJ][4];
+#pragma unroll
+            for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
+                    sbh[jj][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                }
+#pragma unroll
+            for (int i = 0; i < IM; ++i) {
+                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                f16x4 o[NJ][4];
+#pragma unroll
+                for (int jj = 0; jj < NJ; ++jj)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
+                            if (bias) yv = yv + bih[jj][gq][e];
+                            o[jj][gq][e] = yv;
+                        }
+                store_slab_rows<NJ>((u32x2*)(lds_raw + wave * SLAB), o, lane,
+                                    Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+            }
+        }
+        return;
+    }
     // column scales (and bias) of this lane's 4-column groups, fetched up front as 8-byte vectors
     f16x4 sb4[JN][4], bi4[JN][4];
     if (DEQ) {
@@ -269,7 +287,6 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N * KSPLIT) void gemm_i4_kerne
         if (DEQ) sa = sA[row];
 #pragma unroll
         for (int j = 0; j < JN; ++j) {
-            if (j < j_first || j >= j_first + JH) continue;     // the other K-group stores this tile
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
                 const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
@@ -551,9 +568,31 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
                 }
             }
     }
+    // whole tiles of an fp16 output leave as full rows through LDS (each K-group its 64 columns)
+    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    if (DEQ && by_rows) __syncthreads();                    // the exchange buffers are no longer read
 #pragma unroll
     for (int i = 0; i < IM; ++i) {
         const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (DEQ && by_rows) {
+            const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+            f16x4 o[JH][4];
+#pragma unroll
+            for (int j = 0; j < JN; ++j) {
+                if (j < j_first || j >= j_first + JH) continue;
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        f16 yv = (f16)(sa * sb4[j % JH][gq][e]) * (f16)(float)(acc[i][j][gq * 4 + e] >> 8);
+                        if (bias) yv = yv + bi4[j % JH][gq][e];
+                        o[j % JH][gq][e] = yv;
+                    }
+            }
+            store_slab_rows<JH>((u32x2*)(ks_lds + wave * (32 * JH * 32 * 2 / 16)), o, lane,
+                                Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + j_first * 32, N);
+            continue;
+        }
         if (row >= M) continue;
         f16 sa = (f16)0;
         if (DEQ) sa = sA[row];
@@ -926,20 +965,20 @@ int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, v
     return qr_launch_status();
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int KSPLIT>
+template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st) {
-    constexpr int NT = 64 * WAVES_M * WAVES_N * KSPLIT;
+    constexpr int NT = 64 * WAVES_M * WAVES_N;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     if (Y)
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, KSPLIT, true><<<dim3(grid), dim3(NT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, (const f16*)sA, (const f16*)sB,
             (const f16*)bias, tiles_m, tiles_n);
     else
-        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, KSPLIT, false><<<dim3(grid), dim3(NT), 0, st>>>(
+        gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr, nullptr, nullptr, nullptr, tiles_m,
             tiles_n);
     return qr_launch_status();
@@ -960,15 +999,15 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
         // once per tile); otherwise eight waves split K over 32 rows
         if ((N + 255) / 256 >= 128) {
-            if (M <= 32) return launch_cfg<32, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-            return launch_cfg<64, 256, 1, 4, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+            if (M <= 32) return launch_cfg<32, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+            return launch_cfg<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         }
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
-    if (t256 >= 512) return launch_cfg<256, 256, 4, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
     if (t128x256 >= 128) return launch_ks<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-    return launch_cfg<128, 128, 2, 2, 1>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
 
 }  // namespace
