@@ -84,6 +84,7 @@ int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, int64_t col
  * and quantised from there, without the fp16 tensor making a round trip through HBM.
  *   x fp16 [rows, n]; mode QR_DTYPE_F16 (fp16 staging) or QR_DTYPE_F32 (OnlineHadamard force_fp32:
  *   hadK is then fp32 [K,K]); y_or_null: optional fp16 [rows, n] copy of the transformed rows.
+ *   x and y 16-byte aligned, q 8-byte aligned.
  */
 int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, int K, const void* hadK,
                                 int mode, float scale, float clip, void* q, void* scales,

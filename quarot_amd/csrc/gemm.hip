@@ -706,8 +706,8 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
         const int sc = sidx < steps ? sidx : steps - 1;
         const bool dead = half_tail && sc == steps - 1 && h == 1;
         const int off = sc * 64 - (dead ? 32 : 0);
-        st.w[0] = __builtin_nontemporal_load((const u32x4*)(wp + off));
-        st.w[1] = __builtin_nontemporal_load((const u32x4*)(wp + off + 16));
+        st.w[0] = *(const u32x4*)(wp + off);
+        st.w[1] = *(const u32x4*)(wp + off + 16);
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             st.x[t][0] = *(const u32x4*)(xp[t] + off);

@@ -54,7 +54,7 @@ __device__ __forceinline__ void reg_fwht8(float (&v)[8]) {
 }
 
 __device__ __forceinline__ void load8(const f16* p, float (&v)[8]) {
-    u32x4 raw = __builtin_nontemporal_load((const u32x4*)p);
+    u32x4 raw = *((const u32x4*)p);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         v[2 * i] = (float)f16_from_bits((unsigned short)(raw[i] & 0xffffu));
@@ -62,8 +62,8 @@ __device__ __forceinline__ void load8(const f16* p, float (&v)[8]) {
     }
 }
 __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
-    f32x4 a = __builtin_nontemporal_load((const f32x4*)p);
-    f32x4 b = __builtin_nontemporal_load((const f32x4*)p + 1);
+    f32x4 a = *((const f32x4*)p);
+    f32x4 b = *((const f32x4*)p + 1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         v[i] = a[i];
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(HT) void hadamard_km_kernel(const f16* __restrict__
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c = tid + i * HT;
-            raw[i] = c < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + row * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
+            raw[i] = c < nchunks ? *((const u32x4*)(x + row * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
         }
     }
     __syncthreads();
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(HT) void hadamard_km_kernel(const f16* __restrict__
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
                 const int c = tid + i * HT;
-                raw[i] = c < nchunks ? __builtin_nontemporal_load((const u32x4*)(x + nrow * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
+                raw[i] = c < nchunks ? *((const u32x4*)(x + nrow * (int64_t)n) + c) : u32x4{0, 0, 0, 0};
             }
         }
         __syncthreads();
@@ -491,7 +491,7 @@ bool km_applies(int n, int K, bool mode32) {
 //                                    a lane ends with 4 consecutive r of one output k: 8-byte writes
 //                                    into the fp16 result row in LDS.
 //   stage 3   result row -> global, with the quantiser when fused.
-template <bool MODE32, bool QUANT, int LOG2M, int KS2>
+template <bool MODE32, bool QUANT, int LOG2M, int KS2, bool XLDS>
 __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
                                                          int n, int K, const void* __restrict__ hadK, float scale,
                                                          float clip, u32* __restrict__ q, f16* __restrict__ scales) {
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
     constexpr bool FULL_ROW = (M_ == 64);
     constexpr int SLOTS = FULL_ROW ? KS2 : 2;
     extern __shared__ f32x4 smem_raw[];
-    __shared__ u32 red[HT / QR_WAVE];
+    __shared__ u32 red[2 * (HT / QR_WAVE)];       // per-wave row maxima, double-buffered by row parity
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int nchunks = n >> 3;
@@ -514,6 +514,35 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
     u32x4* Tl = (u32x4*)smem_raw;                              // [CT][KS2][64 lanes] fragments of T (hi plane)
     u32x4* Tlo = Tl + CT * KS2 * 64;                           // lo plane (fp32 mode)
     f16* Yl = (f16*)(Tl + (MODE32 ? 2 : 1) * CT * KS2 * 64);   // [K][YS]
+    // XLDS: the input row is fetched with fully coalesced 16-byte loads (consecutive lanes,
+    // consecutive addresses), one row ahead in registers, and staged in LDS, from where the stage-1
+    // fragments are read; fragment loads straight from global memory touch sixteen different lines
+    // per instruction and were measured to bound the kernel.  Xl: [32 KS2 rows][PPR 16-byte pieces],
+    // piece index XOR-keyed by the row so that the sixteen rows of a fragment read spread over all
+    // bank groups; rows K.. are zero.
+    constexpr int PPR = M_ / 8;
+    constexpr int NCH = KS2 * M_ / 64;          // 16-byte chunks per thread: n / 8 <= 32 KS2 M_ / 8
+    u32x4* Xl = (u32x4*)(Yl + ((K * YS + 7) & ~7));
+    auto xslot = [](int row, int piece) { return row * PPR + (piece ^ ((PPR == 8 ? row >> 1 : row) & (PPR - 1))); };
+    u32x4 xr[XLDS ? NCH : 1];
+    auto load_row = [&](const f16* src) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            int c = tid + i * HT;
+            c = c < nchunks ? c : nchunks - 1;
+            xr[i] = *((const u32x4*)src + c);
+        }
+    };
+    auto deposit_row = [&]() {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * HT;
+            if (c < nchunks) Xl[xslot(c / PPR, c % PPR)] = xr[i];
+        }
+    };
+    if (XLDS) {
+        for (int i = K * PPR + tid; i < KS2 * 32 * PPR; i += HT) Xl[i] = u32x4{0, 0, 0, 0};
+    }
 
     // hadK fragments, contraction index in the stage-1 accumulator order: for each (step, half) a
     // lane needs 4 consecutive k -- one 8-byte (fp16) or 16-byte (fp32) load (every order is a
@@ -564,7 +593,7 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
             const int k = (2 * s2 + h) * 16 + l16;
 #pragma unroll
             for (int ks = 0; ks < KS1; ++ks)
-                dst[h][ks] = k < K ? __builtin_nontemporal_load((const u32x4*)(xr + k * M_ + ks * 32 + g * 8)) : u32x4{0, 0, 0, 0};
+                dst[h][ks] = k < K ? *((const u32x4*)(xr + k * M_ + ks * 32 + g * 8)) : u32x4{0, 0, 0, 0};
         }
     };
     // one tile pair through stage 1: T fragments for this wave's column tile(s) -> LDS
@@ -597,10 +626,20 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
         }
     };
 
-    u32x4 fr[SLOTS][2][KS1];
+    auto lds_pair = [&](int s2, u32x4(&dst)[2][KS1]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int ks = 0; ks < KS1; ++ks) dst[h][ks] = Xl[xslot((2 * s2 + h) * 16 + l16, ks * 4 + g)];
+    };
+
+    u32x4 fr[XLDS ? 1 : SLOTS][2][KS1];
+    int row_parity = 0;
     int64_t row = blockIdx.x;
     if (row < rows) {
-        if (FULL_ROW) {
+        if (XLDS) {
+            load_row(x + row * (int64_t)n);
+        } else if (FULL_ROW) {
 #pragma unroll
             for (int s2 = 0; s2 < KS2; ++s2) load_pair(x + row * (int64_t)n, s2, fr[s2 % SLOTS]);
         } else {
@@ -611,9 +650,17 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
         const f16* xr = x + row * (int64_t)n;
         const int64_t nrow = row + gridDim.x;
         // ---- stage 1
+        if (XLDS) {
+            deposit_row();
+            if (nrow < rows) load_row(x + nrow * (int64_t)n);
+            __syncthreads();
+        }
 #pragma unroll
         for (int s2 = 0; s2 < KS2; ++s2) {
-            if (FULL_ROW) {
+            if (XLDS) {
+                lds_pair(s2, fr[0]);
+                stage1(s2, fr[0]);
+            } else if (FULL_ROW) {
                 stage1(s2, fr[s2 % SLOTS]);
                 if (nrow < rows) load_pair(x + nrow * (int64_t)n, s2, fr[s2 % SLOTS]);
             } else {
@@ -624,14 +671,15 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
                 stage1(s2, fr[s2 % SLOTS]);
             }
         }
-        if (!FULL_ROW && (KS2 % 2) == 1) {
+        if (!XLDS && !FULL_ROW && (KS2 % 2) == 1) {
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
                 for (int ks = 0; ks < KS1; ++ks) fr[0][h][ks] = fr[1][h][ks];
         }
         __syncthreads();
-        // ---- stage 2
+        // ---- stage 2 (when fused, the row's abs-max is taken from the rounded results on the way)
+        u16x2 mx2 = {0, 0};
         for (int ct = 0; ct < CT; ++ct) {
             f16x8 th[KS2], tl[KS2];
 #pragma unroll
@@ -655,41 +703,54 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
                         o[0] = (u32)f16_bits((f16)acc[0]) | ((u32)f16_bits((f16)acc[1]) << 16);
                         o[1] = (u32)f16_bits((f16)acc[2]) | ((u32)f16_bits((f16)acc[3]) << 16);
                         *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
+                        if (QUANT) {
+                            mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & 0x7fff7fffu));
+                            mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[1] & 0x7fff7fffu));
+                        }
                     }
                 }
             }
         }
+        u32 mx = 0;
+        if (QUANT) {
+            mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            mx = wave_max_u32(mx);
+            if (lane == 0) red[(row_parity << 2) + wave] = mx;
+        }
         __syncthreads();
         // ---- stage 3
         if (QUANT) {
-            u32 mx = 0;
-            for (int c = tid; c < nchunks; c += HT) {
-                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
-                const u32 mc = absmax_bits8(h);
-                mx = mx > mc ? mx : mc;
-            }
-            mx = wave_max_u32(mx);
-            if (lane == 0) red[wave] = mx;
-            __syncthreads();
 #pragma unroll
-            for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+            for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[(row_parity << 2) + w] ? mx : red[(row_parity << 2) + w];
+            row_parity ^= 1;
             const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
             if (tid == 0) scales[row] = sh;
             const float s = (float)sh;
+            // two chunks (16 elements) per thread and step: 8-byte stores of codes
+            const int nunits = nchunks >> 1;
+            u32x2* qrow = (u32x2*)(q + row * (int64_t)nchunks);
             if (fast_quant_ok(mx, s)) {
                 const FastRecip fq = make_fast_recip(s);
-                for (int c = tid; c < nchunks; c += HT) {
-                    const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
-                    q[row * (int64_t)nchunks + c] = sym_codes8_fast(h, fq);
-                    if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+                for (int u = tid; u < nunits; u += HT) {
+                    const f16* src = Yl + ((u * 16) >> LOG2M) * YS + ((u * 16) & (M_ - 1));
+                    const u32x4 h0 = *(const u32x4*)src, h1 = *(const u32x4*)(src + 8);
+                    qrow[u] = u32x2{sym_codes8_fast(h0, fq), sym_codes8_fast(h1, fq)};
+                    if (y) {
+                        __builtin_nontemporal_store(h0, (u32x4*)(y + row * (int64_t)n) + 2 * u);
+                        __builtin_nontemporal_store(h1, (u32x4*)(y + row * (int64_t)n) + 2 * u + 1);
+                    }
                 }
             } else {
                 const bool fast = scale_fast_ok(s);
                 const float rs = fast ? 1.0f / s : 0.0f;
-                for (int c = tid; c < nchunks; c += HT) {
-                    const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
-                    q[row * (int64_t)nchunks + c] = sym_codes8(h, s, rs, fast);
-                    if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+                for (int u = tid; u < nunits; u += HT) {
+                    const f16* src = Yl + ((u * 16) >> LOG2M) * YS + ((u * 16) & (M_ - 1));
+                    const u32x4 h0 = *(const u32x4*)src, h1 = *(const u32x4*)(src + 8);
+                    qrow[u] = u32x2{sym_codes8(h0, s, rs, fast), sym_codes8(h1, s, rs, fast)};
+                    if (y) {
+                        __builtin_nontemporal_store(h0, (u32x4*)(y + row * (int64_t)n) + 2 * u);
+                        __builtin_nontemporal_store(h1, (u32x4*)(y + row * (int64_t)n) + 2 * u + 1);
+                    }
                 }
             }
         } else {
@@ -720,12 +781,16 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
                        void* q, void* scales, hipStream_t st) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
-    const size_t lds = (size_t)(MODE32 ? 2 : 1) * (m / 16) * KS2 * 64 * 16 + (size_t)K * (m + 8) * 2;
-#define QR_MM(L2M, KS)                                                                                                 \
+    const size_t lds0 = (size_t)(MODE32 ? 2 : 1) * (m / 16) * KS2 * 64 * 16 + (((size_t)K * (m + 8) + 7) & ~(size_t)7) * 2;
+    const size_t lds_x = lds0 + (size_t)KS2 * 32 * m * 2;
+    // the staged-input form when at least two workgroups still fit on a CU
+    const bool xlds = lds_x <= 78 * 1024;
+    const size_t lds = xlds ? lds_x : lds0;
+#define QR_MM(L2M, KS, XL)                                                                                             \
     do {                                                                                                               \
-        auto kern = hadamard_mm_kernel<MODE32, QUANT, L2M, KS>;                                                        \
+        auto kern = hadamard_mm_kernel<MODE32, QUANT, L2M, KS, XL>;                                                    \
         if (lds > 48 * 1024) {                                                                                         \
-            hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
+            hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);                                               \
             if (e != hipSuccess) return (int)e;                                                                        \
         }                                                                                                              \
         const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);                                      \
@@ -733,18 +798,22 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
                                                 (f16*)scales);                                                         \
     } while (0)
-#define QR_MM_K(L2M)                     \
-    switch (KS2) {                       \
-        case 1: QR_MM(L2M, 1); break;    \
-        case 2: QR_MM(L2M, 2); break;    \
-        case 3: QR_MM(L2M, 3); break;    \
-        case 4: QR_MM(L2M, 4); break;    \
-        case 5: QR_MM(L2M, 5); break;    \
-        default: QR_MM(L2M, 6); break;   \
+#define QR_MM_X(L2M, KS)                 \
+    if (xlds) QR_MM(L2M, KS, true);      \
+    else QR_MM(L2M, KS, false)
+#define QR_MM_K(L2M)                       \
+    switch (KS2) {                         \
+        case 1: QR_MM_X(L2M, 1); break;    \
+        case 2: QR_MM_X(L2M, 2); break;    \
+        case 3: QR_MM_X(L2M, 3); break;    \
+        case 4: QR_MM_X(L2M, 4); break;    \
+        case 5: QR_MM_X(L2M, 5); break;    \
+        default: QR_MM_X(L2M, 6); break;   \
     }
     if (m == 64) { QR_MM_K(6) }
     else { QR_MM_K(7) }
 #undef QR_MM_K
+#undef QR_MM_X
 #undef QR_MM
     return qr_launch_status();
 }
@@ -800,7 +869,7 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
             const int k = wave + NW * sg;
 #pragma unroll
             for (int i = 0; i < CPL; ++i)
-                raw[sg][i] = k < K ? __builtin_nontemporal_load((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
+                raw[sg][i] = k < K ? *((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
                                    : u32x4{0, 0, 0, 0};
         }
     };
@@ -1002,7 +1071,7 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (rc != QR_OK) return rc;
     if (rows == 0) return QR_OK;
     if (!x || !q || !scales || (K > 1 && !hadK)) return QR_E_NULL;
-    if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
+    if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 7)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
     if (K == 1 && pow2_split(n))

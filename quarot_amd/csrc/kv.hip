@@ -46,7 +46,7 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
     for (int64_t c0 = (int64_t)blockIdx.x * KT; c0 < nchunks; c0 += stride) {
         const int64_t c = c0 + threadIdx.x;
         const bool live = c < nchunks;                   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
-        u32x4 raw = live ? __builtin_nontemporal_load(x + c) : u32x4{0, 0, 0, 0};
+        u32x4 raw = live ? *(x + c) : u32x4{0, 0, 0, 0};
         float v[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(KT) void kv_dequant_kernel(const u32* __restrict__ 
                                                         u32x4* __restrict__ y) {
     const int64_t stride = (int64_t)gridDim.x * KT;
     for (int64_t c = (int64_t)blockIdx.x * KT + threadIdx.x; c < nchunks; c += stride) {
-        const u32 w = __builtin_nontemporal_load(q + c);
+        const u32 w = *(q + c);
         const f16 sc = scale[c >> LG], zp = zero[c >> LG];
         u32x4 o;
 #pragma unroll

@@ -6,6 +6,7 @@
 
 typedef _Float16 f16;
 typedef f16 f16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 typedef f16 f16x4 __attribute__((ext_vector_type(4)));
 typedef f16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -102,11 +103,13 @@ __device__ __forceinline__ u32 wave_max_u32(u32 v) {
     return v;
 }
 
-// Quantiser scale: fp16( float(fp16(amax / 7)) * clip ), each step correctly rounded.  The fp32
-// quotient of an fp16 by 7 rounds to fp16 like the exact quotient does (24 >= 2*11 + 2); it is
-// formed in double so no fast-division lowering can touch it.
+// Quantiser scale: fp16( float(fp16(amax / 7)) * clip ), each step correctly rounded.  amax / 7
+// never lies on (or within 2^-14 relative of) an fp16 rounding boundary: a boundary (i + 1/2) ulp
+// would need amax = 7 i + 3.5 units of its own grid.  So the fp32 product with the rounded
+// constant 1/7 (relative error < 2^-23) rounds to the same fp16 as the exact quotient (checked for
+// every finite fp16 amax).
 __device__ __forceinline__ f16 quantizer_scale(f16 amax, float clip) {
-    f16 s = (f16)(float)((double)(float)amax / 7.0);
+    const f16 s = narrow_f16((float)amax * (1.0f / 7.0f));
     return narrow_f16((float)s * clip);
 }
 
@@ -161,11 +164,15 @@ __device__ __forceinline__ u32 sym_codes8(u32x4 v, float s, float rs, bool fast_
 struct FastRecip {
     float rh, rl;
 };
+// s: a finite non-zero fp16 value as float.  v_rcp_f32 + one Newton step give r1 ~ 1/s; rh = r1
+// cut to 13 bits makes s * rh exact (11 + 13 bits), so e2 = 1 - s rh is exact and rl = e2 r1
+// completes 1/s to a relative 2^-35.
 __device__ __forceinline__ FastRecip make_fast_recip(float s) {
-    const double r = 1.0 / (double)s;
+    const float r0 = __builtin_amdgcn_rcpf(s);
+    const float r1 = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
     FastRecip f;
-    f.rh = __builtin_bit_cast(float, __builtin_bit_cast(u32, (float)r) & 0xFFFFF800u);
-    f.rl = (float)(r - (double)f.rh);
+    f.rh = __builtin_bit_cast(float, __builtin_bit_cast(u32, r1) & 0xFFFFF800u);
+    f.rl = __builtin_fmaf(-s, f.rh, 1.0f) * r1;
     return f;
 }
 __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
