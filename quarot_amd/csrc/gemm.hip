@@ -994,14 +994,11 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M <= 8) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 4 || (M <= 8 && (N + 255) / 256 < 128)) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     if (M <= 64) {
         // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
         // once per tile); otherwise eight waves split K over 32 rows
-        if ((N + 255) / 256 >= 128) {
-            if (M <= 32) return launch_cfg<32, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-            return launch_cfg<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-        }
+        if ((N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
