@@ -33,11 +33,11 @@ __device__ __forceinline__ float lane_xor(float v) {
 
 template <int MASK>
 __device__ __forceinline__ void lane_stage(float (&v)[8], int lane) {
-    const bool upper = (lane & MASK) != 0;
+    const float sgn = (lane & MASK) != 0 ? -1.0f : 1.0f;     // upper lane of a pair: partner - own
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float p = lane_xor<MASK>(v[e]);
-        v[e] = upper ? p - v[e] : v[e] + p;
+        v[e] = __builtin_fmaf(v[e], sgn, p);
     }
 }
 
@@ -76,7 +76,7 @@ __device__ __forceinline__ u32x4 to_f16x8(const float (&v)[8]) {
     u32x4 o;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-        o[i] = (u32)f16_bits(narrow_f16(v[2 * i])) | ((u32)f16_bits(narrow_f16(v[2 * i + 1])) << 16);
+        o[i] = narrow_f16x2(v[2 * i], v[2 * i + 1]);
     return o;
 }
 

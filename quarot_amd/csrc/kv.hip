@@ -21,11 +21,11 @@ __device__ __forceinline__ float kv_lane_xor(float v) {
 
 template <int MASK>
 __device__ __forceinline__ void kv_butterfly(float (&v)[8], int lane) {
-    const bool upper = (lane & MASK) != 0;
+    const float sgn = (lane & MASK) != 0 ? -1.0f : 1.0f;     // upper lane of a pair: partner - own
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         float p = kv_lane_xor<MASK>(v[e]);
-        v[e] = upper ? p - v[e] : v[e] + p;
+        v[e] = __builtin_fmaf(v[e], sgn, p);
     }
 }
 
@@ -34,6 +34,43 @@ __device__ __forceinline__ void kv_minmax(float& mn, float& mx) {
     float a = kv_lane_xor<MASK>(mn), b = kv_lane_xor<MASK>(mx);
     mn = a < mn ? a : mn;
     mx = b > mx ? b : mx;
+}
+
+// (min, -max) of a vector as one packed pair, reduced across the vector's lanes with one packed min
+template <int MASK>
+__device__ __forceinline__ f16x2 kv_pair_min(f16x2 p) {
+    int i = __builtin_bit_cast(int, p);
+    int r;
+    if constexpr (MASK == 1) r = __builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true);
+    else if constexpr (MASK == 2) r = __builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true);
+    else if constexpr (MASK == 4) r = __builtin_amdgcn_ds_swizzle(i, 0x101F);
+    else if constexpr (MASK == 8) r = __builtin_amdgcn_mov_dpp(i, 0x128, 0xF, 0xF, true);
+    else r = __builtin_amdgcn_ds_swizzle(i, 0x401F);
+    return __builtin_elementwise_min(p, __builtin_bit_cast(f16x2, r));
+}
+
+// Eight codes clamp(round_half_even(fp16(fp16(x + zero) / scale)), 0, 15) for all-finite input: the
+// add is one packed fp16 add, the division the exact-product / fma form of sym_codes8_fast (the
+// shifted value has at most 11 significant bits), the rounding the +1536 trick.
+__device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) {
+    const f16x2 z2 = {zero, zero};
+    u32 b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const f16x2 sh = as_f16x2(v[i]) + z2;
+        const float x0 = (float)sh[0], x1 = (float)sh[1];
+        float q0 = __builtin_fmaf(x0, f.rl, x0 * f.rh);
+        float q1 = __builtin_fmaf(x1, f.rl, x1 * f.rh);
+        q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
+        q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);
+        f16x2 h = {(f16)q0, (f16)q1};
+        h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
+        const u32 w = __builtin_bit_cast(u32, h);
+        b[i] = (w & 0xFu) | ((w >> 12) & ~0xFu);    // low byte: code0 | code1 << 4
+    }
+    const u32 t01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
+    const u32 t23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
+    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
 }
 
 // LG = log2(lanes per vector) = log2(dim) - 3, 1..5
@@ -46,14 +83,14 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
     for (int64_t c0 = (int64_t)blockIdx.x * KT; c0 < nchunks; c0 += stride) {
         const int64_t c = c0 + threadIdx.x;
         const bool live = c < nchunks;                   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
-        u32x4 raw = live ? *(x + c) : u32x4{0, 0, 0, 0};
-        float v[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            v[2 * i] = (float)f16_from_bits((unsigned short)(raw[i] & 0xffffu));
-            v[2 * i + 1] = (float)f16_from_bits((unsigned short)(raw[i] >> 16));
-        }
+        u32x4 hp = live ? *(x + c) : u32x4{0, 0, 0, 0};  // the 8 fp16 values to quantise, packed
         if (HAD) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = (float)f16_from_bits((unsigned short)(hp[i] & 0xffffu));
+                v[2 * i + 1] = (float)f16_from_bits((unsigned short)(hp[i] >> 16));
+            }
 #pragma unroll
             for (int h = 1; h < 8; h <<= 1)
 #pragma unroll
@@ -69,42 +106,79 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
             if (LG > 3) kv_butterfly<8>(v, lane);
             if (LG > 4) kv_butterfly<16>(v, lane);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (float)narrow_f16(v[e] * hscale);   // the transform's fp16 output
+            for (int i = 0; i < 4; ++i)                  // the transform's fp16 output
+                hp[i] = narrow_f16x2(v[2 * i] * hscale, v[2 * i + 1] * hscale);
         }
-        float mn = v[0], mx = v[0];
+        u32 outw;
+        f16 sc, zp;
+        const u32 amax = absmax_bits8(hp);
+        if (__builtin_amdgcn_ballot_w64(amax >= 0x7c00u) == 0) {
+            // every value in the wave is finite: packed min / max, then the lean code path
+            f16x2 mn2 = as_f16x2(hp[0]), mx2 = mn2;
 #pragma unroll
-        for (int e = 1; e < 8; ++e) {
-            mn = v[e] < mn ? v[e] : mn;
-            mx = v[e] > mx ? v[e] : mx;
-        }
-        if (LG > 0) kv_minmax<1>(mn, mx);
-        if (LG > 1) kv_minmax<2>(mn, mx);
-        if (LG > 2) kv_minmax<4>(mn, mx);
-        if (LG > 3) kv_minmax<8>(mn, mx);
-        if (LG > 4) kv_minmax<16>(mn, mx);
-        // scale = max(fp16(max - min), fp16(1e-5)) / 15 ; zero = -min   (each step one fp16 rounding)
-        f16 rng = (f16)(mx - mn);
-        const f16 floor_ = (f16)1e-5f;
-        rng = rng < floor_ ? floor_ : rng;
-        const f16 sc = (f16)(float)((double)(float)rng / 15.0);
-        const f16 zp = (f16)(-mn);
-        const float s = (float)sc, z = (float)zp;
-        const float rs = 1.0f / s;                       // s >= fp16(1e-5)/15 > 0, finite
-        u32 out = 0;
+            for (int i = 1; i < 4; ++i) {
+                mn2 = __builtin_elementwise_min(mn2, as_f16x2(hp[i]));
+                mx2 = __builtin_elementwise_max(mx2, as_f16x2(hp[i]));
+            }
+            const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+            const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            f16x2 pr = {mn0, -mx0};
+            if (LG > 0) pr = kv_pair_min<1>(pr);
+            if (LG > 1) pr = kv_pair_min<2>(pr);
+            if (LG > 2) pr = kv_pair_min<4>(pr);
+            if (LG > 3) pr = kv_pair_min<8>(pr);
+            if (LG > 4) pr = kv_pair_min<16>(pr);
+            const f16 mn = pr[0], mx = -pr[1];
+            // scale = max(fp16(max - min), fp16(1e-5)) / 15 ; zero = -min   (each step one fp16 rounding).
+            // range / 15 is never within 2^-16 (relative) of an fp16 rounding boundary, so the fp32
+            // product with the rounded constant rounds like the exact quotient (checked for every fp16).
+            f16 rng = narrow_f16((float)mx - (float)mn);
+            const f16 floor_ = (f16)1e-5f;
+            rng = rng < floor_ ? floor_ : rng;
+            sc = narrow_f16((float)rng * (1.0f / 15.0f));
+            zp = -mn;
+            outw = asym_codes8_fast(hp, zp, make_fast_recip((float)sc));
+        } else {
+            float v[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float sh = (float)(f16)(v[e] + z);
-            const float q0 = sh * rs;
-            const float er = __builtin_fmaf(-q0, s, sh);
-            const float q1 = __builtin_fabsf(q0) < __builtin_inff() ? __builtin_fmaf(er, rs, q0) : q0;
-            const float r = __builtin_rintf((float)(f16)q1);
-            int code = (int)r;
-            code = code < 0 ? 0 : (code > 15 ? 15 : code);
-            code = (r != r) ? 0 : code;
-            out |= (u32)code << (4 * e);
+            for (int i = 0; i < 4; ++i) {
+                v[2 * i] = (float)f16_from_bits((unsigned short)(hp[i] & 0xffffu));
+                v[2 * i + 1] = (float)f16_from_bits((unsigned short)(hp[i] >> 16));
+            }
+            float mn = v[0], mx = v[0];
+#pragma unroll
+            for (int e = 1; e < 8; ++e) {
+                mn = v[e] < mn ? v[e] : mn;
+                mx = v[e] > mx ? v[e] : mx;
+            }
+            if (LG > 0) kv_minmax<1>(mn, mx);
+            if (LG > 1) kv_minmax<2>(mn, mx);
+            if (LG > 2) kv_minmax<4>(mn, mx);
+            if (LG > 3) kv_minmax<8>(mn, mx);
+            if (LG > 4) kv_minmax<16>(mn, mx);
+            f16 rng = (f16)(mx - mn);
+            const f16 floor_ = (f16)1e-5f;
+            rng = rng < floor_ ? floor_ : rng;
+            sc = (f16)(float)((double)(float)rng / 15.0);
+            zp = (f16)(-mn);
+            const float s = (float)sc, z = (float)zp;
+            const float rs = 1.0f / s;
+            outw = 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float sh = (float)(f16)(v[e] + z);
+                const float q0 = sh * rs;
+                const float er = __builtin_fmaf(-q0, s, sh);
+                const float q1 = __builtin_fabsf(q0) < __builtin_inff() ? __builtin_fmaf(er, rs, q0) : q0;
+                const float r = __builtin_rintf((float)(f16)q1);
+                int code = (int)r;
+                code = code < 0 ? 0 : (code > 15 ? 15 : code);
+                code = (r != r) ? 0 : code;
+                outw |= (u32)code << (4 * e);
+            }
         }
         if (live) {
-            q[c] = out;
+            q[c] = outw;
             if ((lane & ((1 << LG) - 1)) == 0) {
                 scale[c >> LG] = sc;
                 zero[c >> LG] = zp;

@@ -79,6 +79,22 @@ __device__ __forceinline__ f16 narrow_f16(float v) {
     return (f16)v;
 }
 
+// Two floats -> two fp16 (round to nearest even) packed in one word, `a` in the low half
+// (v_cvt_pk_f16_f32).  The empty asm keeps a producing multiply from being folded into a
+// single-rounding mixed-precision instruction, as in narrow_f16.
+__device__ __forceinline__ u32 narrow_f16x2(float a, float b) {
+    asm("" : "+v"(a), "+v"(b));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    const f16x2 h = __builtin_convertvector(v, f16x2);
+    return __builtin_bit_cast(u32, h);
+}
+
+// Reinterpret one 32-bit word as two halves.  Always go through this by-value helper: applying
+// __builtin_bit_cast directly to an element of an ext-vector (v[i]) was seen to read element 0
+// whatever the index.
+__device__ __forceinline__ f16x2 as_f16x2(u32 w) { return __builtin_bit_cast(f16x2, w); }
+
 // max over |x| for the 8 halves held in a uint4, as raw magnitudes (sign bit cleared).  Comparing
 // magnitudes as unsigned integers orders finite values and inf correctly and lets a NaN win, which
 // is how torch.max propagates it.
