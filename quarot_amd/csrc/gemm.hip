@@ -668,51 +668,67 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decode (M <= 64): the weights are streamed once from HBM and nothing is reused, so no LDS
-// staging.  A workgroup of eight waves owns 32 weight rows; the waves split K into eight contiguous
-// ranges, each wave loads its W fragments (16 bytes per lane, straight into registers) and the
-// matching X fragments (small, L2-resident), unpacks and multiplies; the eight partial 32 x M tiles
-// are summed through LDS and dequantised.  Loads run PF steps ahead in a register ring.
-template <int MT, bool DEQ>
+// Decode (M <= 64) with too few column tiles for the tiled kernels.  A workgroup of eight waves owns
+// 32 weight rows; the waves split K into eight contiguous ranges and the eight partial 32 x M tiles
+// are summed through LDS and dequantised.  Nothing is shared between waves in the main loop, so there
+// are no barriers in it: every wave streams its own slices of W and X with coalesced 16-byte loads
+// (SB / 16 lanes per row piece of SB bytes, PF steps ahead in a register ring) and turns them into
+// MFMA fragments (lane = row) through a wave-private LDS buffer.  Loading fragments straight from
+// global memory makes every instruction touch 32 different lines and was measured 1.5-2x slower.
+template <int MT, int SB, bool DEQ>
 __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
                                                         const f16* __restrict__ sB, const f16* __restrict__ bias) {
-    constexpr int PF = 4;                                   // steps in flight; a step = 64 packed bytes (128 k) per row
-    __shared__ i32x4 red[8 * MT * 4 * 64];                  // [wave][m tile][4-register group][lane]
+    constexpr int CPR = SB / 16;                            // 16-byte chunks per row and step (4, 8 or 16)
+    constexpr int PF = SB == 64 ? 4 : 3;                    // steps in flight
+    constexpr int ROWS = (1 + MT) * 32;                     // staged rows per wave: 32 of W, then 32 MT of X
+    constexpr int NLD = ROWS * CPR / 64;                    // chunks per lane and step
+    constexpr int STAGE = ROWS * CPR;                       // u32x4 per wave
+    constexpr int RED = MT * 4 * 64;                        // i32x4 per wave for the final sum
+    extern __shared__ u32x4 dec_smem[];                     // 8 * max(STAGE, RED)
+    i32x4* red = (i32x4*)dec_smem;                          // [wave][m tile][4-register group][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int n0 = blockIdx.x * 32;
-    const int steps = (Kb + 63) / 64;
+    const int steps = (Kb + SB - 1) / SB;
     const int s_begin = (int)((int64_t)steps * wave / 8), s_end = (int)((int64_t)steps * (wave + 1) / 8);
+    u32x4* stage = dec_smem + wave * STAGE;
+    // chunk position XOR-keyed by the row: the 16 rows of a fragment read spread over all bank groups
+    auto slot = [](int row, int chunk) {
+        return CPR == 4 ? row * 4 + (chunk ^ ((row >> 2) & 3))
+               : CPR == 8 ? row * 8 + (chunk ^ ((row >> 1) & 7)) : row * 16 + (chunk ^ (row & 15));
+    };
 
-    int nr = n0 + r;
-    nr = nr < N ? nr : N - 1;
-    const uint8_t* wp = B + (int64_t)nr * Kb + h * 32;
-    const uint8_t* xp[MT];
+    // chunk i of this lane: row (lane + 64 i) / CPR, 16-byte piece lane % CPR
+    const int piece = lane % CPR;
+    const uint8_t* src[NLD];
+    int dst[NLD];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        int mr = t * 32 + r;
-        mr = mr < M ? mr : M - 1;
-        xp[t] = A + (int64_t)mr * Kb + h * 32;
+    for (int i = 0; i < NLD; ++i) {
+        const int row = lane / CPR + (64 / CPR) * i;
+        if (row < 32) {
+            int nr = n0 + row;
+            nr = nr < N ? nr : N - 1;
+            src[i] = B + (int64_t)nr * Kb;
+        } else {
+            int mr = row - 32;
+            mr = mr < M ? mr : M - 1;
+            src[i] = A + (int64_t)mr * Kb;
+        }
+        dst[i] = slot(row, piece);
     }
-    // in a half-full last step (K % 128 == 64) the upper 32 bytes lie beyond the row: those lanes
-    // re-read the lower half and their fragments are zeroed
-    const bool half_tail = (Kb & 63) != 0;
+    // K % 64 == 0: a row is a whole number of 32-byte pairs of pieces.  Pieces of the last step that
+    // lie beyond the row re-read piece 0 or 1 of that step and are deposited as zeros.
     struct Step {
-        u32x4 w[2], x[MT][2];
+        u32x4 v[NLD];
     };
     auto fetch = [&](int sidx, Step& st) {
         const int sc = sidx < steps ? sidx : steps - 1;
-        const bool dead = half_tail && sc == steps - 1 && h == 1;
-        const int off = sc * 64 - (dead ? 32 : 0);
-        st.w[0] = *(const u32x4*)(wp + off);
-        st.w[1] = *(const u32x4*)(wp + off + 16);
+        const bool dead = sc * SB + piece * 16 >= Kb;
+        const int off = sc * SB + (dead ? (piece & 1) : piece) * 16;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            st.x[t][0] = *(const u32x4*)(xp[t] + off);
-            st.x[t][1] = *(const u32x4*)(xp[t] + off + 16);
-        }
+        for (int i = 0; i < NLD; ++i) st.v[i] = *(const u32x4*)(src[i] + off);
     };
     i32x16 acc[MT];
 #pragma unroll
@@ -720,14 +736,18 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t][v] = 0;
     auto consume = [&](int sidx, const Step& st) {
-        const bool dead = half_tail && sidx == steps - 1 && h == 1;
+        const bool dead = sidx * SB + piece * 16 >= Kb;
+        // LDS operations of one wave execute in order: these writes follow the previous step's reads
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const u32x4 wq = dead ? u32x4{0, 0, 0, 0} : st.w[c];
+        for (int i = 0; i < NLD; ++i) stage[dst[i]] = dead ? u32x4{0, 0, 0, 0} : st.v[i];
+#pragma unroll
+        for (int c = 0; c < CPR / 2; ++c) {                 // lane half h takes pieces 2c + h of both operands
+            const u32x4 wq = stage[slot(r, 2 * c + h)];
             const i32x4 wlo = (i32x4)((wq << 4) & 0xF0F0F0F0u), whi = (i32x4)(wq & 0xF0F0F0F0u);
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const i32x4 xlo = (i32x4)((st.x[t][c] << 4) & 0xF0F0F0F0u), xhi = (i32x4)(st.x[t][c] & 0xF0F0F0F0u);
+                const u32x4 xq = stage[slot(32 + t * 32 + r, 2 * c + h)];
+                const i32x4 xlo = (i32x4)((xq << 4) & 0xF0F0F0F0u), xhi = (i32x4)(xq & 0xF0F0F0F0u);
                 acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, xlo, acc[t], 0, 0, 0);
                 acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, xhi, acc[t], 0, 0, 0);
             }
@@ -745,6 +765,7 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
             }
         }
     }
+    __syncthreads();                                        // the staging buffers become the reduction buffer
     // ---- sum the eight partial tiles
 #pragma unroll
     for (int t = 0; t < MT; ++t)
@@ -948,19 +969,27 @@ int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, voi
 int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                   const void* bias, hipStream_t st) {
     const unsigned grid = (unsigned)((N + 31) / 32);
-#define QR_DEC(MT)                                                                                                    \
+#define QR_DEC(MT, SB)                                                                                                \
     do {                                                                                                              \
-        if (Y)                                                                                                        \
-            decode_i4_kernel<MT, true><<<dim3(grid), dim3(512), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N,  \
-                                                                         Kb, nullptr, (f16*)Y, (const f16*)sA,        \
-                                                                         (const f16*)sB, (const f16*)bias);           \
-        else                                                                                                          \
-            decode_i4_kernel<MT, false><<<dim3(grid), dim3(512), 0, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, \
-                                                                          Kb, (int32_t*)C, nullptr, nullptr, nullptr, \
-                                                                          nullptr);                                   \
+        constexpr int STAGE = (1 + MT) * 32 * (SB / 16), RED = MT * 4 * 64;                                           \
+        constexpr size_t LDS = (size_t)8 * (STAGE > RED ? STAGE : RED) * 16;                                          \
+        hipError_t e;                                                                                                 \
+        if (Y) {                                                                                                      \
+            auto kern = decode_i4_kernel<MT, SB, true>;                                                               \
+            e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
+            if (e != hipSuccess) return (int)e;                                                                       \
+            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr,         \
+                                                     (f16*)Y, (const f16*)sA, (const f16*)sB, (const f16*)bias);      \
+        } else {                                                                                                      \
+            auto kern = decode_i4_kernel<MT, SB, false>;                                                              \
+            e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
+            if (e != hipSuccess) return (int)e;                                                                       \
+            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
+                                                     nullptr, nullptr, nullptr, nullptr);                             \
+        }                                                                                                             \
     } while (0)
-    if (M <= 32) QR_DEC(1);
-    else QR_DEC(2);
+    if (M <= 32) QR_DEC(1, 128);
+    else QR_DEC(2, 128);
 #undef QR_DEC
     return qr_launch_status();
 }
@@ -994,7 +1023,7 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M <= 4 || (M <= 8 && (N + 255) / 256 < 128)) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (M <= 4) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     if (M <= 64) {
         // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
         // once per tile); otherwise eight waves split K over 32 rows

@@ -1,6 +1,7 @@
 // Shared device helpers for the gfx950 kernels of libquarot_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <stdint.h>
 #include "../../include/quarot_hip.h"
 
@@ -29,9 +30,11 @@ static inline hipError_t qr_allow_dynamic_lds(const void* kernel, size_t bytes) 
     };
     static Entry table[64];
     static int used = 0;
+    static std::mutex guard;                    // entry points may be called from several host threads
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(guard);
     for (int i = 0; i < used; ++i)
         if (table[i].fn == kernel && table[i].dev == dev && table[i].bytes >= bytes) return hipSuccess;
     e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
@@ -50,8 +53,10 @@ static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) 
     };
     static Entry table[64];
     static int used = 0;
+    static std::mutex guard;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 1;
+    std::lock_guard<std::mutex> lock(guard);
     for (int i = 0; i < used; ++i)
         if (table[i].fn == kernel && table[i].dev == dev && table[i].threads == threads && table[i].lds == lds)
             return table[i].blocks;
