@@ -67,6 +67,7 @@ def test_argument_errors_are_returned_before_any_launch(lib):
     assert lib.qr_hadamard(one, one, 2, 64, 1, None, 7, 1.0, None) == -5
     assert lib.qr_hadamard(one, one, 2, 11008, 172, None, 0, 1.0, None) == -1  # hadK missing
     assert lib.qr_hadamard_quantize_f16_i4(one, 2, 64, 1, None, 0, 1.0, 1.0, None, one, None, None) == -1
+    assert lib.qr_hadamard_quantize_f16_i4(one, 2, 64, 1, None, 0, 1.0, 1.0, ctypes.c_void_p(20), one, None, None) == -4  # codes: 8-byte aligned
     assert lib.qr_kv_quant_f16_i4(one, 4, 100, 0, one, one, one, None) == -3
     assert lib.qr_kv_quant_f16_i4(one, 4, 128, 3, one, one, one, None) == -5
     assert lib.qr_kv_dequant_i4_f16(one, one, one, 0, 128, one, None) == 0

@@ -325,6 +325,23 @@ def test_kv_quant_dequant_bit_exact(dim, hadamard):
     assert bool((err <= s.float() / 2 + 0.004 * (15 * s.float() + z.float().abs()) + 1e-3).all())
 
 
+def test_kv_vectors_with_infinities_take_the_ieee_path():
+    """An infinite element makes range and scale infinite: every finite element then gets code 0 and
+    inf / inf (NaN) converts to 0, as round/clamp/cast give in the reference; neighbouring finite
+    vectors in the same wave are unaffected."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((64, 128)).astype(F16)
+    x[5, 17] = np.inf
+    x[9, 3] = -np.inf
+    q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=False)
+    q, s, z = q.cpu().numpy(), s.cpu().numpy(), z.cpu().numpy()
+    assert np.isposinf(s[5, 0]) and np.all(q[5] == 0) and z[5, 0] == -x[5][np.isfinite(x[5])].min()
+    assert np.isposinf(s[9, 0]) and np.isposinf(z[9, 0])
+    keep = [i for i in range(64) if i not in (5, 9)]
+    wq, ws, wz = o.kv_asym_quant(x[keep])
+    assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
+
+
 def test_kv_full_size_round_trip():
     """The benchmark tensor [32, 4096, 8, 128]: codes in range, extremes hit, error bound, and a
     strided sample against the oracle."""
