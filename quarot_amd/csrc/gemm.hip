@@ -471,12 +471,17 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 
     // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during iteration
     // ks from registers requested at the end of iteration ks-1 (a second register set would spill).
+    // (the first three stages are requested together: the accumulators are not live yet, so two
+    // more register sets are free, and the prologue costs one memory round trip instead of three)
     u32x4 regs[NL];
-    fetch(0, regs);
-    deposit(0, 0, regs);
-    fetch(1, regs);
-    deposit(1, 1, regs);
-    fetch(2, regs);
+    {
+        u32x4 first[NL], second[NL];
+        fetch(0, first);
+        fetch(1, second);
+        fetch(2, regs);
+        deposit(0, 0, first);
+        deposit(1, 1, second);
+    }
     __syncthreads();                                        // stages 0 and 1 visible
     Ops ops;
     if (kg == 1) load_ops(0, 0, ops);                       // group 1 starts one unpack ahead
@@ -663,6 +668,250 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
+    }
+    return qr_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Software-pipelined variant of the 128x256 tile: four waves (2 x 2), ONE per SIMD, each owning a
+// 64x128 wave tile over the whole K range (no K split, no accumulator exchange).  A wave hides its
+// own LDS latency and unpacking under its own MFMAs: while the 16 MFMAs of 64-k sub-step u run, the
+// packed fragments of sub-step u+1 are unpacked and those of sub-step u+2 are read from LDS; the
+// instruction order is pinned with scheduling-group barriers (one MFMA, then a few VALU / LDS /
+// global-load slots).  A stage is 256 k (a 128-byte line per row); two LDS stage buffers, global
+// loads one stage ahead in registers, one workgroup barrier per stage.
+template <bool DEQ, bool RAGGED>
+__global__ __launch_bounds__(256) void gemm_sp_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
+    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
+    int tiles_m, int tiles_n) {
+    constexpr int BM = 128, BN = 256, NT = 256;
+    constexpr int TM = 64, TN = 128, IM = 2, JN = 4;
+    constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
+    constexpr int NL = CH / NT;                             // 12 per thread
+    extern __shared__ u32x4 sp_lds[];                       // [2][CH]; later the output slabs
+
+    const int nxcd = 8;
+    const int per_xcd = gridDim.x / nxcd;
+    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (tile >= tiles_m * tiles_n) return;
+    constexpr int GROUP_M = 8;
+    const int group_sz = GROUP_M * tiles_n;
+    const int g = tile / group_sz;
+    const int gm0 = g * GROUP_M;
+    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
+    const int tm = gm0 + (tile - g * group_sz) % gh;
+    const int tn = (tile - g * group_sz) / gh;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int khalf = lane >> 5;
+    const int stages = (Kb + 127) / 128;
+    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
+
+    // staging: chunk id = tid + i * 256: row = tid / 8 + 32 i, piece tid % 8
+    const int srow = tid >> 3;
+    const int scoff = (tid & 7) * 16;
+    const int dst0 = slot8(srow, tid & 7);                  // rows differ by multiples of 32: same swizzle key
+    u32 goff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int row = srow + i * 32;
+        int gr = row < BM ? m0 + row : n0 + row - BM;
+        const int lim = row < BM ? M - 1 : N - 1;
+        gr = gr < lim ? gr : lim;
+        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
+    }
+    u32x4 regs[NL];
+    // one 16-byte chunk of stage st (branch-free: stages past the end repeat the last one)
+    auto fetch1 = [&](int st, int i) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        const uint8_t* base = (i * 32 < BM) ? A : B;
+        if (RAGGED) {
+            const u32 off = (u32)((kb + scoff < Kb) ? kb + scoff : kb);
+            regs[i] = *(const u32x4*)(base + (size_t)(goff[i] + off));
+        } else {
+            regs[i] = *(const u32x4*)(base + (size_t)(goff[i] + (u32)kb));
+        }
+    };
+    auto deposit1 = [&](int st, int buf, int i) {             // st past the end: a repeat of the last stage, never read
+        const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
+        sp_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[i];
+    };
+
+    i32x16 acc[IM][JN];
+#pragma unroll
+    for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    // fragment slots of sub-step u: logical chunk 2 u + khalf
+    int aslot[4], bslot[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        aslot[u] = slot8(wm * TM + (lane & 31), 2 * u + khalf);
+        bslot[u] = slot8(BM + wn * TN + (lane & 31), 2 * u + khalf);
+    }
+    // fragments: index 0..1 = A (32-row tiles of the wave tile), 2..5 = B
+    struct Packed {
+        u32x4 f[IM + JN];
+    };
+    struct Ops {
+        i32x4 lo[IM + JN], hi[IM + JN];
+    };
+    auto read1 = [&](int buf, int u, int r, Packed& p) {
+        p.f[r] = r < IM ? sp_lds[buf * CH + aslot[u] + r * 32 * 8] : sp_lds[buf * CH + bslot[u] + (r - IM) * 32 * 8];
+    };
+    // unpacking as 72 single instructions: dword d = n / 3 of the 24 packed dwords,
+    // n % 3 = 0: lo = p << 4;  1: lo &= mask;  2: hi = p & mask
+    auto unpack1 = [&](const Packed& p, Ops& o, int n) {
+        const int d = n / 3, f = d >> 2, e = d & 3, kind = n % 3;
+        if (kind == 0) o.lo[f][e] = (int)(p.f[f][e] << 4);
+        else if (kind == 1) o.lo[f][e] = o.lo[f][e] & (int)0xF0F0F0F0u;
+        else o.hi[f][e] = (int)(p.f[f][e] & 0xF0F0F0F0u);
+    };
+    auto mfma1 = [&](const Ops& o, int q) {
+        const int i = (q & 7) >> 2, j = q & 3;
+        if (q < 8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.lo[IM + j], o.lo[i], acc[i][j], 0, 0, 0);
+        else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.hi[IM + j], o.hi[i], acc[i][j], 0, 0, 0);
+    };
+    // One 64-k sub-step = 16 slots.  Slot q: MFMA q of the current operands; 4 or 5 of the 72
+    // unpacking instructions of the next sub-step; at most one LDS read (fragments of the sub-step
+    // after next), LDS write (stage ks+1) or global load (stage ks+2).  A full scheduling barrier
+    // after every slot keeps this order.
+#define QR_SP_SUBSTEP(CUR, NXT, PK_NEXT, PK_FILL, RBUF, RU, DEP, FET)                           \
+    _Pragma("unroll") for (int q_ = 0; q_ < 16; ++q_) {                                          \
+        mfma1(CUR, q_);                                                                          \
+        _Pragma("unroll") for (int n_ = (q_ * 72) / 16; n_ < ((q_ + 1) * 72) / 16; ++n_) unpack1(PK_NEXT, NXT, n_); \
+        if (q_ < IM + JN) read1(RBUF, RU, q_, PK_FILL);                                          \
+        if ((DEP) && q_ >= 2 && q_ < 2 + NL) deposit1(ks + 1, nb, q_ - 2);                       \
+        if ((FET) && q_ >= 2 && q_ < 2 + NL) fetch1(ks + 2, q_ - 2);                             \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    }
+
+    // prologue: stage 0 into LDS, stage 1 requested; sub-step 0 unpacked, sub-step 1 fragments in flight
+    Packed pk[2];
+    Ops ops[2];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) deposit1(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(1, i);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < IM + JN; ++r) read1(0, 0, r, pk[0]);
+#pragma unroll
+    for (int r = 0; r < IM + JN; ++r) read1(0, 1, r, pk[1]);
+#pragma unroll
+    for (int n = 0; n < 72; ++n) unpack1(pk[0], ops[0], n);
+    for (int ks = 0; ks < stages; ++ks) {
+        const int b = ks & 1, nb = b ^ 1;
+        // sub-step 0: multiply (ks,0); unpack (ks,1); read (ks,2); stage ks+1 -> LDS
+        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], b, 2, true, false)
+        // sub-step 1: multiply (ks,1); unpack (ks,2); read (ks,3); request stage ks+2
+        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], b, 3, false, true)
+        __syncthreads();                                    // stage ks+1 visible; stage ks fully read
+        // sub-step 2: multiply (ks,2); unpack (ks,3); read (ks+1,0)
+        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], nb, 0, false, false)
+        // sub-step 3: multiply (ks,3); unpack (ks+1,0); read (ks+1,1)
+        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], nb, 1, false, false)
+    }
+#undef QR_SP_SUBSTEP
+    __syncthreads();                                        // stage buffers free for the output slabs
+
+    // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    if (DEQ && by_rows) {
+#pragma unroll
+        for (int jb = 0; jb < JN; jb += 2) {
+            f16x4 sbh[2][4], bih[2][4];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
+                    sbh[jj][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                }
+#pragma unroll
+            for (int i = 0; i < IM; ++i) {
+                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                f16x4 o[2][4];
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
+                            if (bias) yv = yv + bih[jj][gq][e];
+                            o[jj][gq][e] = yv;
+                        }
+                store_slab_rows<2>((u32x2*)(sp_lds + wave * 256), o, lane,
+                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < IM; ++i) {
+        const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (row >= M) continue;
+        f16 sa = (f16)0;
+        if (DEQ) sa = sA[row];
+#pragma unroll
+        for (int j = 0; j < JN; ++j) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
+                if (col >= N) continue;
+                int v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
+                if (DEQ) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (col + e < N) {
+                            f16 yv = (f16)(sa * sB[col + e]) * (f16)(float)v4[e];
+                            if (bias) yv = yv + bias[col + e];
+                            Y[(int64_t)row * N + col + e] = yv;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) C[(int64_t)row * N + col + e] = v4[e];
+                }
+            }
+        }
+    }
+}
+
+int launch_sp(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+              const void* bias, hipStream_t st) {
+    constexpr size_t LDS = (size_t)2 * (128 + 256) * 8 * 16;
+    const int tiles_m = (M + 127) / 128, tiles_n = (N + 255) / 256;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles > 0x3fffffff) return QR_E_SHAPE;
+    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const bool ragged = (Kb & 127) != 0;
+    hipError_t e;
+    if (Y) {
+        auto kern = ragged ? gemm_sp_kernel<true, true> : gemm_sp_kernel<true, false>;
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
+                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+    } else {
+        auto kern = ragged ? gemm_sp_kernel<false, true> : gemm_sp_kernel<false, false>;
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
+                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
     }
     return qr_launch_status();
 }
@@ -1032,7 +1281,7 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     }
     if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 128) return launch_ks<128, 256, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t128x256 >= 128) return launch_sp(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     if (N > 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
