@@ -723,21 +723,22 @@ __global__ __launch_bounds__(256) void gemm_sp_kernel(
         gr = gr < lim ? gr : lim;
         goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
     }
-    u32x4 regs[NL];
-    // one 16-byte chunk of stage st (branch-free: stages past the end repeat the last one)
-    auto fetch1 = [&](int st, int i) {
+    u32x4 regs[2][NL];                                      // two sets: loads run two stages ahead of their LDS write
+    // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
+    // buffer load: scalar descriptor + scalar stage offset + constant 32-bit per-thread offset, so
+    // the address costs no vector instruction and half the address traffic of a 64-bit pointer.
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((u32)M * (u32)Kb), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (int)((u32)N * (u32)Kb), 0x00020000);
+    auto fetch1 = [&](int st, int set, int i) {
         const int kb = (st < stages ? st : stages - 1) * 128;
-        const uint8_t* base = (i * 32 < BM) ? A : B;
-        if (RAGGED) {
-            const u32 off = (u32)((kb + scoff < Kb) ? kb + scoff : kb);
-            regs[i] = *(const u32x4*)(base + (size_t)(goff[i] + off));
-        } else {
-            regs[i] = *(const u32x4*)(base + (size_t)(goff[i] + (u32)kb));
-        }
+        u32 off = goff[i];
+        if (RAGGED) off += (u32)((kb + scoff < Kb) ? scoff : 0);
+        regs[set][i] = (i * 32 < BM) ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, kb, 0)
+                                     : __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, kb, 0);
     };
-    auto deposit1 = [&](int st, int buf, int i) {             // st past the end: a repeat of the last stage, never read
+    auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
         const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
-        sp_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[i];
+        sp_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
     };
 
     i32x16 acc[IM][JN];
@@ -782,25 +783,46 @@ __global__ __launch_bounds__(256) void gemm_sp_kernel(
     // unpacking instructions of the next sub-step; at most one LDS read (fragments of the sub-step
     // after next), LDS write (stage ks+1) or global load (stage ks+2).  A full scheduling barrier
     // after every slot keeps this order.
-#define QR_SP_SUBSTEP(CUR, NXT, PK_NEXT, PK_FILL, RBUF, RU, DEP, FET)                           \
+#define QR_SP_SUBSTEP(CUR, NXT, PK_NEXT, PK_FILL, RBUF, RU, DEP, SET)                           \
     _Pragma("unroll") for (int q_ = 0; q_ < 16; ++q_) {                                          \
         mfma1(CUR, q_);                                                                          \
         _Pragma("unroll") for (int n_ = (q_ * 72) / 16; n_ < ((q_ + 1) * 72) / 16; ++n_) unpack1(PK_NEXT, NXT, n_); \
         if (q_ < IM + JN) read1(RBUF, RU, q_, PK_FILL);                                          \
-        if ((DEP) && q_ >= 2 && q_ < 2 + NL) deposit1(ks + 1, nb, q_ - 2);                       \
-        if ((FET) && q_ >= 2 && q_ < 2 + NL) fetch1(ks + 2, q_ - 2);                             \
+        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
+            deposit1(ks_ + 1, nb_, SET, q_ - 2);                                                 \
+            fetch1(ks_ + 3, SET, q_ - 2);                                                        \
+        }                                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     }
 
-    // prologue: stage 0 into LDS, stage 1 requested; sub-step 0 unpacked, sub-step 1 fragments in flight
+    // one stage: KS = stage index, B = its LDS buffer (compile-time), SET = register set that holds
+    // stage KS+1 on entry and receives stage KS+3
+#define QR_SP_STAGE(KS, B, SET)                                                                  \
+    {                                                                                            \
+        const int ks_ = (KS);                                                                    \
+        constexpr int b_ = (B), nb_ = 1 - (B);                                                   \
+        /* sub-step 0: multiply (ks,0); unpack (ks,1); read (ks,2); stage ks+1 -> LDS, request ks+3 */ \
+        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], b_, 2, true, SET)                            \
+        /* sub-step 1: multiply (ks,1); unpack (ks,2); read (ks,3) */                            \
+        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], b_, 3, false, SET)                           \
+        __syncthreads(); /* stage ks+1 visible; stage ks fully read */                           \
+        /* sub-step 2: multiply (ks,2); unpack (ks,3); read (ks+1,0) */                          \
+        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], nb_, 0, false, SET)                          \
+        /* sub-step 3: multiply (ks,3); unpack (ks+1,0); read (ks+1,1) */                        \
+        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], nb_, 1, false, SET)                          \
+    }
+
+    // prologue: stage 0 into LDS, stages 1 and 2 requested; sub-step 0 unpacked, sub-step 1 fragments in flight
     Packed pk[2];
     Ops ops[2];
 #pragma unroll
-    for (int i = 0; i < NL; ++i) fetch1(0, i);
+    for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
 #pragma unroll
-    for (int i = 0; i < NL; ++i) deposit1(0, 0, i);
+    for (int i = 0; i < NL; ++i) fetch1(2, 1, i);
 #pragma unroll
-    for (int i = 0; i < NL; ++i) fetch1(1, i);
+    for (int i = 0; i < NL; ++i) deposit1(0, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(1, 0, i);
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < IM + JN; ++r) read1(0, 0, r, pk[0]);
@@ -808,18 +830,15 @@ __global__ __launch_bounds__(256) void gemm_sp_kernel(
     for (int r = 0; r < IM + JN; ++r) read1(0, 1, r, pk[1]);
 #pragma unroll
     for (int n = 0; n < 72; ++n) unpack1(pk[0], ops[0], n);
-    for (int ks = 0; ks < stages; ++ks) {
-        const int b = ks & 1, nb = b ^ 1;
-        // sub-step 0: multiply (ks,0); unpack (ks,1); read (ks,2); stage ks+1 -> LDS
-        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], b, 2, true, false)
-        // sub-step 1: multiply (ks,1); unpack (ks,2); read (ks,3); request stage ks+2
-        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], b, 3, false, true)
-        __syncthreads();                                    // stage ks+1 visible; stage ks fully read
-        // sub-step 2: multiply (ks,2); unpack (ks,3); read (ks+1,0)
-        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], nb, 0, false, false)
-        // sub-step 3: multiply (ks,3); unpack (ks+1,0); read (ks+1,1)
-        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], nb, 1, false, false)
+    // (pairs of stages without a branch in between: the wait before an LDS write then counts the
+    // other set's loads as still allowed in flight)
+    int ks = 0;
+    for (; ks + 1 < stages; ks += 2) {
+        QR_SP_STAGE(ks, 0, 0)
+        QR_SP_STAGE(ks + 1, 1, 1)
     }
+    if (ks < stages) QR_SP_STAGE(ks, 0, 0)
+#undef QR_SP_STAGE
 #undef QR_SP_SUBSTEP
     __syncthreads();                                        // stage buffers free for the output slabs
 
@@ -899,6 +918,9 @@ int launch_sp(const void* A, const void* B, int M, int N, int Kb, void* C, void*
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     const bool ragged = (Kb & 127) != 0;
+    // operands are addressed through 32-bit buffer offsets
+    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
+        return launch_ks<128, 256, 2, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
     hipError_t e;
     if (Y) {
         auto kern = ragged ? gemm_sp_kernel<true, true> : gemm_sp_kernel<true, false>;
