@@ -51,8 +51,8 @@ HBM_PEAK_GBS = 8000.0
 FETCH_SCALE, WRITE_SCALE = 262144.0 / 131083.8, 262144.0 / 262144.0
 TRAFFIC_KIB = {
     #        FETCH_SIZE   WRITE_SIZE
-    "c1": (16573.2, 16384.0),
-    "c2": (44221.2, 16384.0),
+    "c1": (16568.9, 16384.0),
+    "c2": (44236.7, 16384.0),
     "c3d": (528728.3, 262144.0),
     "c4": (72440.1, 1024.0),
     "c4m1": (61875.4, 16.0),
@@ -215,7 +215,8 @@ def main():
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel"] = ("gemv_i4_kernel" if m <= 4 else
                       ("gemm_ks_kernel<64,256>" if (n + 255) // 256 >= 128 else "decode_i4_kernel") if decode else
-                      "gemm_ks_kernel" if ((m + 255) // 256) * ((n + 255) // 256) < 512 else "gemm_i4_kernel<256,256>")
+                      "gemm_i4_kernel<256,256>" if ((m + 255) // 256) * ((n + 255) // 256) >= 512 else
+                      "gemm_sp_kernel" if ((m + 127) // 128) * ((n + 255) // 256) >= 128 else "gemm_ks_kernel<64,256>")
     roof["kernel"] += " (int4 GEMM + dequant epilogue)"
     roof["kernel_ms"] = round(gemm_ms, 4)
 
