@@ -910,6 +910,226 @@ __global__ __launch_bounds__(256) void gemm_sp_kernel(
     }
 }
 
+template <bool DEQ, bool RAGGED>
+__global__ __launch_bounds__(256) void gemm_sp256_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
+    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
+    int tiles_m, int tiles_n) {
+    constexpr int BM = 256, BN = 256, NT = 256;
+    constexpr int TM = 128, TN = 128, IM = 4, JN = 4;
+    constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
+    constexpr int NL = CH / NT;                             // 16 per thread
+    constexpr int NF = IM + JN;                             // fragments per sub-step
+    constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
+    constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
+    constexpr int S0 = 8;                                   // first slot that unpacks (LDS reads issued in slots 0..7)
+    extern __shared__ u32x4 sp2_lds[];                       // [2][CH]; later the output slabs
+
+    const int nxcd = 8;
+    const int per_xcd = gridDim.x / nxcd;
+    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (tile >= tiles_m * tiles_n) return;
+    constexpr int GROUP_M = 8;
+    const int group_sz = GROUP_M * tiles_n;
+    const int g = tile / group_sz;
+    const int gm0 = g * GROUP_M;
+    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
+    const int tm = gm0 + (tile - g * group_sz) % gh;
+    const int tn = (tile - g * group_sz) / gh;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int khalf = lane >> 5;
+    const int stages = (Kb + 127) / 128;
+    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
+
+    // staging: chunk id = tid + i * 256: row = tid / 8 + 32 i, piece tid % 8
+    const int srow = tid >> 3;
+    const int scoff = (tid & 7) * 16;
+    const int dst0 = slot8(srow, tid & 7);                  // rows differ by multiples of 32: same swizzle key
+    u32 goff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int row = srow + i * 32;
+        int gr = row < BM ? m0 + row : n0 + row - BM;
+        const int lim = row < BM ? M - 1 : N - 1;
+        gr = gr < lim ? gr : lim;
+        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
+    }
+    u32x4 regs[1][NL];                                      // one set: loads run one (long) stage ahead of their LDS write
+    // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
+    // buffer load: scalar descriptor + scalar stage offset + constant 32-bit per-thread offset, so
+    // the address costs no vector instruction and half the address traffic of a 64-bit pointer.
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((u32)M * (u32)Kb), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (int)((u32)N * (u32)Kb), 0x00020000);
+    auto fetch1 = [&](int st, int set, int i) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        u32 off = goff[i];
+        if (RAGGED) off += (u32)((kb + scoff < Kb) ? scoff : 0);
+        regs[set][i] = (i * 32 < BM) ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, kb, 0)
+                                     : __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, kb, 0);
+    };
+    auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
+        const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
+        sp2_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
+    };
+
+    i32x16 acc[IM][JN];
+#pragma unroll
+    for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    // fragment slots of sub-step u: logical chunk 2 u + khalf
+    int aslot[4], bslot[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        aslot[u] = slot8(wm * TM + (lane & 31), 2 * u + khalf);
+        bslot[u] = slot8(BM + wn * TN + (lane & 31), 2 * u + khalf);
+    }
+    // fragments: index 0..1 = A (32-row tiles of the wave tile), 2..5 = B
+    struct Packed {
+        u32x4 f[IM + JN];
+    };
+    struct Ops {
+        i32x4 lo[IM + JN], hi[IM + JN];
+    };
+    auto read1 = [&](int buf, int u, int r, Packed& p) {
+        p.f[r] = r < IM ? sp2_lds[buf * CH + aslot[u] + r * 32 * 8] : sp2_lds[buf * CH + bslot[u] + (r - IM) * 32 * 8];
+    };
+    // unpacking as UNP single instructions: dword d = n / 3 of the packed dwords,
+    // n % 3 = 0: lo = p << 4;  1: lo &= mask;  2: hi = p & mask
+    auto unpack1 = [&](const Packed& p, Ops& o, int n) {
+        const int d = n / 3, f = d >> 2, e = d & 3, kind = n % 3;
+        if (kind == 0) o.lo[f][e] = (int)(p.f[f][e] << 4);
+        else if (kind == 1) o.lo[f][e] = o.lo[f][e] & (int)0xF0F0F0F0u;
+        else o.hi[f][e] = (int)(p.f[f][e] & 0xF0F0F0F0u);
+    };
+    auto mfma1 = [&](const Ops& o, int q) {
+        const int t = q % (IM * JN), i = t / JN, j = t % JN;
+        if (q < IM * JN) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.lo[IM + j], o.lo[i], acc[i][j], 0, 0, 0);
+        else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.hi[IM + j], o.hi[i], acc[i][j], 0, 0, 0);
+    };
+    // One 64-k sub-step = NMF = 32 slots.  Slot q: MFMA q of the current operands; slots 0..7 read
+    // the packed fragments of the NEXT sub-step (one fragment buffer), slots S0.. unpack them
+    // (UNP / (NMF - S0) = 4 instructions per slot); in sub-step 0, slots 2.. also write one chunk of
+    // stage ks+1 to LDS and request the same chunk of stage ks+2.  A full scheduling barrier after
+    // every slot keeps this order.
+#define QR_SP2_SUBSTEP(CUR, NXT, RBUF, RU, DEP)                                                  \
+    _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
+        mfma1(CUR, q_);                                                                          \
+        if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
+        if (q_ >= S0) {                                                                          \
+            _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
+                unpack1(pk, NXT, n_);                                                            \
+        }                                                                                        \
+        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
+            deposit1(ks + 1, nb, 0, q_ - 2);                                                     \
+            fetch1(ks + 2, 0, q_ - 2);                                                           \
+        }                                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    }
+
+    // prologue: stage 0 into LDS, stage 1 requested; sub-step 0 unpacked
+    Packed pk;
+    Ops ops[2];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) deposit1(0, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(1, 0, i);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NF; ++r) read1(0, 0, r, pk);
+#pragma unroll
+    for (int n = 0; n < UNP; ++n) unpack1(pk, ops[0], n);
+    for (int ks = 0; ks < stages; ++ks) {
+        const int b = ks & 1, nb = b ^ 1;
+        // sub-step 0: multiply (ks,0); read + unpack (ks,1); stage ks+1 -> LDS, request ks+2
+        QR_SP2_SUBSTEP(ops[0], ops[1], b, 1, true)
+        // sub-step 1: multiply (ks,1); read + unpack (ks,2)
+        QR_SP2_SUBSTEP(ops[1], ops[0], b, 2, false)
+        // sub-step 2: multiply (ks,2); read + unpack (ks,3)
+        QR_SP2_SUBSTEP(ops[0], ops[1], b, 3, false)
+        __syncthreads();                                    // stage ks+1 visible; stage ks fully read
+        // sub-step 3: multiply (ks,3); read + unpack (ks+1,0)
+        QR_SP2_SUBSTEP(ops[1], ops[0], nb, 0, false)
+    }
+#undef QR_SP2_SUBSTEP
+    __syncthreads();                                        // stage buffers free for the output slabs
+
+    // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    if (DEQ && by_rows) {
+#pragma unroll
+        for (int jb = 0; jb < JN; jb += 2) {
+            f16x4 sbh[2][4], bih[2][4];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
+                    sbh[jj][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                }
+#pragma unroll
+            for (int i = 0; i < IM; ++i) {
+                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                f16x4 o[2][4];
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
+                            if (bias) yv = yv + bih[jj][gq][e];
+                            o[jj][gq][e] = yv;
+                        }
+                store_slab_rows<2>((u32x2*)(sp2_lds + wave * 256), o, lane,
+                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < IM; ++i) {
+        const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (row >= M) continue;
+        f16 sa = (f16)0;
+        if (DEQ) sa = sA[row];
+#pragma unroll
+        for (int j = 0; j < JN; ++j) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
+                if (col >= N) continue;
+                int v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
+                if (DEQ) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (col + e < N) {
+                            f16 yv = (f16)(sa * sB[col + e]) * (f16)(float)v4[e];
+                            if (bias) yv = yv + bias[col + e];
+                            Y[(int64_t)row * N + col + e] = yv;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) C[(int64_t)row * N + col + e] = v4[e];
+                }
+            }
+        }
+    }
+}
+
 int launch_sp(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
               const void* bias, hipStream_t st) {
     constexpr size_t LDS = (size_t)2 * (128 + 256) * 8 * 16;
@@ -930,6 +1150,38 @@ int launch_sp(const void* A, const void* B, int M, int N, int Kb, void* C, void*
                                                  (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
     } else {
         auto kern = ragged ? gemm_sp_kernel<false, true> : gemm_sp_kernel<false, false>;
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
+                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
+    }
+    return qr_launch_status();
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+               const void* bias, hipStream_t st);
+
+int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+                 const void* bias, hipStream_t st) {
+    constexpr size_t LDS = (size_t)2 * (256 + 256) * 8 * 16;
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles > 0x3fffffff) return QR_E_SHAPE;
+    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const bool ragged = (Kb & 127) != 0;
+    // operands are addressed through 32-bit buffer offsets
+    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
+        return launch_cfg<256, 256, 4, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
+    hipError_t e;
+    if (Y) {
+        auto kern = ragged ? gemm_sp256_kernel<true, true> : gemm_sp256_kernel<true, false>;
+        e = qr_allow_dynamic_lds((const void*)kern, LDS);
+        if (e != hipSuccess) return (int)e;
+        kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
+                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+    } else {
+        auto kern = ragged ? gemm_sp256_kernel<false, true> : gemm_sp256_kernel<false, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
@@ -1301,9 +1553,16 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         if ((N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
-    if (t256 >= 512) return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 128) return launch_sp(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    if (t128x256 >= 128) {
+        // 256x256 tiles run ~1.2x faster per unit of work (3 instead of 4.5 unpacking instructions per
+        // MFMA) but quantise worse over the 256 CUs: compare rounds of tiles, a 128x256 tile costing
+        // 0.61 of a 256x256 one
+        const double rounds256 = (double)((t256 + 255) / 256);
+        const double rounds128 = (double)((t128x256 + 255) / 256) * 0.61;
+        if (rounds256 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        return launch_sp(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    }
     if (N > 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
 }
