@@ -673,243 +673,20 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
 }
 
 // ------------------------------------------------------------------------------------------------
-// Software-pipelined variant of the 128x256 tile: four waves (2 x 2), ONE per SIMD, each owning a
-// 64x128 wave tile over the whole K range (no K split, no accumulator exchange).  A wave hides its
-// own LDS latency and unpacking under its own MFMAs: while the 16 MFMAs of 64-k sub-step u run, the
-// packed fragments of sub-step u+1 are unpacked and those of sub-step u+2 are read from LDS; the
-// instruction order is pinned with scheduling-group barriers (one MFMA, then a few VALU / LDS /
-// global-load slots).  A stage is 256 k (a 128-byte line per row); two LDS stage buffers, global
-// loads one stage ahead in registers, one workgroup barrier per stage.
-template <bool DEQ, bool RAGGED>
-__global__ __launch_bounds__(256) void gemm_sp_kernel(
-    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
-    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n) {
-    constexpr int BM = 128, BN = 256, NT = 256;
-    constexpr int TM = 64, TN = 128, IM = 2, JN = 4;
-    constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
-    constexpr int NL = CH / NT;                             // 12 per thread
-    extern __shared__ u32x4 sp_lds[];                       // [2][CH]; later the output slabs
-
-    const int nxcd = 8;
-    const int per_xcd = gridDim.x / nxcd;
-    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
-    if (tile >= tiles_m * tiles_n) return;
-    constexpr int GROUP_M = 8;
-    const int group_sz = GROUP_M * tiles_n;
-    const int g = tile / group_sz;
-    const int gm0 = g * GROUP_M;
-    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
-    const int tm = gm0 + (tile - g * group_sz) % gh;
-    const int tn = (tile - g * group_sz) / gh;
-    const int m0 = tm * BM, n0 = tn * BN;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int khalf = lane >> 5;
-    const int stages = (Kb + 127) / 128;
-    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
-
-    // staging: chunk id = tid + i * 256: row = tid / 8 + 32 i, piece tid % 8
-    const int srow = tid >> 3;
-    const int scoff = (tid & 7) * 16;
-    const int dst0 = slot8(srow, tid & 7);                  // rows differ by multiples of 32: same swizzle key
-    u32 goff[NL];
-#pragma unroll
-    for (int i = 0; i < NL; ++i) {
-        const int row = srow + i * 32;
-        int gr = row < BM ? m0 + row : n0 + row - BM;
-        const int lim = row < BM ? M - 1 : N - 1;
-        gr = gr < lim ? gr : lim;
-        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
-    }
-    u32x4 regs[2][NL];                                      // two sets: loads run two stages ahead of their LDS write
-    // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
-    // buffer load: scalar descriptor + scalar stage offset + constant 32-bit per-thread offset, so
-    // the address costs no vector instruction and half the address traffic of a 64-bit pointer.
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((u32)M * (u32)Kb), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (int)((u32)N * (u32)Kb), 0x00020000);
-    auto fetch1 = [&](int st, int set, int i) {
-        const int kb = (st < stages ? st : stages - 1) * 128;
-        u32 off = goff[i];
-        if (RAGGED) off += (u32)((kb + scoff < Kb) ? scoff : 0);
-        regs[set][i] = (i * 32 < BM) ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, kb, 0)
-                                     : __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, kb, 0);
-    };
-    auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
-        const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
-        sp_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
-    };
-
-    i32x16 acc[IM][JN];
-#pragma unroll
-    for (int i = 0; i < IM; ++i)
-#pragma unroll
-        for (int j = 0; j < JN; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-
-    // fragment slots of sub-step u: logical chunk 2 u + khalf
-    int aslot[4], bslot[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        aslot[u] = slot8(wm * TM + (lane & 31), 2 * u + khalf);
-        bslot[u] = slot8(BM + wn * TN + (lane & 31), 2 * u + khalf);
-    }
-    // fragments: index 0..1 = A (32-row tiles of the wave tile), 2..5 = B
-    struct Packed {
-        u32x4 f[IM + JN];
-    };
-    struct Ops {
-        i32x4 lo[IM + JN], hi[IM + JN];
-    };
-    auto read1 = [&](int buf, int u, int r, Packed& p) {
-        p.f[r] = r < IM ? sp_lds[buf * CH + aslot[u] + r * 32 * 8] : sp_lds[buf * CH + bslot[u] + (r - IM) * 32 * 8];
-    };
-    // unpacking as 72 single instructions: dword d = n / 3 of the 24 packed dwords,
-    // n % 3 = 0: lo = p << 4;  1: lo &= mask;  2: hi = p & mask
-    auto unpack1 = [&](const Packed& p, Ops& o, int n) {
-        const int d = n / 3, f = d >> 2, e = d & 3, kind = n % 3;
-        if (kind == 0) o.lo[f][e] = (int)(p.f[f][e] << 4);
-        else if (kind == 1) o.lo[f][e] = o.lo[f][e] & (int)0xF0F0F0F0u;
-        else o.hi[f][e] = (int)(p.f[f][e] & 0xF0F0F0F0u);
-    };
-    auto mfma1 = [&](const Ops& o, int q) {
-        const int i = (q & 7) >> 2, j = q & 3;
-        if (q < 8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.lo[IM + j], o.lo[i], acc[i][j], 0, 0, 0);
-        else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.hi[IM + j], o.hi[i], acc[i][j], 0, 0, 0);
-    };
-    // One 64-k sub-step = 16 slots.  Slot q: MFMA q of the current operands; 4 or 5 of the 72
-    // unpacking instructions of the next sub-step; at most one LDS read (fragments of the sub-step
-    // after next), LDS write (stage ks+1) or global load (stage ks+2).  A full scheduling barrier
-    // after every slot keeps this order.
-#define QR_SP_SUBSTEP(CUR, NXT, PK_NEXT, PK_FILL, RBUF, RU, DEP, SET)                           \
-    _Pragma("unroll") for (int q_ = 0; q_ < 16; ++q_) {                                          \
-        mfma1(CUR, q_);                                                                          \
-        _Pragma("unroll") for (int n_ = (q_ * 72) / 16; n_ < ((q_ + 1) * 72) / 16; ++n_) unpack1(PK_NEXT, NXT, n_); \
-        if (q_ < IM + JN) read1(RBUF, RU, q_, PK_FILL);                                          \
-        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
-            deposit1(ks_ + 1, nb_, SET, q_ - 2);                                                 \
-            fetch1(ks_ + 3, SET, q_ - 2);                                                        \
-        }                                                                                        \
-        __builtin_amdgcn_sched_barrier(0);                                                       \
-    }
-
-    // one stage: KS = stage index, B = its LDS buffer (compile-time), SET = register set that holds
-    // stage KS+1 on entry and receives stage KS+3
-#define QR_SP_STAGE(KS, B, SET)                                                                  \
-    {                                                                                            \
-        const int ks_ = (KS);                                                                    \
-        constexpr int b_ = (B), nb_ = 1 - (B);                                                   \
-        /* sub-step 0: multiply (ks,0); unpack (ks,1); read (ks,2); stage ks+1 -> LDS, request ks+3 */ \
-        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], b_, 2, true, SET)                            \
-        /* sub-step 1: multiply (ks,1); unpack (ks,2); read (ks,3) */                            \
-        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], b_, 3, false, SET)                           \
-        __syncthreads(); /* stage ks+1 visible; stage ks fully read */                           \
-        /* sub-step 2: multiply (ks,2); unpack (ks,3); read (ks+1,0) */                          \
-        QR_SP_SUBSTEP(ops[0], ops[1], pk[1], pk[0], nb_, 0, false, SET)                          \
-        /* sub-step 3: multiply (ks,3); unpack (ks+1,0); read (ks+1,1) */                        \
-        QR_SP_SUBSTEP(ops[1], ops[0], pk[0], pk[1], nb_, 1, false, SET)                          \
-    }
-
-    // prologue: stage 0 into LDS, stages 1 and 2 requested; sub-step 0 unpacked, sub-step 1 fragments in flight
-    Packed pk[2];
-    Ops ops[2];
-#pragma unroll
-    for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
-#pragma unroll
-    for (int i = 0; i < NL; ++i) fetch1(2, 1, i);
-#pragma unroll
-    for (int i = 0; i < NL; ++i) deposit1(0, 0, 0, i);
-#pragma unroll
-    for (int i = 0; i < NL; ++i) fetch1(1, 0, i);
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < IM + JN; ++r) read1(0, 0, r, pk[0]);
-#pragma unroll
-    for (int r = 0; r < IM + JN; ++r) read1(0, 1, r, pk[1]);
-#pragma unroll
-    for (int n = 0; n < 72; ++n) unpack1(pk[0], ops[0], n);
-    // (pairs of stages without a branch in between: the wait before an LDS write then counts the
-    // other set's loads as still allowed in flight)
-    int ks = 0;
-    for (; ks + 1 < stages; ks += 2) {
-        QR_SP_STAGE(ks, 0, 0)
-        QR_SP_STAGE(ks + 1, 1, 1)
-    }
-    if (ks < stages) QR_SP_STAGE(ks, 0, 0)
-#undef QR_SP_STAGE
-#undef QR_SP_SUBSTEP
-    __syncthreads();                                        // stage buffers free for the output slabs
-
-    // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
-    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
-    if (DEQ && by_rows) {
-#pragma unroll
-        for (int jb = 0; jb < JN; jb += 2) {
-            f16x4 sbh[2][4], bih[2][4];
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                for (int gq = 0; gq < 4; ++gq) {
-                    const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
-                    sbh[jj][gq] = *(const f16x4*)(sB + col);
-                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
-                }
-#pragma unroll
-            for (int i = 0; i < IM; ++i) {
-                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
-                f16x4 o[2][4];
-#pragma unroll
-                for (int jj = 0; jj < 2; ++jj)
-#pragma unroll
-                    for (int gq = 0; gq < 4; ++gq)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
-                            if (bias) yv = yv + bih[jj][gq][e];
-                            o[jj][gq][e] = yv;
-                        }
-                store_slab_rows<2>((u32x2*)(sp_lds + wave * 256), o, lane,
-                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
-            }
-        }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < IM; ++i) {
-        const int row = m0 + wm * TM + i * 32 + (lane & 31);
-        if (row >= M) continue;
-        f16 sa = (f16)0;
-        if (DEQ) sa = sA[row];
-#pragma unroll
-        for (int j = 0; j < JN; ++j) {
-#pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                const int col = n0 + wn * TN + j * 32 + gq * 8 + khalf * 4;
-                if (col >= N) continue;
-                int v4[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
-                if (DEQ) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (col + e < N) {
-                            f16 yv = (f16)(sa * sB[col + e]) * (f16)(float)v4[e];
-                            if (bias) yv = yv + bias[col + e];
-                            Y[(int64_t)row * N + col + e] = yv;
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (col + e < N) C[(int64_t)row * N + col + e] = v4[e];
-                }
-            }
-        }
-    }
-}
-
+// Software-pipelined kernels: four waves, ONE per SIMD, each owning a 128x128 wave tile (16 MFMA
+// tiles, all 256 AGPRs), so that unpacking costs 3 instructions per MFMA.  A wave hides its own LDS
+// latency and unpacking under its own MFMAs: while the 32 MFMAs of a 64-k sub-step run, the packed
+// fragments of its next sub-step are read from LDS and unpacked.  The loop is written as explicit
+// slots -- one MFMA, up to 4 unpacking instructions, at most one LDS read / LDS write / global
+// load -- and a full scheduling barrier after every slot keeps the compiler from regrouping them
+// (measured for one wave per SIMD: up to 5 VALU per MFMA cost 9 %, 6 cost 40 %).  A stage is 256 k
+// (a 128-byte line per row); two LDS stage buffers; global loads are raw buffer loads (scalar
+// descriptor + scalar stage offset + constant 32-bit lane offset: no address arithmetic in the loop)
+// running ahead in registers; one workgroup barrier per stage.
+//   gemm_sp256_kernel  256x256 tile, waves 2 (M) x 2 (N), whole K per wave: shapes with many tiles.
+//   gemm_spk_kernel    128x256 tile (one per CU at M = 2048, N = 4096), waves 2 (N) x 2 (K): the two
+//                      K-groups take alternate pairs of sub-steps and exchange half of their
+//                      accumulators through LDS at the end.
 template <bool DEQ, bool RAGGED>
 __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
@@ -1130,26 +907,292 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     }
 }
 
-int launch_sp(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
-              const void* bias, hipStream_t st) {
+template <bool DEQ, bool RAGGED>
+__global__ __launch_bounds__(256) void gemm_spk_kernel(
+    const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
+    f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
+    int tiles_m, int tiles_n) {
+    constexpr int BM = 128, BN = 256, NT = 256;
+    constexpr int TM = 128, TN = 128, IM = 4, JN = 4;
+    constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
+    constexpr int NL = CH / NT;                             // 12 per thread
+    constexpr int NF = IM + JN;                             // fragments per sub-step
+    constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
+    constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
+    constexpr int S0 = 8;                                   // first slot that unpacks (LDS reads issued in slots 0..7)
+    extern __shared__ u32x4 spk_lds[];                       // [2][CH]; later the output slabs
+
+    const int nxcd = 8;
+    const int per_xcd = gridDim.x / nxcd;
+    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (tile >= tiles_m * tiles_n) return;
+    constexpr int GROUP_M = 8;
+    const int group_sz = GROUP_M * tiles_n;
+    const int g = tile / group_sz;
+    const int gm0 = g * GROUP_M;
+    const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
+    const int tm = gm0 + (tile - g * group_sz) % gh;
+    const int tn = (tile - g * group_sz) / gh;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = 0, wn = wave & 1, kg = wave >> 1;        // K-group kg multiplies sub-steps 2 kg and 2 kg + 1 of every stage
+    const int khalf = lane >> 5;
+    const int stages = (Kb + 127) / 128;
+    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
+
+    // staging: chunk id = tid + i * 256: row = tid / 8 + 32 i, piece tid % 8
+    const int srow = tid >> 3;
+    const int scoff = (tid & 7) * 16;
+    const int dst0 = slot8(srow, tid & 7);                  // rows differ by multiples of 32: same swizzle key
+    u32 goff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int row = srow + i * 32;
+        int gr = row < BM ? m0 + row : n0 + row - BM;
+        const int lim = row < BM ? M - 1 : N - 1;
+        gr = gr < lim ? gr : lim;
+        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
+    }
+    u32x4 regs[2][NL];                                      // two sets: loads run two stages ahead of their LDS write
+    // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
+    // buffer load: scalar descriptor + scalar stage offset + constant 32-bit per-thread offset, so
+    // the address costs no vector instruction and half the address traffic of a 64-bit pointer.
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)((u32)M * (u32)Kb), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (int)((u32)N * (u32)Kb), 0x00020000);
+    auto fetch1 = [&](int st, int set, int i) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        u32 off = goff[i];
+        if (RAGGED) off += (u32)((kb + scoff < Kb) ? scoff : 0);
+        regs[set][i] = (i * 32 < BM) ? __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, kb, 0)
+                                     : __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, off, kb, 0);
+    };
+    auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
+        const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
+        spk_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
+    };
+
+    i32x16 acc[IM][JN];
+#pragma unroll
+    for (int i = 0; i < IM; ++i)
+#pragma unroll
+        for (int j = 0; j < JN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+    // fragment slots of this wave's two sub-steps u0 = 2 kg, u1 = 2 kg + 1: logical chunk 2 u + khalf
+    const int u0 = 2 * kg, u1 = 2 * kg + 1;
+    const int aslot0 = slot8(wm * TM + (lane & 31), 2 * u0 + khalf), aslot1 = slot8(wm * TM + (lane & 31), 2 * u1 + khalf);
+    const int bslot0 = slot8(BM + wn * TN + (lane & 31), 2 * u0 + khalf), bslot1 = slot8(BM + wn * TN + (lane & 31), 2 * u1 + khalf);
+    // fragments: index 0..1 = A (32-row tiles of the wave tile), 2..5 = B
+    struct Packed {
+        u32x4 f[IM + JN];
+    };
+    struct Ops {
+        i32x4 lo[IM + JN], hi[IM + JN];
+    };
+    // K-group 1 holds its B fragments (and so its accumulator columns) with the two 64-column halves
+    // swapped: either group then KEEPS accumulator tiles j = 0, 1 and SENDS j = 2, 3, with
+    // compile-time register indices on both sides
+    const int bswap = kg * 64 * 8;                          // LDS offset of 64 rows
+    auto read1 = [&](int buf, int second, int r, Packed& p) {  // second: sub-step u1 rather than u0
+        const int as = second ? aslot1 : aslot0, bs = second ? bslot1 : bslot0;
+        if (r < IM) p.f[r] = spk_lds[buf * CH + as + r * 32 * 8];
+        else p.f[r] = spk_lds[buf * CH + bs + ((r - IM) * 32 * 8 ^ bswap)];
+    };
+    // unpacking as UNP single instructions: dword d = n / 3 of the packed dwords,
+    // n % 3 = 0: lo = p << 4;  1: lo &= mask;  2: hi = p & mask
+    auto unpack1 = [&](const Packed& p, Ops& o, int n) {
+        const int d = n / 3, f = d >> 2, e = d & 3, kind = n % 3;
+        if (kind == 0) o.lo[f][e] = (int)(p.f[f][e] << 4);
+        else if (kind == 1) o.lo[f][e] = o.lo[f][e] & (int)0xF0F0F0F0u;
+        else o.hi[f][e] = (int)(p.f[f][e] & 0xF0F0F0F0u);
+    };
+    auto mfma1 = [&](const Ops& o, int q) {
+        const int t = q % (IM * JN), i = t / JN, j = t % JN;
+        if (q < IM * JN) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.lo[IM + j], o.lo[i], acc[i][j], 0, 0, 0);
+        else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.hi[IM + j], o.hi[i], acc[i][j], 0, 0, 0);
+    };
+    // One 64-k sub-step = NMF = 32 slots.  Slot q: MFMA q of the current operands; slots 0..7 read
+    // the packed fragments of this wave's NEXT sub-step (one fragment buffer), slots S0.. unpack
+    // them (4 instructions per slot); in a stage's first sub-step, slots 2.. also write one chunk
+    // of stage ks+1 to LDS and request the same chunk of stage ks+2.  A full scheduling barrier
+    // after every slot keeps this order.
+#define QR_SPK_SUBSTEP(CUR, NXT, RBUF, RU, DEP, SET)                                             \
+    _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
+        mfma1(CUR, q_);                                                                          \
+        if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
+        if (q_ >= S0) {                                                                          \
+            _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
+                unpack1(pk, NXT, n_);                                                            \
+        }                                                                                        \
+        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
+            deposit1(ks_ + 1, nb_, SET, q_ - 2);                                                 \
+            fetch1(ks_ + 3, SET, q_ - 2);                                                        \
+        }                                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    }
+    // one stage: KS = stage index, B = its LDS buffer (compile-time), SET = register set that holds
+    // stage KS+1 on entry and receives stage KS+3
+#define QR_SPK_STAGE(KS, B, SET)                                                                 \
+    {                                                                                            \
+        const int ks_ = (KS);                                                                    \
+        constexpr int b_ = (B), nb_ = 1 - (B);                                                   \
+        /* first sub-step: multiply (ks,u0); read + unpack (ks,u1); stage ks+1 -> LDS, request ks+3 */ \
+        QR_SPK_SUBSTEP(ops[0], ops[1], b_, 1, true, SET)                                         \
+        __syncthreads(); /* stage ks+1 visible; stage ks fully read */                           \
+        /* second sub-step: multiply (ks,u1); read + unpack (ks+1,u0) */                         \
+        QR_SPK_SUBSTEP(ops[1], ops[0], nb_, 0, false, SET)                                       \
+    }
+
+    // prologue: stage 0 into LDS, stages 1 and 2 requested; this wave's first sub-step unpacked
+    Packed pk;
+    Ops ops[2];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(2, 1, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) deposit1(0, 0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NL; ++i) fetch1(1, 0, i);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NF; ++r) read1(0, 0, r, pk);
+#pragma unroll
+    for (int n = 0; n < UNP; ++n) unpack1(pk, ops[0], n);
+    // (pairs of stages without a branch in between: the wait before an LDS write then counts the
+    // other set's loads as still allowed in flight)
+    int ks = 0;
+    for (; ks + 1 < stages; ks += 2) {
+        QR_SPK_STAGE(ks, 0, 0)
+        QR_SPK_STAGE(ks + 1, 1, 1)
+    }
+    if (ks < stages) QR_SPK_STAGE(ks, 0, 0)
+#undef QR_SPK_STAGE
+#undef QR_SPK_SUBSTEP
+
+    // K-split: the two K-groups hold partial sums of the same 128x128 wave tile.  Each finalises the
+    // 64 output columns held in its accumulator tiles j = 0, 1 (group 0: columns 0..63 of the wave
+    // tile, group 1: 64..127) and sends tiles j = 2, 3 across through LDS, two 32-row tiles (i) per
+    // round, four 16-byte pieces per lane and tile.
+    {
+        u32x4* xbuf = spk_lds;
+#pragma unroll
+        for (int ip = 0; ip < IM; ip += 2) {
+            __syncthreads();
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int qv = 0; qv < 4; ++qv) {
+                        const i32x16& t = acc[ip + ii][2 + jj];
+                        xbuf[((((wn * 2 + (1 - kg)) * 2 + ii) * 2 + jj) * 4 + qv) * 64 + lane] =
+                            u32x4{(u32)t[qv * 4], (u32)t[qv * 4 + 1], (u32)t[qv * 4 + 2], (u32)t[qv * 4 + 3]};
+                    }
+            __syncthreads();
+#pragma unroll
+            for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int qv = 0; qv < 4; ++qv) {
+                        const u32x4 piece = xbuf[((((wn * 2 + kg) * 2 + ii) * 2 + jj) * 4 + qv) * 64 + lane];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[ip + ii][jj][qv * 4 + e] += (int)piece[e];
+                    }
+        }
+    }
+    __syncthreads();                                        // stage buffers free for the output slabs
+
+    // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
+    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    if (DEQ && by_rows) {
+        const int jb = 2 * kg;
+        {
+            f16x4 sbh[2][4], bih[2][4];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
+                    sbh[jj][gq] = *(const f16x4*)(sB + col);
+                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                }
+#pragma unroll
+            for (int i = 0; i < IM; ++i) {
+                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                f16x4 o[2][4];
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jj][gq * 4 + e] >> 8);
+                            if (bias) yv = yv + bih[jj][gq][e];
+                            o[jj][gq][e] = yv;
+                        }
+                store_slab_rows<2>((u32x2*)(spk_lds + wave * 256), o, lane,
+                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < IM; ++i) {
+        const int row = m0 + wm * TM + i * 32 + (lane & 31);
+        if (row >= M) continue;
+        f16 sa = (f16)0;
+        if (DEQ) sa = sA[row];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {                       // this K-group's tiles: output column tiles j + 2 kg
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = n0 + wn * TN + (j + 2 * kg) * 32 + gq * 8 + khalf * 4;
+                if (col >= N) continue;
+                int v4[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v4[e] = acc[i][j][gq * 4 + e] >> 8;
+                if (DEQ) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (col + e < N) {
+                            f16 yv = (f16)(sa * sB[col + e]) * (f16)(float)v4[e];
+                            if (bias) yv = yv + bias[col + e];
+                            Y[(int64_t)row * N + col + e] = yv;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) C[(int64_t)row * N + col + e] = v4[e];
+                }
+            }
+        }
+    }
+}
+
+int launch_spk(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
+               const void* bias, hipStream_t st) {
     constexpr size_t LDS = (size_t)2 * (128 + 256) * 8 * 16;
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     const bool ragged = (Kb & 127) != 0;
-    // operands are addressed through 32-bit buffer offsets
     if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
         return launch_ks<128, 256, 2, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
     hipError_t e;
     if (Y) {
-        auto kern = ragged ? gemm_sp_kernel<true, true> : gemm_sp_kernel<true, false>;
+        auto kern = ragged ? gemm_spk_kernel<true, true> : gemm_spk_kernel<true, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
                                                  (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
     } else {
-        auto kern = ragged ? gemm_sp_kernel<false, true> : gemm_sp_kernel<false, false>;
+        auto kern = ragged ? gemm_spk_kernel<false, true> : gemm_spk_kernel<false, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
@@ -1561,7 +1604,7 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         const double rounds256 = (double)((t256 + 255) / 256);
         const double rounds128 = (double)((t128x256 + 255) / 256) * 0.61;
         if (rounds256 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
-        return launch_sp(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        return launch_spk(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     if (N > 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
