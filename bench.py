@@ -51,9 +51,9 @@ HBM_PEAK_GBS = 8000.0
 FETCH_SCALE, WRITE_SCALE = 262144.0 / 131083.8, 262144.0 / 262144.0
 TRAFFIC_KIB = {
     #        FETCH_SIZE   WRITE_SIZE
-    "c1": (16568.9, 16384.0),
-    "c2": (44236.7, 16384.0),
-    "c3d": (528728.3, 262144.0),
+    "c1": (16566.0, 16384.0),
+    "c2": (44225.0, 16384.0),
+    "c3d": (528828.0, 262144.0),
     "c4": (72440.1, 1024.0),
     "c4m1": (61875.4, 16.0),
     "c4g64": (115876.5, 7168.0),
@@ -213,10 +213,17 @@ def main():
         roof = {"bound": "mfma", "achieved": round(ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
                 "unit": "TFLOP/s", "traffic": traffic}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = ("gemv_i4_kernel" if m <= 4 else
-                      ("gemm_ks_kernel<64,256>" if (n + 255) // 256 >= 128 else "decode_i4_kernel") if decode else
-                      "gemm_i4_kernel<256,256>" if ((m + 255) // 256) * ((n + 255) // 256) >= 512 else
-                      "gemm_sp_kernel" if ((m + 127) // 128) * ((n + 255) // 256) >= 128 else "gemm_ks_kernel<64,256>")
+    t256 = ((m + 255) // 256) * ((n + 255) // 256)
+    t128 = ((m + 127) // 128) * ((n + 255) // 256)
+    if m <= 4:
+        kern = "gemv_i4_kernel"
+    elif decode:
+        kern = "gemm_ks_kernel<64,256>" if (n + 255) // 256 >= 128 else "decode_i4_kernel"
+    elif t128 >= 128:       # the library's choice between its two pipelined kernels, by rounds of tiles
+        kern = "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
+    else:
+        kern = "gemm_ks_kernel<64,256>"
+    roof["kernel"] = kern
     roof["kernel"] += " (int4 GEMM + dequant epilogue)"
     roof["kernel_ms"] = round(gemm_ms, 4)
 
