@@ -132,7 +132,9 @@ def test_sym_quant_odd_columns_and_views():
 
 GEMM_SHAPES = [(1, 1, 64), (32, 32, 64), (33, 65, 128), (64, 64, 192), (100, 200, 192), (128, 128, 256), (1, 256, 4096),
                (8, 300, 1024), (40, 512, 512), (64, 1000, 2048), (65, 256, 320), (129, 257, 448), (256, 512, 4096),
-               (300, 700, 11008), (512, 1024, 2048), (1000, 3000, 1024), (2048, 4096, 4096)]
+               (300, 700, 11008), (512, 1024, 2048), (1000, 3000, 1024), (2048, 4096, 4096),
+               # the pipelined kernels: whole and partly filled K stages, whole and ragged tiles
+               (2048, 4096, 320), (2050, 4100, 448), (4096, 4096, 256), (4090, 4090, 192), (2304, 8192, 64)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -175,7 +177,8 @@ def test_sym_dequant_bit_exact(rows, cols):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (33, 65, 128), (64, 512, 1024), (100, 200, 192), (300, 700, 11008),
-                                   (512, 1024, 2048), (2048, 4096, 4096)])
+                                   (512, 1024, 2048), (2048, 4096, 4096), (2048, 4096, 320), (2050, 4100, 448),
+                                   (4096, 4096, 256), (4090, 4096, 192)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_linear_fused_equals_staged_reference_ops(m, n, k, with_bias):
     rng = np.random.default_rng(m + n + k)
