@@ -615,10 +615,12 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
             u32x4 hi, lo;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const f16 h0 = narrow_f16(t[2 * e]), h1 = narrow_f16(t[2 * e + 1]);
-                hi[e] = (u32)f16_bits(h0) | ((u32)f16_bits(h1) << 16);
-                if (MODE32)
-                    lo[e] = (u32)f16_bits((f16)(t[2 * e] - (float)h0)) | ((u32)f16_bits((f16)(t[2 * e + 1] - (float)h1)) << 16);
+                const u32 hw = narrow_f16x2(t[2 * e], t[2 * e + 1]);
+                hi[e] = hw;
+                if (MODE32) {
+                    const f16x2 h = as_f16x2(hw);
+                    lo[e] = narrow_f16x2(t[2 * e] - (float)h[0], t[2 * e + 1] - (float)h[1]);
+                }
             }
             const int slot = ((wave + 4 * c) * KS2 + s2) * 64 + lane;
             Tl[slot] = hi;
@@ -700,8 +702,8 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
                     const int kp = rt * 16 + l16;
                     if (kp < K) {
                         u32x2 o;
-                        o[0] = (u32)f16_bits((f16)acc[0]) | ((u32)f16_bits((f16)acc[1]) << 16);
-                        o[1] = (u32)f16_bits((f16)acc[2]) | ((u32)f16_bits((f16)acc[3]) << 16);
+                        o[0] = narrow_f16x2(acc[0], acc[1]);
+                        o[1] = narrow_f16x2(acc[2], acc[3]);
                         *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
                         if (QUANT) {
                             mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & 0x7fff7fffu));
@@ -934,8 +936,8 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                     const int kp = rt * 16 + l16;
                     if (kp < K) {
                         u32x2 o;
-                        o[0] = (u32)f16_bits((f16)acc[0]) | ((u32)f16_bits((f16)acc[1]) << 16);
-                        o[1] = (u32)f16_bits((f16)acc[2]) | ((u32)f16_bits((f16)acc[3]) << 16);
+                        o[0] = narrow_f16x2(acc[0], acc[1]);
+                        o[1] = narrow_f16x2(acc[2], acc[3]);
                         *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
                     }
                 }
