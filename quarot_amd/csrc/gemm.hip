@@ -64,6 +64,22 @@ __device__ __forceinline__ void store_slab_rows(u32x2* region, const f16x4 (&o)[
     }
 }
 
+// Four dequantised outputs of one row: fp16( fp16(sa * sb) * fp16(acc >> 8) ) (+ bias), the three
+// (four) fp16 operations as packed instructions on column pairs -- each lane of a packed fp16
+// multiply or add rounds exactly like the scalar instruction.
+__device__ __forceinline__ f16x4 dequant4(int a0, int a1, int a2, int a3, f16 sa, f16x4 sb, f16x4 bi, bool with_bias) {
+    const f16x2 s2 = {sa, sa};
+    const f16x2 q01 = as_f16x2(narrow_f16x2((float)(a0 >> 8), (float)(a1 >> 8)));
+    const f16x2 q23 = as_f16x2(narrow_f16x2((float)(a2 >> 8), (float)(a3 >> 8)));
+    f16x2 y01 = (s2 * f16x2{sb[0], sb[1]}) * q01;
+    f16x2 y23 = (s2 * f16x2{sb[2], sb[3]}) * q23;
+    if (with_bias) {
+        y01 = y01 + f16x2{bi[0], bi[1]};
+        y23 = y23 + f16x2{bi[2], bi[3]};
+    }
+    return f16x4{y01[0], y01[1], y23[0], y23[1]};
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
@@ -236,7 +252,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
                 for (int gq = 0; gq < 4; ++gq) {
                     const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
                     sbh[jj][gq] = *(const f16x4*)(sB + col);
-                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                    bih[jj][gq] = bias ? *(const f16x4*)(bias + col) : f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
@@ -246,12 +262,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
                 for (int jj = 0; jj < NJ; ++jj)
 #pragma unroll
                     for (int gq = 0; gq < 4; ++gq)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
-                            if (bias) yv = yv + bih[jj][gq][e];
-                            o[jj][gq][e] = yv;
-                        }
+                        o[jj][gq] = dequant4(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
+                                             acc[i][jb + jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<NJ>((u32x2*)(lds_raw + wave * SLAB), o, lane,
                                     Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
             }
@@ -851,7 +863,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
                 for (int gq = 0; gq < 4; ++gq) {
                     const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
                     sbh[jj][gq] = *(const f16x4*)(sB + col);
-                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                    bih[jj][gq] = bias ? *(const f16x4*)(bias + col) : f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
@@ -861,12 +873,8 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
                 for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                     for (int gq = 0; gq < 4; ++gq)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jb + jj][gq * 4 + e] >> 8);
-                            if (bias) yv = yv + bih[jj][gq][e];
-                            o[jj][gq][e] = yv;
-                        }
+                        o[jj][gq] = dequant4(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
+                                             acc[i][jb + jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<2>((u32x2*)(sp2_lds + wave * 256), o, lane,
                                    Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
             }
@@ -1118,7 +1126,7 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
                 for (int gq = 0; gq < 4; ++gq) {
                     const int col = n0 + wn * TN + (jb + jj) * 32 + gq * 8 + khalf * 4;
                     sbh[jj][gq] = *(const f16x4*)(sB + col);
-                    if (bias) bih[jj][gq] = *(const f16x4*)(bias + col);
+                    bih[jj][gq] = bias ? *(const f16x4*)(bias + col) : f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
@@ -1128,12 +1136,8 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
                 for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                     for (int gq = 0; gq < 4; ++gq)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            f16 yv = (f16)(sa * sbh[jj][gq][e]) * (f16)(float)(acc[i][jj][gq * 4 + e] >> 8);
-                            if (bias) yv = yv + bih[jj][gq][e];
-                            o[jj][gq][e] = yv;
-                        }
+                        o[jj][gq] = dequant4(acc[i][jj][gq * 4], acc[i][jj][gq * 4 + 1], acc[i][jj][gq * 4 + 2],
+                                             acc[i][jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<2>((u32x2*)(spk_lds + wave * 256), o, lane,
                                    Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
             }
