@@ -711,7 +711,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     constexpr int NF = IM + JN;                             // fragments per sub-step
     constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
     constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
-    constexpr int S0 = 8;                                   // first slot that unpacks (LDS reads issued in slots 0..7)
+    constexpr int S0 = 4;                                   // first slot that unpacks (LDS reads are issued in slots 0..7, in fragment order)
     extern __shared__ u32x4 sp2_lds[];                       // [2][CH]; later the output slabs
 
     const int nxcd = 8;
@@ -815,9 +815,9 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
             _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
                 unpack1(pk, NXT, n_);                                                            \
         }                                                                                        \
-        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
-            deposit1(ks + 1, nb, 0, q_ - 2);                                                     \
-            fetch1(ks + 2, 0, q_ - 2);                                                           \
+        if ((DEP) && q_ >= 8 && q_ < 8 + NL) {                                                   \
+            deposit1(ks + 1, nb, 0, q_ - 8);                                                     \
+            fetch1(ks + 2, 0, q_ - 8);                                                           \
         }                                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     }
@@ -927,7 +927,7 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     constexpr int NF = IM + JN;                             // fragments per sub-step
     constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
     constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
-    constexpr int S0 = 8;                                   // first slot that unpacks (LDS reads issued in slots 0..7)
+    constexpr int S0 = 4;                                   // first slot that unpacks (LDS reads are issued in slots 0..7, in fragment order)
     extern __shared__ u32x4 spk_lds[];                       // [2][CH]; later the output slabs
 
     const int nxcd = 8;
@@ -1034,9 +1034,9 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
             _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
                 unpack1(pk, NXT, n_);                                                            \
         }                                                                                        \
-        if ((DEP) && q_ >= 2 && q_ < 2 + NL) {                                                   \
-            deposit1(ks_ + 1, nb_, SET, q_ - 2);                                                 \
-            fetch1(ks_ + 3, SET, q_ - 2);                                                        \
+        if ((DEP) && q_ >= 8 && q_ < 8 + NL) {                                                   \
+            deposit1(ks_ + 1, nb_, SET, q_ - 8);                                                 \
+            fetch1(ks_ + 3, SET, q_ - 8);                                                        \
         }                                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     }
