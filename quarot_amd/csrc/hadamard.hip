@@ -764,6 +764,266 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
     }
 }
 
+// ---- K > 1, m = 64, fp16 I/O: the same two matrix-core stages, organised for latency ------------
+// hadamard_mm_kernel above is bound by exposed latencies (every LDS read, dependent MFMA chain and
+// conversion waits for the one before it) and reads the staged input four times.  Here
+//   * a wave owns whole 16-row tiles of X (tile t = wave + 4 i): it fetches them with coalesced
+//     16-byte loads one row ahead, stages them in a wave-private LDS region (no workgroup barrier:
+//     LDS operations of one wave execute in order) and reads its stage-1 fragments from there, so X
+//     is read from LDS once; all column tiles of T for these rows come from eight Sylvester
+//     fragments held in registers;
+//   * T is kept as [column tile][16-row tile][lane] 8-byte halves: stage 1 writes 8 contiguous bytes
+//     per lane, stage 2 assembles a 32-deep fragment from two of them;
+//   * stage 2 fetches the fragments of the next column tile while the MFMAs of the current one run,
+//     all hadK tiles of a wave are independent accumulator chains in one basic block (rows of hadK
+//     beyond K are zero fragments and produce zero rows of Y: no branches), stage 3 issues all its
+//     LDS reads before the first conversion.
+// Two workgroup barriers per row.
+template <bool MODE32, bool QUANT, int KS2>
+__global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
+    const f16* __restrict__ x, f16* __restrict__ y, int64_t rows, int n, int K, const void* __restrict__ hadK,
+    float scale, float clip, u32* __restrict__ q, f16* __restrict__ scales) {
+    constexpr int CT = 4;                        // 16-column tiles of T / Y
+    constexpr int YS = 64 + 8;                   // halves per row of Yl
+    constexpr int NT = 2 * KS2;                  // 16-row tiles of X / T / hadK (order padded to 32 KS2)
+    constexpr int TPW = (NT + 3) / 4;            // tiles per wave
+    constexpr int YROWS = TPW * 64;              // every wave writes TPW full tiles of Y
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[HT / QR_WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int nchunks = n >> 3;
+    u32x2* Tl = (u32x2*)smem_raw;                                      // [CT][NT][64 lanes], hi plane
+    u32x2* Tlo = Tl + CT * NT * 64;                                    // lo plane (fp32 mode)
+    f16* Yl = (f16*)(Tl + (MODE32 ? 2 : 1) * CT * NT * 64);            // [YROWS][YS]
+    u32x4* Xs = (u32x4*)(Yl + YROWS * YS) + wave * (TPW * 128);        // wave-private [TPW][16 rows][8 pieces]
+
+    // T slots of tiles beyond K and staged rows beyond K are never written afterwards: clear once
+    for (int i = tid; i < (MODE32 ? 2 : 1) * CT * NT * 32; i += HT) ((u32x4*)Tl)[i] = u32x4{0, 0, 0, 0};
+    for (int i = lane; i < TPW * 128; i += QR_WAVE) Xs[i] = u32x4{0, 0, 0, 0};
+
+    // hadK fragments of this wave's tiles (second MFMA operand of stage 2), contraction index in
+    // the order k = 32 s + 16 (j / 4) + 4 (lane / 16) + j % 4
+    f16x8 hf[TPW][KS2];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        const int hr = (wave + 4 * t) * 16 + l16;
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int hc = ks * 32 + hh * 16 + g * 4;
+                f16x4 v = {(f16)0, (f16)0, (f16)0, (f16)0};
+                if (hr < K && hc < K) {
+                    if (hadK == nullptr) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = (__builtin_popcount(hr & (hc + e)) & 1) ? (f16)-1.0f : (f16)1.0f;
+                    } else if (MODE32) {
+                        const f32x4 w = *(const f32x4*)((const float*)hadK + hr * K + hc);
+                        v = f16x4{(f16)w[0], (f16)w[1], (f16)w[2], (f16)w[3]};
+                    } else {
+                        v = *(const f16x4*)((const f16*)hadK + hr * K + hc);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hf[t][ks][hh * 4 + e] = v[e];
+            }
+    }
+    // Sylvester fragments of all four column tiles: H_64[r][r'] = (-1)^popcount(r & r')
+    f16x8 b1[CT][2];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                b1[ct][ks][j] = (__builtin_popcount((ks * 32 + g * 8 + j) & (ct * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+
+    // staging: load c of a tile covers its rows 8 c .. 8 c + 7, lane -> (row 8 c + lane / 8, piece
+    // lane % 8): 1 KB of consecutive addresses per instruction.  Pieces are XOR-keyed by the row so
+    // that the sixteen rows of a fragment read fall into sixteen different bank groups.
+    int dslot[2], rslot[2], goff[TPW][2];
+    bool dval[TPW][2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const int rc = c * 8 + (lane >> 3);
+        dslot[c] = rc * 8 + ((lane & 7) ^ ((rc >> 1) & 7));
+        rslot[c] = l16 * 8 + ((c * 4 + g) ^ ((l16 >> 1) & 7));
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            dval[i][c] = (wave + 4 * i) * 16 + rc < K;
+            goff[i][c] = dval[i][c] ? (wave + 4 * i) * 128 + c * 64 + lane : 0;
+        }
+    }
+    u32x4 xr[TPW][2];
+    auto load_row = [&](const f16* src) {
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) xr[i][c] = *((const u32x4*)src + goff[i][c]);
+    };
+
+    int64_t row = blockIdx.x;
+    if (row < rows) load_row(x + row * (int64_t)n);
+    // the hadK fragments must have arrived before the loop: otherwise their first use in every
+    // iteration would also wait for the row just requested
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks) asm volatile("" : "+v"(hf[t][ks]));
+    __syncthreads();
+    for (; row < rows; row += gridDim.x) {
+        const int64_t nrow = row + gridDim.x;
+        // ---- stage 1: T = X . H_64 for this wave's tiles
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+                if (dval[i][c]) Xs[i * 128 + dslot[c]] = xr[i][c];
+        if (nrow < rows) load_row(x + nrow * (int64_t)n);
+        u32x4 af[TPW][2];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) af[i][ks] = Xs[i * 128 + rslot[ks]];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int t = wave + 4 * i;
+            if (4 * i + 3 < NT || t < NT) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][0]), b1[ct][0], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][1]), b1[ct][1], acc, 0, 0, 0);
+                    float tv[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) tv[e] = acc[e] * scale;
+                    u32x2 hi, lo;
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const u32 hw = narrow_f16x2(tv[2 * e], tv[2 * e + 1]);
+                        hi[e] = hw;
+                        if (MODE32) {
+                            const f16x2 h = as_f16x2(hw);
+                            lo[e] = narrow_f16x2(tv[2 * e] - (float)h[0], tv[2 * e + 1] - (float)h[1]);
+                        }
+                    }
+                    Tl[(ct * NT + t) * 64 + lane] = hi;
+                    if (MODE32) Tlo[(ct * NT + t) * 64 + lane] = lo;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- stage 2: Y^T = T^T . hadK^T (the row's abs-max is taken from the rounded results)
+        u16x2 mx2 = {0, 0};
+        u32x4 th[2][KS2], tlo[2][KS2];
+        auto fetch = [&](int ct, int b) {
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                const u32x2 p0 = Tl[(ct * NT + 2 * ks) * 64 + lane], p1 = Tl[(ct * NT + 2 * ks + 1) * 64 + lane];
+                th[b][ks] = u32x4{p0[0], p0[1], p1[0], p1[1]};
+                if (MODE32) {
+                    const u32x2 r0 = Tlo[(ct * NT + 2 * ks) * 64 + lane], r1 = Tlo[(ct * NT + 2 * ks + 1) * 64 + lane];
+                    tlo[b][ks] = u32x4{r0[0], r0[1], r1[0], r1[1]};
+                }
+            }
+        };
+        fetch(0, 0);
+        f16* ybase = Yl + (wave * 16 + l16) * YS + g * 4;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ct + 1 < CT) fetch(ct + 1, (ct + 1) & 1);
+            f32x4 acc[TPW];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, th[ct & 1][ks]), hf[i][ks], acc[i], 0, 0, 0);
+                    if (MODE32)
+                        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, tlo[ct & 1][ks]), hf[i][ks], acc[i], 0, 0, 0);
+                }
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                u32x2 o;
+                o[0] = narrow_f16x2(acc[i][0], acc[i][1]);
+                o[1] = narrow_f16x2(acc[i][2], acc[i][3]);
+                *(u32x2*)(ybase + i * 64 * YS + ct * 16) = o;
+                if (QUANT) {
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & 0x7fff7fffu));
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[1] & 0x7fff7fffu));
+                }
+            }
+        }
+        u32 mx = 0;
+        if (QUANT) {
+            mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            mx = wave_max_u32_dpp(mx);
+            if (lane == 0) red[wave] = mx;
+        }
+        __syncthreads();
+        // ---- stage 3
+        if (QUANT) {
+#pragma unroll
+            for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+            const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+            const float s = (float)sh;
+            // units of 16 elements (two chunks): 8-byte stores of codes
+            constexpr int NUI = (KS2 + 1) / 2;
+            const int nunits = nchunks >> 1;
+            u32x2* qrow = (u32x2*)(q + row * (int64_t)nchunks);
+            int un[NUI];
+            u32x4 h[NUI][2];
+#pragma unroll
+            for (int j = 0; j < NUI; ++j) {
+                const int u = tid + j * HT;
+                un[j] = u < nunits ? u : nunits - 1;
+                const f16* src = Yl + (un[j] >> 2) * YS + (un[j] & 3) * 16;
+                h[j][0] = *(const u32x4*)src;
+                h[j][1] = *(const u32x4*)(src + 8);
+            }
+            u32x2 codes[NUI];
+            if (fast_quant_ok(mx, s)) {
+                const FastRecip fq = make_fast_recip(s);
+#pragma unroll
+                for (int j = 0; j < NUI; ++j) codes[j] = u32x2{sym_codes8_fast(h[j][0], fq), sym_codes8_fast(h[j][1], fq)};
+            } else {
+                const bool fast = scale_fast_ok(s);
+                const float rs = fast ? 1.0f / s : 0.0f;
+#pragma unroll
+                for (int j = 0; j < NUI; ++j) codes[j] = u32x2{sym_codes8(h[j][0], s, rs, fast), sym_codes8(h[j][1], s, rs, fast)};
+            }
+            // Stores without conditions (threads past the end of the row repeat the last unit, same
+            // value): the number of stores in flight is then known when the next row's loads are
+            // awaited, and that wait need not include them.
+#pragma unroll
+            for (int j = 0; j < NUI; ++j) qrow[un[j]] = codes[j];
+            scales[row] = sh;
+            if (y) {
+#pragma unroll
+                for (int j = 0; j < NUI; ++j) {
+                    __builtin_nontemporal_store(h[j][0], (u32x4*)(y + row * (int64_t)n) + 2 * un[j]);
+                    __builtin_nontemporal_store(h[j][1], (u32x4*)(y + row * (int64_t)n) + 2 * un[j] + 1);
+                }
+            }
+        } else {
+            u32x4 h[KS2];
+            int cn[KS2];
+#pragma unroll
+            for (int j = 0; j < KS2; ++j) {
+                const int c = tid + j * HT;
+                cn[j] = c < nchunks ? c : nchunks - 1;
+                h[j] = *(const u32x4*)(Yl + (cn[j] >> 3) * YS + (cn[j] & 7) * 8);
+            }
+#pragma unroll
+            for (int j = 0; j < KS2; ++j) __builtin_nontemporal_store(h[j], (u32x4*)(y + row * (int64_t)n) + cn[j]);
+        }
+        // Tl is next written after this barrier, Yl after the next row's first barrier, red[] after
+        // it as well: every reader of this row has passed by then
+    }
+}
+
 // A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
 // kernel applies with a generated outer factor, in its fp32-precision mode so that the result is
 // rounded to fp16 once, like a plain fp32 transform.  Returns the outer order (0: not applicable).
@@ -773,7 +1033,7 @@ int pow2_split(int n) {
 }
 
 bool mm_applies(int n, int K) {
-    if (K <= 1 || K > 32 * KS_MAX) return false;
+    if (K <= 1 || K > 32 * KS_MAX || (K & 3) != 0) return false;     // hadK is fetched four columns at a time
     const int m = n / K;
     return m == 64 || m == 128;
 }
@@ -783,6 +1043,35 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
                        void* q, void* scales, hipStream_t st) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
+    if (m == 64) {
+        // the latency-organised kernel, while two workgroups still fit on a CU
+        const int tpw = (2 * KS2 + 3) / 4;
+        const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
+        if (lds64 <= 80 * 1024) {
+#define QR_M64(KS)                                                                                                     \
+    do {                                                                                                               \
+        auto kern = hadamard_m64_kernel<MODE32, QUANT, KS>;                                                            \
+        if (lds64 > 48 * 1024) {                                                                                       \
+            hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds64);                                             \
+            if (e != hipSuccess) return (int)e;                                                                        \
+        }                                                                                                              \
+        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds64);                                    \
+        const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
+        kern<<<dim3(grid), dim3(HT), lds64, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,      \
+                                                  (f16*)scales);                                                       \
+    } while (0)
+            switch (KS2) {
+                case 1: QR_M64(1); break;
+                case 2: QR_M64(2); break;
+                case 3: QR_M64(3); break;
+                case 4: QR_M64(4); break;
+                case 5: QR_M64(5); break;
+                default: QR_M64(6); break;
+            }
+#undef QR_M64
+            return qr_launch_status();
+        }
+    }
     const size_t lds0 = (size_t)(MODE32 ? 2 : 1) * (m / 16) * KS2 * 64 * 16 + (((size_t)K * (m + 8) + 7) & ~(size_t)7) * 2;
     const size_t lds_x = lds0 + (size_t)KS2 * 32 * m * 2;
     // the staged-input form when at least two workgroups still fit on a CU
@@ -981,7 +1270,7 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
 }
 
 bool bm_applies(int n, int K) {
-    if (K <= 1) return false;
+    if (K <= 1 || (K & 3) != 0) return false;                        // hadK is fetched four columns at a time
     const int m = n / K;
     return (m == 512 && K <= 64) || (m == 1024 && K <= 32);
 }

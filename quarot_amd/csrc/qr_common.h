@@ -124,6 +124,25 @@ __device__ __forceinline__ u32 wave_max_u32(u32 v) {
     return v;
 }
 
+// The same maximum without LDS round trips: four DPP steps reduce each row of 16 lanes (every lane
+// of a row ends with the row's maximum), four lane reads and scalar maxima combine the rows.  The
+// result is wave-uniform.
+__device__ __forceinline__ u32 wave_max_u32_dpp(u32 v) {
+    int o;
+    o = __builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);     // quad_perm [1,0,3,2]
+    v = v > (u32)o ? v : (u32)o;
+    o = __builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);     // quad_perm [2,3,0,1]
+    v = v > (u32)o ? v : (u32)o;
+    o = __builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);    // row_half_mirror
+    v = v > (u32)o ? v : (u32)o;
+    o = __builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);    // row_mirror
+    v = v > (u32)o ? v : (u32)o;
+    const u32 r0 = (u32)__builtin_amdgcn_readlane((int)v, 0), r1 = (u32)__builtin_amdgcn_readlane((int)v, 16);
+    const u32 r2 = (u32)__builtin_amdgcn_readlane((int)v, 32), r3 = (u32)__builtin_amdgcn_readlane((int)v, 48);
+    const u32 a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
+}
+
 // Quantiser scale: fp16( float(fp16(amax / 7)) * clip ), each step correctly rounded.  amax / 7
 // never lies on (or within 2^-14 relative of) an fp16 rounding boundary: a boundary (i + 1/2) ulp
 // would need amax = 7 i + 3.5 units of its own grid.  So the fp32 product with the rounded
@@ -202,8 +221,11 @@ __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
     for (int i = 0; i < 4; ++i) {
         const float x0 = (float)f16_from_bits((unsigned short)(v[i] & 0xffffu));
         const float x1 = (float)f16_from_bits((unsigned short)(v[i] >> 16));
-        float q0 = __builtin_fmaf(x0, f.rl, x0 * f.rh);
-        float q1 = __builtin_fmaf(x1, f.rl, x1 * f.rh);
+        // x * rh written as fma(x, rh, 0): the same value (the product is exact; a zero of either sign
+        // ends as code 0), and it lets both steps take the half straight from the packed word
+        // (v_fma_mix_f32) instead of converting it first
+        float q0 = __builtin_fmaf(x0, f.rl, __builtin_fmaf(x0, f.rh, 0.0f));
+        float q1 = __builtin_fmaf(x1, f.rl, __builtin_fmaf(x1, f.rh, 0.0f));
         q0 = __builtin_amdgcn_fmed3f(q0, -8.0f, 7.0f);
         q1 = __builtin_amdgcn_fmed3f(q1, -8.0f, 7.0f);
         f16x2 h = {(f16)q0, (f16)q1};

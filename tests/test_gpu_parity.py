@@ -218,7 +218,7 @@ def test_linear4bit_module_from_float_and_state_dict():
 
 # ------------------------------------------------------------------------------ Hadamard
 
-HAD_SIZES = [8, 64, 128, 512, 1024, 4096, 8192, 32768, 96, 224, 320, 1376, 5120, 11008, 13824, 14336, 28672]
+HAD_SIZES = [8, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
 
 
 def close(got, want):
@@ -242,7 +242,7 @@ def test_hadamard_within_tolerance(n, dtype):
     assert np.all(np.abs(got - cf) <= tol * (1 + np.abs(cf)))
 
 
-@pytest.mark.parametrize("n", [64, 4096, 8192, 224, 11008, 28672, 13824])
+@pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 224, 3840, 6912, 8960, 11008, 28672, 13824])
 @pytest.mark.parametrize("fp32", [False, True])
 def test_fused_hadamard_quantize_equals_staged(n, fp32):
     """Codes of the fused kernel are judged on the kernel's OWN fp16 Hadamard output (returned on
