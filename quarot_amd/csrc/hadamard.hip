@@ -956,58 +956,58 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
                 }
             }
         }
-        u32 mx = 0;
-        if (QUANT) {
-            mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
-            mx = wave_max_u32_dpp(mx);
-            if (lane == 0) red[wave] = mx;
-        }
-        __syncthreads();
         // ---- stage 3
         if (QUANT) {
+            u32 mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            mx = wave_max_u32_dpp(mx);
+            if (lane == 0) red[wave] = mx;
+            // Units of 16 elements (two chunks, 8-byte stores of codes).  Unit (i, lane) is row
+            // kp = 16 (wave + 4 i) + lane / 4, columns 16 (lane % 4)..: rows of this wave's own tiles,
+            // which it wrote itself, so the reads are issued before the barrier that publishes the row
+            // maximum.  Lanes on rows beyond K repeat the unit of their first tile (K >= 64: always
+            // inside) and store it again, the same value from the same lane: all stores are
+            // unconditional, so their number is known when the next row's loads are awaited and that
+            // wait need not include them.
+            int un[TPW];
+            u32x4 h[TPW][2];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                int kp = (wave + 4 * i) * 16 + (lane >> 2);
+                kp = kp < K ? kp : wave * 16 + (lane >> 2);
+                const f16* src = Yl + kp * YS + (lane & 3) * 16;
+                h[i][0] = *(const u32x4*)src;
+                h[i][1] = *(const u32x4*)(src + 8);
+                un[i] = kp * 4 + (lane & 3);
+            }
+            __syncthreads();
 #pragma unroll
             for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
             const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
             const float s = (float)sh;
-            // units of 16 elements (two chunks): 8-byte stores of codes
-            constexpr int NUI = (KS2 + 1) / 2;
-            const int nunits = nchunks >> 1;
             u32x2* qrow = (u32x2*)(q + row * (int64_t)nchunks);
-            int un[NUI];
-            u32x4 h[NUI][2];
-#pragma unroll
-            for (int j = 0; j < NUI; ++j) {
-                const int u = tid + j * HT;
-                un[j] = u < nunits ? u : nunits - 1;
-                const f16* src = Yl + (un[j] >> 2) * YS + (un[j] & 3) * 16;
-                h[j][0] = *(const u32x4*)src;
-                h[j][1] = *(const u32x4*)(src + 8);
-            }
-            u32x2 codes[NUI];
+            u32x2 codes[TPW];
             if (fast_quant_ok(mx, s)) {
                 const FastRecip fq = make_fast_recip(s);
 #pragma unroll
-                for (int j = 0; j < NUI; ++j) codes[j] = u32x2{sym_codes8_fast(h[j][0], fq), sym_codes8_fast(h[j][1], fq)};
+                for (int i = 0; i < TPW; ++i) codes[i] = u32x2{sym_codes8_fast(h[i][0], fq), sym_codes8_fast(h[i][1], fq)};
             } else {
                 const bool fast = scale_fast_ok(s);
                 const float rs = fast ? 1.0f / s : 0.0f;
 #pragma unroll
-                for (int j = 0; j < NUI; ++j) codes[j] = u32x2{sym_codes8(h[j][0], s, rs, fast), sym_codes8(h[j][1], s, rs, fast)};
+                for (int i = 0; i < TPW; ++i) codes[i] = u32x2{sym_codes8(h[i][0], s, rs, fast), sym_codes8(h[i][1], s, rs, fast)};
             }
-            // Stores without conditions (threads past the end of the row repeat the last unit, same
-            // value): the number of stores in flight is then known when the next row's loads are
-            // awaited, and that wait need not include them.
 #pragma unroll
-            for (int j = 0; j < NUI; ++j) qrow[un[j]] = codes[j];
+            for (int i = 0; i < TPW; ++i) qrow[un[i]] = codes[i];
             scales[row] = sh;
             if (y) {
 #pragma unroll
-                for (int j = 0; j < NUI; ++j) {
-                    __builtin_nontemporal_store(h[j][0], (u32x4*)(y + row * (int64_t)n) + 2 * un[j]);
-                    __builtin_nontemporal_store(h[j][1], (u32x4*)(y + row * (int64_t)n) + 2 * un[j] + 1);
+                for (int i = 0; i < TPW; ++i) {
+                    __builtin_nontemporal_store(h[i][0], (u32x4*)(y + row * (int64_t)n) + 2 * un[i]);
+                    __builtin_nontemporal_store(h[i][1], (u32x4*)(y + row * (int64_t)n) + 2 * un[i] + 1);
                 }
             }
         } else {
+            __syncthreads();
             u32x4 h[KS2];
             int cn[KS2];
 #pragma unroll
@@ -1019,8 +1019,9 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 #pragma unroll
             for (int j = 0; j < KS2; ++j) __builtin_nontemporal_store(h[j], (u32x4*)(y + row * (int64_t)n) + cn[j]);
         }
-        // Tl is next written after this barrier, Yl after the next row's first barrier, red[] after
-        // it as well: every reader of this row has passed by then
+        // Tl is next written after the barrier above (all of this row's stage-2 reads precede it);
+        // red[] is next written after the next row's first barrier; Yl rows and the staging region
+        // are private to a wave
     }
 }
 
@@ -1043,8 +1044,9 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
                        void* q, void* scales, hipStream_t st) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
-    if (m == 64) {
-        // the latency-organised kernel, while two workgroups still fit on a CU
+    if (m == 64 && K >= 64) {
+        // the latency-organised kernel (it relies on every wave's first tile lying inside hadK), while
+        // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
         const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
         if (lds64 <= 80 * 1024) {

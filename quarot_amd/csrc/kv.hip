@@ -59,18 +59,15 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
     for (int i = 0; i < 4; ++i) {
         const f16x2 sh = as_f16x2(v[i]) + z2;
         const float x0 = (float)sh[0], x1 = (float)sh[1];
-        float q0 = __builtin_fmaf(x0, f.rl, x0 * f.rh);
-        float q1 = __builtin_fmaf(x1, f.rl, x1 * f.rh);
+        float q0 = __builtin_fmaf(x0, f.rl, __builtin_fmaf(x0, f.rh, 0.0f));
+        float q1 = __builtin_fmaf(x1, f.rl, __builtin_fmaf(x1, f.rh, 0.0f));
         q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
         q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);
         f16x2 h = {(f16)q0, (f16)q1};
         h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
-        const u32 w = __builtin_bit_cast(u32, h);
-        b[i] = (w & 0xFu) | ((w >> 12) & ~0xFu);    // low byte: code0 | code1 << 4
+        b[i] = __builtin_bit_cast(u32, h);
     }
-    const u32 t01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-    const u32 t23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
-    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+    return pack_nibbles8(b);
 }
 
 // LG = log2(lanes per vector) = log2(dim) - 3, 1..5

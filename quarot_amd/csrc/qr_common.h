@@ -215,6 +215,17 @@ __device__ __forceinline__ FastRecip make_fast_recip(float s) {
     f.rl = __builtin_fmaf(-s, f.rh, 1.0f) * r1;
     return f;
 }
+// w[i] holds two fp16 values 1536 + code (codes in the low four bits of each half, element 2 i in
+// the low half): gather the eight nibbles into one word, element 0 lowest.  Two byte permutes bring
+// the low bytes of all eight halves together, two more split them into the bytes of the even and of
+// the odd elements, a shift and a bit-select merge them: six instructions.
+__device__ __forceinline__ u32 pack_nibbles8(const u32 (&w)[4]) {
+    const u32 p01 = __builtin_amdgcn_perm(w[1], w[0], 0x06020400u);     // w0.b0 w1.b0 w0.b2 w1.b2
+    const u32 p23 = __builtin_amdgcn_perm(w[3], w[2], 0x06020400u);
+    const u32 even = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+    const u32 odd = __builtin_amdgcn_perm(p23, p01, 0x07060302u);
+    return (even & 0x0F0F0F0Fu) | ((odd << 4) & 0xF0F0F0F0u);
+}
 __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
     u32 b[4];
 #pragma unroll
@@ -230,12 +241,9 @@ __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
         q1 = __builtin_amdgcn_fmed3f(q1, -8.0f, 7.0f);
         f16x2 h = {(f16)q0, (f16)q1};
         h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
-        const u32 w = __builtin_bit_cast(u32, h);
-        b[i] = (w & 0xFu) | ((w >> 12) & ~0xFu);    // low byte: code0 | code1 << 4 (upper bytes: don't care)
+        b[i] = __builtin_bit_cast(u32, h);
     }
-    const u32 t01 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u);
-    const u32 t23 = __builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u);
-    return __builtin_amdgcn_perm(t23, t01, 0x05040100u);
+    return pack_nibbles8(b);
 }
 // amax bits below 0x7c00 <=> every element of the row is finite
 __device__ __forceinline__ bool fast_quant_ok(u32 amax_bits, float s) {
