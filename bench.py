@@ -51,9 +51,9 @@ HBM_PEAK_GBS = 8000.0
 FETCH_SCALE, WRITE_SCALE = 262144.0 / 131083.8, 262144.0 / 262144.0
 TRAFFIC_KIB = {
     #        FETCH_SIZE   WRITE_SIZE
-    "c1": (16566.0, 16384.0),
-    "c2": (44225.0, 16384.0),
-    "c3d": (528828.0, 262144.0),
+    "c1": (16551.0, 16384.0),
+    "c2": (44210.0, 16384.0),
+    "c3d": (528791.7, 262144.0),
     "c4": (72440.1, 1024.0),
     "c4m1": (61875.4, 16.0),
     "c4g64": (115876.5, 7168.0),
