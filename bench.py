@@ -8,6 +8,7 @@ quantise + int4 GEMM + fp16 dequant) over one batch of seeded synthetic tokens a
 HBM.  Workloads (shapes of Llama-2; inputs as in the reference's qlinear benchmark but with the
 outlier channels that motivate the Hadamard):
     c1  q_proj 7B      X [2048, 4096]   W int4 [4096, 4096]     no online Hadamard
+    c1n the same with the RMSNorm in front of the quantiser (fused RMSNorm + Quantizer kernel)
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
     c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
     c4  down_proj 70B decode  X [64, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28
@@ -32,6 +33,7 @@ if ROOT not in sys.path:
 WORKLOADS = {
     #        M      K      N     hadamard
     "c1": (2048, 4096, 4096, False),
+    "c1n": (2048, 4096, 4096, False),       # input_layernorm -> Quantizer -> q_proj
     "c2": (2048, 11008, 4096, True),
     "c3d": (32768, 11008, 4096, True),
     "c4": (64, 28672, 8192, True),          # decode, 70B down_proj
@@ -79,7 +81,7 @@ def synth_w(n, k, seed=1):
     return pack_i4(codes), s
 
 
-def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows):
+def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=False):
     """The reference's CPU path (torch Hadamard + quant + integer matmul + dequant) on a bounded
     row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
     from oracle import cpu_baseline as cb
@@ -88,17 +90,18 @@ def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows):
     wc = cb.unpacked_codes(w_packed.numpy())
     ws = w_scales.view(-1)
     torch.set_num_threads(os.cpu_count() or 1)
-    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard)          # warm-up
+    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm)          # warm-up
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
-        cb.linear4bit_path(xs, wc, ws, hadamard)
+        cb.linear4bit_path(xs, wc, ws, hadamard, rmsnorm)
         times.append(time.perf_counter() - t0)
     t = float(np.median(times))
     return {"value": round(2.0 * rows * n * k / t / 1e12, 5), "unit": "TOPS", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"first {rows} of {m} rows, full N and K, median of 3 ({t * 1e3:.0f} ms); torch fp32 matmul_hadU + "
-                      f"fp16 sym quant + int32 torch matmul + fp16 dequant"}
+            "sample": f"first {rows} of {m} rows, full N and K, median of 3 ({t * 1e3:.0f} ms); torch "
+                      + ("fp32 RMSNorm + " if rmsnorm else "fp32 matmul_hadU + " if hadamard else "")
+                      + "fp16 sym quant + int32 torch matmul + fp16 dequant"}
 
 
 def main():
@@ -140,7 +143,9 @@ def main():
     lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
     lin.weight.copy_(w_cpu.to(dev))
     lin.weight_scales.copy_(sw_cpu.to(dev))
-    front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if hadamard else quarot_amd.nn.Quantizer()).to(dev)
+    rmsnorm = args.workload == "c1n"
+    front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if hadamard else quarot_amd.nn.RMSNormQuantizer(k) if rmsnorm
+             else quarot_amd.nn.Quantizer()).to(dev)
     # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
     copies = [lin.weight]
     if m <= 64:
@@ -176,6 +181,7 @@ def main():
 
     # staged (reference-shaped) chain for comparison, untimed in `value`
     staged_front = (torch.nn.Sequential(quarot_amd.nn.OnlineHadamard(k), quarot_amd.nn.Quantizer()) if hadamard
+                    else torch.nn.Sequential(quarot_amd.nn.RMSNorm(k), quarot_amd.nn.Quantizer()) if rmsnorm
                     else quarot_amd.nn.Quantizer()).to(dev)
     for _ in range(3):
         lin(staged_front(x))
@@ -233,13 +239,15 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 scales",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: Linear4bit X[{m},{k}] fp16 (1% outlier channels x20) . W int4[{n},{k}]"
-                               + (" with online Hadamard" if hadamard else ""),
-                   "M": m, "K": k, "N": n, "path": "fused Hadamard+quantise kernel, fused GEMM+dequant kernel",
+                               + (" with online Hadamard" if hadamard else " behind RMSNorm" if rmsnorm else ""),
+                   "M": m, "K": k, "N": n,
+                   "path": ("fused Hadamard+quantise kernel" if hadamard else "fused RMSNorm+quantise kernel" if rmsnorm
+                            else "quantise kernel") + ", fused GEMM+dequant kernel",
                    "staged_reference_api_ms": round(staged_ms, 4)},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(x_cpu, w_cpu, sw_cpu, hadamard, m, n, k, args.cpu_rows)
+        out["cpu_baseline"] = cpu_baseline(x_cpu, w_cpu, sw_cpu, hadamard, m, n, k, args.cpu_rows, rmsnorm)
     print(json.dumps(out))
 
 

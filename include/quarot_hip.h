@@ -91,6 +91,19 @@ int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, int K, const
                                 void* y_or_null, void* stream);
 
 /*
+ * Fused RMSNorm + Quantizer: the chain in front of q/k/v_proj and gate/up_proj
+ * (quarot/nn/normalization.py:15-21 then quarot/nn/quantization.py:9-13; chained in
+ * e2e/quantized_llama/modeling_llama.py:40-44,108-110).
+ *   y = fp16( float(x) * rsqrt( sum(float(x)^2) / mean_dim + eps ) ), computed in fp32 and rounded to
+ *   fp16 once, as the unfused module returns it; q and scales as qr_quantize_rows_f16_i4(y).
+ *   x fp16 [rows, cols], cols % 8 == 0 and cols <= 32768 (else QR_E_UNSUPPORTED: use the two
+ *   separate steps); y_or_null: optional fp16 [rows, cols] copy of the normalised rows.
+ *   x and y 16-byte aligned, q 4-byte aligned.
+ */
+int qr_rmsnorm_quantize_f16_i4(const void* x, int64_t rows, int64_t cols, int mean_dim, float eps,
+                               float clip, void* q, void* scales, void* y_or_null, void* stream);
+
+/*
  * int4 x int4 -> int32 GEMM:  C[M, N] = unpack(A)[M, K] . unpack(B)[N, K]^T.
  * Replaces matmul_host (quarot/kernels/gemm.cu:7-46), bound as quarot._CUDA.matmul
  * (quarot/kernels/bindings.cpp:9-25).

@@ -35,8 +35,17 @@ def quantize(x16):
     return q.to(torch.int32), scale
 
 
-def linear4bit_path(x16, w_codes_i32, w_scales16, hadamard=True):
-    """x fp16 [M, K] -> fp16 [M, N]: Hadamard (fp32) -> quantise -> int32 matmul -> dequant."""
+def rmsnorm(x16, eps=1e-5):
+    """quarot/nn/normalization.py:15-21 in torch on the host."""
+    xf = x16.to(torch.float32)
+    var = xf.pow(2).sum(-1, keepdim=True) / x16.shape[-1]
+    return (xf * torch.rsqrt(var + eps)).to(torch.float16)
+
+
+def linear4bit_path(x16, w_codes_i32, w_scales16, hadamard=True, norm=False):
+    """x fp16 [M, K] -> fp16 [M, N]: (RMSNorm ->) Hadamard (fp32) -> quantise -> int32 matmul -> dequant."""
+    if norm:
+        x16 = rmsnorm(x16)
     xh = matmul_hadU(x16.float()).to(torch.float16) if hadamard else x16
     q, sx = quantize(xh)
     acc = q @ w_codes_i32.t()

@@ -22,6 +22,8 @@ How each function is pinned (see tests/test_oracle.py):
   int4_matmul          int64 brute force, closed-form all-7 x all-(-8) = -56.K, one-hot rows
   sym_dequant          exact rational rounding of each of the three operations
   kv_asym_*            range/extreme-code invariants and exact rational spot checks
+  rmsnorm              float64 closed form x / sqrt(sum(x^2) / mean_dim + eps) rounded once,
+                       constant rows, mean_dim different from the row length, sign symmetry
 """
 from __future__ import annotations
 
@@ -234,6 +236,18 @@ def quantizer(x, clip=1.0):
 
 # ----------------------------------------------------------------------------------------------
 # int4 x int4 GEMM and the dequant epilogue
+
+def rmsnorm(x, mean_dim, eps=1e-5):
+    """quarot/nn/normalization.py:15-21: fp16 input is promoted to fp32, the sum of squares is
+    divided by mean_dim (not necessarily the row length), x * rsqrt(var + eps) is computed in fp32
+    and cast back.  The association order of the fp32 sum is the only freedom (torch's differs
+    from numpy's, the kernel's from both): results agree to within one rounding of the fp32 sum,
+    far below half an fp16 ulp except on exact ties."""
+    xf = np.asarray(x).astype(F32)
+    var = (xf * xf).sum(-1, keepdims=True, dtype=F32) / F32(mean_dim)
+    r = F32(1.0) / np.sqrt(var + F32(eps), dtype=F32)
+    return (xf * r).astype(np.asarray(x).dtype)
+
 
 def int4_matmul(a_packed, b_packed, exact_int=False):
     """matmul_host (quarot/kernels/gemm.cu:7-46): C[M, N] int32 = unpack(A) . unpack(B)^T.

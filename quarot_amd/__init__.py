@@ -15,7 +15,7 @@ from . import nn
 
 __all__ = [
     "matmul", "sym_quant", "sym_dequant", "PackedQuantizedTensor",      # the reference's names
-    "quantize_rows", "hadamard_quantize", "linear_i4",                  # fused entry points
+    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "linear_i4",   # fused entry points
 ]
 
 
@@ -165,6 +165,25 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, -1), s.view(s_shape))
     return (packed, y.view(x.shape)) if return_transformed else packed
+
+
+def rmsnorm_quantize(x, mean_dim, eps=1e-5, clip_ratio=1.0, return_normalized=False):
+    """RMSNorm.forward followed by Quantizer.forward in one kernel
+    (quarot/nn/normalization.py:15-21 + quarot/nn/quantization.py:9-13)."""
+    assert x.dtype == torch.float16
+    x2, lead = _flat2d(x)
+    dev = _require_gpu_contiguous("rmsnorm_quantize", x=x2)
+    rows, cols = x2.shape
+    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
+    s = torch.empty((rows,), dtype=torch.float16, device=dev)
+    y = torch.empty_like(x2) if return_normalized else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_rmsnorm_quantize_f16_i4(_ptr(x2), rows, cols, int(mean_dim), float(eps),
+                                                         float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
+                                                         _lib.stream_ptr(dev)))
+    s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
+    packed = PackedQuantizedTensor(q.view(*lead, -1), s.view(s_shape))
+    return (packed, y.view(x.shape)) if return_normalized else packed
 
 
 def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):

@@ -60,6 +60,100 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
     }
 }
 
+// Wave-wide fp32 sum without LDS: four DPP steps reduce each row of 16 lanes, four lane reads combine
+// the rows.  The result is wave-uniform; the association order is fixed.
+__device__ __forceinline__ float wave_sum_f32_dpp(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// RMSNorm (no gain) followed by the per-token quantiser, one pass over x: the row stays in
+// registers between the two reductions.  The normalised value is rounded to fp16 exactly where
+// the unfused chain stores it -- fp16( float(x) * rsqrt(sum(x^2) / mean_dim + eps) ), all in fp32 --
+// and the quantiser runs on those fp16 values.  Only the association order of the fp32 sum of
+// squares is this kernel's own.
+template <int NV>
+__global__ __launch_bounds__(QT) void rmsnorm_quant_rows_kernel(const u32x4* __restrict__ x, float mean_dim, float eps,
+                                                                float clip, int cols8, u32* __restrict__ q,
+                                                                f16* __restrict__ scale_out, u32x4* __restrict__ y) {
+    __shared__ float redf[QT / QR_WAVE];
+    __shared__ u32 red[QT / QR_WAVE];
+    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x & (QR_WAVE - 1), wave = threadIdx.x / QR_WAVE;
+    const u32x4* xr = x + row * (int64_t)cols8;
+    u32x4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * QT;
+        v[i] = c < cols8 ? xr[c] : u32x4{0, 0, 0, 0};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const f16x2 h = as_f16x2(v[i][w]);
+            const float a = (float)h[0], b = (float)h[1];
+            ss = __builtin_fmaf(a, a, ss);          // a * a is exact in fp32 (22 bits)
+            ss = __builtin_fmaf(b, b, ss);
+        }
+    ss = wave_sum_f32_dpp(ss);
+    if (lane == 0) redf[wave] = ss;
+    __syncthreads();
+    const float total = (redf[0] + redf[1]) + (redf[2] + redf[3]);
+    const float r = 1.0f / __builtin_sqrtf(total / mean_dim + eps);
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const f16x2 h = as_f16x2(v[i][w]);
+            v[i][w] = narrow_f16x2((float)h[0] * r, (float)h[1] * r);
+        }
+        const u32 mi = absmax_bits8(v[i]);
+        m = m > mi ? m : mi;
+    }
+    m = wave_max_u32_dpp(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
+    const f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
+    if (threadIdx.x == 0) scale_out[row] = sh;
+    const float s = (float)sh;
+    u32* qr = q + row * (int64_t)cols8;
+    if (y) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * QT;
+            if (c < cols8) y[row * (int64_t)cols8 + c] = v[i];
+        }
+    }
+    if (fast_quant_ok(m, s)) {       // workgroup-uniform
+        const FastRecip fr = make_fast_recip(s);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = threadIdx.x + i * QT;
+            if (c < cols8) qr[c] = sym_codes8_fast(v[i], fr);
+        }
+        return;
+    }
+    const bool fast = scale_fast_ok(s);
+    const float rs = fast ? 1.0f / s : 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = threadIdx.x + i * QT;
+        if (c < cols8) qr[c] = sym_codes8(v[i], s, rs, fast);
+    }
+}
+
 // Any column count (odd included), any alignment: one workgroup per row, scalar accesses, the row
 // is read twice when the scale has to be derived.  Used only when the vector kernel's
 // preconditions (cols % 8 == 0, cols <= 32768, 16-byte aligned x, 4-byte aligned q) do not hold.
@@ -170,6 +264,31 @@ extern "C" int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, 
     if (cols == 0) return QR_E_SHAPE;   // torch.max over an empty axis raises in the reference
     if (!x || !q || !scales) return QR_E_NULL;
     return launch_quant<false>(x, nullptr, clip, rows, cols, q, scales, (hipStream_t)stream);
+}
+
+extern "C" int qr_rmsnorm_quantize_f16_i4(const void* x, int64_t rows, int64_t cols, int mean_dim, float eps, float clip,
+                                          void* q, void* scales, void* y_or_null, void* stream) {
+    if (rows < 0 || cols <= 0 || mean_dim <= 0) return QR_E_SHAPE;
+    if (rows == 0) return QR_OK;
+    if (rows > 0x7fffffffLL) return QR_E_SHAPE;
+    if (!x || !q || !scales) return QR_E_NULL;
+    if (cols % 8 != 0 || cols > 32768) return QR_E_UNSUPPORTED;
+    if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
+    const int cols8 = (int)(cols / 8);
+    const int nv = (cols8 + QT - 1) / QT;
+    dim3 grid((unsigned)rows), block(QT);
+    hipStream_t st = (hipStream_t)stream;
+#define QR_LAUNCH(NV)                                                                                                 \
+    rmsnorm_quant_rows_kernel<NV><<<grid, block, 0, st>>>((const u32x4*)x, (float)mean_dim, eps, clip, cols8, (u32*)q, \
+                                                          (f16*)scales, (u32x4*)y_or_null)
+    if (nv <= 1) QR_LAUNCH(1);
+    else if (nv <= 2) QR_LAUNCH(2);
+    else if (nv <= 4) QR_LAUNCH(4);
+    else if (nv <= 6) QR_LAUNCH(6);
+    else if (nv <= 8) QR_LAUNCH(8);
+    else QR_LAUNCH(16);
+#undef QR_LAUNCH
+    return qr_launch_status();
 }
 
 extern "C" int qr_sym_dequant_i32_f16(const void* q, const void* scale_row, const void* scale_col, int64_t rows,

@@ -268,6 +268,58 @@ def test_fused_hadamard_quantize_equals_staged(n, fp32):
     assert close(y2.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
 
 
+@pytest.mark.parametrize("shape", [(5, 64), (9, 4096), (7, 5120), (3, 8192), (4, 11008), (2, 32768), (6, 24), (3, 100)])
+@pytest.mark.parametrize("clip", [1.0, 0.9])
+def test_fused_rmsnorm_quantize(shape, clip):
+    """RMSNorm + Quantizer in one kernel.  The normalised rows (returned on request) must agree with
+    the oracle to the stated floating-point tolerance -- only the order of the fp32 sum of squares
+    differs, so almost every element is identical -- and the codes and scales must equal the oracle
+    quantiser applied to the kernel's OWN normalised rows, bit for bit."""
+    rows, cols = shape
+    x = gpu(synth_x(rows, cols, seed=cols + 3))
+    mod = quarot_amd.nn.RMSNormQuantizer(cols, eps=1e-5, input_clip_ratio=clip)
+    p = mod(x)
+    staged_y = quarot_amd.nn.RMSNorm(cols, eps=1e-5)(x)
+    staged = quarot_amd.nn.Quantizer(clip)(staged_y)
+    want_y = o.rmsnorm(x.cpu().numpy(), cols, 1e-5)
+    if cols % 8 == 0:
+        p2, y = quarot_amd.rmsnorm_quantize(x, cols, 1e-5, clip, return_normalized=True)
+        assert torch.equal(p.quantized_x, p2.quantized_x) and torch.equal(p.scales_x, p2.scales_x)
+        yk = y.cpu().numpy()
+        assert close(yk, want_y) and np.mean(yk == want_y) > 0.999
+        wq, ws = o.quantizer(yk, clip)
+        assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+        assert np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+        assert float((y == staged_y).float().mean()) > 0.999
+    assert p.quantized_x.shape == staged.quantized_x.shape and p.scales_x.shape == staged.scales_x.shape
+    assert float((p.quantized_x == staged.quantized_x).float().mean()) > 0.995
+    assert close(staged_y.cpu().numpy(), want_y)
+
+
+def test_fused_rmsnorm_quantize_full_size_and_errors():
+    """Benchmark-size input (2048 x 4096) on strided rows; mean_dim different from the width;
+    argument errors of the C entry point."""
+    x = gpu(synth_x(2048, 4096, seed=5))
+    p, y = quarot_amd.rmsnorm_quantize(x, 4096, 1e-5, 1.0, return_normalized=True)
+    rows = slice(None, None, 129)
+    want_y = o.rmsnorm(x[rows].cpu().numpy(), 4096, 1e-5)
+    assert close(y[rows].cpu().numpy(), want_y)
+    wq, ws = o.quantizer(y[rows].cpu().numpy(), 1.0)
+    assert np.array_equal(p.quantized_x[rows].cpu().numpy(), wq)
+    assert np.array_equal(p.scales_x.view(-1)[rows].cpu().numpy(), ws)
+    assert torch.allclose(y.float().pow(2).mean(-1), torch.ones(2048, device=y.device), rtol=2e-3)
+    p4, y4 = quarot_amd.rmsnorm_quantize(x[:8], 1024, 1e-5, 1.0, return_normalized=True)
+    assert close(y4.cpu().numpy(), o.rmsnorm(x[:8].cpu().numpy(), 1024, 1e-5))
+    L = _lib.lib()
+    q = torch.empty(8, 2048, dtype=torch.uint8, device=x.device)
+    s = torch.empty(8, dtype=torch.float16, device=x.device)
+    st = torch.cuda.current_stream().cuda_stream
+    assert L.qr_rmsnorm_quantize_f16_i4(x.data_ptr(), 8, 4092, 4092, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) == _lib.lib().qr_rmsnorm_quantize_f16_i4(x.data_ptr(), 8, 40000, 40000, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_rmsnorm_quantize_f16_i4(x.data_ptr() + 2, 8, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) == -4
+    assert L.qr_rmsnorm_quantize_f16_i4(x.data_ptr(), 0, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) == 0
+    assert L.qr_rmsnorm_quantize_f16_i4(None, 8, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+
+
 def test_hadamard_full_size_properties():
     """Benchmark-size rows (2048 x 11008 and 2048 x 4096): norm preservation, linearity in a row
     scaling by 2 (exact in floating point), power-of-two transform is an involution."""

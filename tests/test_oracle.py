@@ -339,6 +339,47 @@ def test_kv_asym_exact_rational_spot():
             assert back == o.kv_asym_dequant(p, s, z)[r, c]
 
 
+def test_rmsnorm_closed_form_and_special_cases():
+    """x / sqrt(sum(x^2) / mean_dim + eps) in exact rational arithmetic, rounded once to fp16, on a
+    handful of rows (the square root bracketed by exact integer comparison); then properties a wrong
+    divisor, a missing eps or a mean over the wrong axis would break."""
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((3, 24)) * 3).astype(F16)
+    got = o.rmsnorm(x, 24, 1e-5)
+    x64 = x.astype(np.float64)
+    want64 = x64 / np.sqrt((x64 ** 2).sum(-1, keepdims=True) / 24 + np.float64(F32(1e-5)))
+    # float64 carries 53 bits: its rounding to fp16 is the exact answer unless within 2^-40 of a tie
+    assert np.array_equal(got, want64.astype(F16))
+    # exact rational check of one element: y^2 * (S / d + eps) == x^2 up to the fp16 rounding interval
+    S = sum(Fraction(float(v)) ** 2 for v in x[0])
+    denom = S / 24 + Fraction(float(F32(1e-5)))
+    for j in (0, 7, 23):
+        y = Fraction(float(got[0, j]))
+        ulp = Fraction(float(np.spacing(np.abs(got[0, j]).astype(F16))))
+        lo, hi = abs(y) - ulp / 2, abs(y) + ulp / 2
+        assert lo ** 2 * denom <= Fraction(float(x[0, j])) ** 2 <= hi ** 2 * denom
+        assert (y < 0) == (x[0, j] < 0)
+    # constant row c with mean_dim = length: c / sqrt(c^2 + eps) ~ sign(c)
+    c = np.full((1, 64), -2.0, F16)
+    assert np.array_equal(o.rmsnorm(c, 64, 1e-5), np.full((1, 64), F16(-2.0 / np.sqrt(4.0 + 1e-5)), F16))
+    # mean_dim is a parameter, not the row length: quadrupling it doubles the output (eps negligible)
+    big = (rng.standard_normal((2, 32)) * 8).astype(F16)
+    a, b = o.rmsnorm(big, 32, 0.0).astype(np.float64), o.rmsnorm(big, 128, 0.0).astype(np.float64)
+    assert np.allclose(b, 2 * a, rtol=2e-3)
+    # eps matters for tiny rows: an all-zero row stays zero instead of dividing by zero
+    assert np.array_equal(o.rmsnorm(np.zeros((1, 16), F16), 16, 1e-5), np.zeros((1, 16), F16))
+    # each row is normalised on its own
+    assert np.array_equal(o.rmsnorm(x, 24, 1e-5)[1], o.rmsnorm(x[1:2], 24, 1e-5)[0])
+    # torch's CPU kernels on the same statement (the timed CPU baseline uses them): same values up to
+    # the order of the fp32 sum
+    import torch
+    from oracle import cpu_baseline as cb
+    wide = (rng.standard_normal((16, 4096)) * 2).astype(F16)
+    t = cb.rmsnorm(torch.from_numpy(wide)).numpy()
+    w = o.rmsnorm(wide, 4096, 1e-5)
+    assert np.mean(t == w) > 0.999 and np.allclose(t.astype(F32), w.astype(F32), rtol=1e-3, atol=1e-3)
+
+
 def test_cpu_baseline_port_agrees_with_oracle():
     """The torch chain timed as the CPU baseline computes what the oracle computes (Hadamard to
     tolerance; given the same Hadamard output, identical codes and identical fp16 outputs)."""
