@@ -712,6 +712,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
     constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
     constexpr int S0 = 4;                                   // first slot that unpacks (LDS reads are issued in slots 0..7, in fragment order)
+    constexpr bool DIRECT = !RAGGED;                        // whole stages go straight into LDS (see gemm_spk_kernel)
     extern __shared__ u32x4 sp2_lds[];                       // [2][CH]; later the output slabs
 
     const int nxcd = 8;
@@ -744,7 +745,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
         int gr = row < BM ? m0 + row : n0 + row - BM;
         const int lim = row < BM ? M - 1 : N - 1;
         gr = gr < lim ? gr : lim;
-        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
+        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : DIRECT ? (u32)(((tid & 7) ^ ((srow >> 1) & 7)) * 16) : (u32)scoff);
     }
     u32x4 regs[1][NL];                                      // one set: loads run one (long) stage ahead of their LDS write
     // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
@@ -762,6 +763,16 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
         const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
         sp2_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
+    };
+
+    // direct form: chunk i of stage st into stage buffer buf (a wave's 64 lanes fill 1 KB of consecutive LDS)
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto dma1 = [&](int st, int buf, int i) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        __attribute__((address_space(3))) void* dst =
+            (__attribute__((address_space(3))) void*)(sp2_lds + buf * CH + i * NT + wave_u * 64);
+        if (i * 32 < BM) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, goff[i], kb, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, goff[i], kb, 0, 0);
     };
 
     i32x16 acc[IM][JN];
@@ -804,10 +815,10 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     };
     // One 64-k sub-step = NMF = 32 slots.  Slot q: MFMA q of the current operands; slots 0..7 read
     // the packed fragments of the NEXT sub-step (one fragment buffer), slots S0.. unpack them
-    // (UNP / (NMF - S0) = 4 instructions per slot); in sub-step 0, slots 2.. also write one chunk of
-    // stage ks+1 to LDS and request the same chunk of stage ks+2.  A full scheduling barrier after
-    // every slot keeps this order.
-#define QR_SP2_SUBSTEP(CUR, NXT, RBUF, RU, DEP)                                                  \
+    // (UNP / (NMF - S0) = 4 instructions per slot); slots 8.. of sub-step 0 also write one chunk of
+    // stage ks+1 to LDS each, slots 8.. of sub-step 1 request the same chunks of stage ks+2 (at most
+    // one memory instruction per slot).  A full scheduling barrier after every slot keeps this order.
+#define QR_SP2_SUBSTEP(CUR, NXT, RBUF, RU, DEP, FET)                                             \
     _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
         mfma1(CUR, q_);                                                                          \
         if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
@@ -815,16 +826,54 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
             _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
                 unpack1(pk, NXT, n_);                                                            \
         }                                                                                        \
-        if ((DEP) && q_ >= 8 && q_ < 8 + NL) {                                                   \
-            deposit1(ks + 1, nb, 0, q_ - 8);                                                     \
-            fetch1(ks + 2, 0, q_ - 8);                                                           \
-        }                                                                                        \
+        if ((DEP) && q_ >= 8 && q_ < 8 + NL) deposit1(ks + 1, nb, 0, q_ - 8);                    \
+        if ((FET) && q_ >= 8 && q_ < 8 + NL) fetch1(ks + 2, 0, q_ - 8);                          \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     }
 
-    // prologue: stage 0 into LDS, stage 1 requested; sub-step 0 unpacked
     Packed pk;
     Ops ops[2];
+    if constexpr (DIRECT) {
+        // Two stage buffers.  Sub-step 0 of stage s is read during sub-step 3 of stage s - 1, the rest
+        // during sub-steps 0..2 of stage s; after the barrier of stage s (before its sub-step 3) nobody
+        // reads buffer s % 2 any more, and the loads of stage s + 2 into it are issued in that sub-step 3:
+        // they have three sub-steps (~2 us) to land before the next barrier, which waits for all of this
+        // wave's loads.
+#define QR_SP2D_BARRIER(ALLOWED)                                                                 \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(ALLOWED) : "memory");
+#define QR_SP2D_SUBSTEP(CUR, NXT, RBUF, RU, FET)                                                 \
+    _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
+        mfma1(CUR, q_);                                                                          \
+        if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
+        if (q_ >= S0) {                                                                          \
+            _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
+                unpack1(pk, NXT, n_);                                                            \
+        }                                                                                        \
+        if ((FET) && q_ >= 8 && q_ < 8 + NL) dma1(ks + 2, b, q_ - 8);                            \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    }
+#pragma unroll
+        for (int i = 0; i < NL; ++i) dma1(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) dma1(1, 1, i);
+        QR_SP2D_BARRIER(NL)
+#pragma unroll
+        for (int r = 0; r < NF; ++r) read1(0, 0, r, pk);
+#pragma unroll
+        for (int n = 0; n < UNP; ++n) unpack1(pk, ops[0], n);
+        for (int ks = 0; ks < stages; ++ks) {
+            const int b = ks & 1, nb = b ^ 1;
+            QR_SP2D_SUBSTEP(ops[0], ops[1], b, 1, false)
+            QR_SP2D_SUBSTEP(ops[1], ops[0], b, 2, false)
+            QR_SP2D_SUBSTEP(ops[0], ops[1], b, 3, false)
+            QR_SP2D_BARRIER(0)                              // stage ks+1 landed; stage ks fully read
+            QR_SP2D_SUBSTEP(ops[1], ops[0], nb, 0, true)
+        }
+#undef QR_SP2D_SUBSTEP
+#undef QR_SP2D_BARRIER
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // repeats of the last stage still landing
+    } else {
+    // prologue: stage 0 into LDS, stage 1 requested; sub-step 0 unpacked
 #pragma unroll
     for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
 #pragma unroll
@@ -839,14 +888,15 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     for (int ks = 0; ks < stages; ++ks) {
         const int b = ks & 1, nb = b ^ 1;
         // sub-step 0: multiply (ks,0); read + unpack (ks,1); stage ks+1 -> LDS, request ks+2
-        QR_SP2_SUBSTEP(ops[0], ops[1], b, 1, true)
-        // sub-step 1: multiply (ks,1); read + unpack (ks,2)
-        QR_SP2_SUBSTEP(ops[1], ops[0], b, 2, false)
+        QR_SP2_SUBSTEP(ops[0], ops[1], b, 1, true, false)
+        // sub-step 1: multiply (ks,1); read + unpack (ks,2); request ks+2 into the registers just written out
+        QR_SP2_SUBSTEP(ops[1], ops[0], b, 2, false, true)
         // sub-step 2: multiply (ks,2); read + unpack (ks,3)
-        QR_SP2_SUBSTEP(ops[0], ops[1], b, 3, false)
+        QR_SP2_SUBSTEP(ops[0], ops[1], b, 3, false, false)
         __syncthreads();                                    // stage ks+1 visible; stage ks fully read
         // sub-step 3: multiply (ks,3); read + unpack (ks+1,0)
-        QR_SP2_SUBSTEP(ops[1], ops[0], nb, 0, false)
+        QR_SP2_SUBSTEP(ops[1], ops[0], nb, 0, false, false)
+    }
     }
 #undef QR_SP2_SUBSTEP
     __syncthreads();                                        // stage buffers free for the output slabs
@@ -928,7 +978,12 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
     constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
     constexpr int S0 = 4;                                   // first slot that unpacks (LDS reads are issued in slots 0..7, in fragment order)
-    extern __shared__ u32x4 spk_lds[];                       // [2][CH]; later the output slabs
+    // Whole stages (K % 256 == 0) go from global memory straight into LDS (buffer_load ... lds, 16
+    // bytes per lane): no staging registers, no LDS write instructions, a third stage buffer instead.
+    // Measured 3-5 % faster than the register-staged form (kept for ragged K, where dead pieces must
+    // be written as zeros) at M = 2048, N = 4096, K = 11008 and K = 4096.
+    constexpr bool DIRECT = !RAGGED;
+    extern __shared__ u32x4 spk_lds[];                       // [DIRECT ? 3 : 2][CH]; later the output slabs
 
     const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
@@ -960,7 +1015,9 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
         int gr = row < BM ? m0 + row : n0 + row - BM;
         const int lim = row < BM ? M - 1 : N - 1;
         gr = gr < lim ? gr : lim;
-        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : (u32)scoff);
+        // direct form: a lane's data lands at LDS position (row, tid % 8), so the lane fetches the
+        // piece that the XOR-keyed layout keeps there (the key is the same for all of a lane's rows)
+        goff[i] = (u32)gr * (u32)Kb + (RAGGED ? 0u : DIRECT ? (u32)(((tid & 7) ^ ((srow >> 1) & 7)) * 16) : (u32)scoff);
     }
     u32x4 regs[2][NL];                                      // two sets: loads run two stages ahead of their LDS write
     // One 16-byte chunk of stage st (branch-free: stages past the end repeat the last one), as a raw
@@ -978,6 +1035,18 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     auto deposit1 = [&](int st, int buf, int set, int i) {    // st past the end: a repeat of the last stage, never read
         const bool dead = RAGGED && st >= stages - 1 && (stages - 1) * 128 + scoff >= Kb;
         spk_lds[buf * CH + dst0 + i * 32 * 8] = dead ? u32x4{0, 0, 0, 0} : regs[set][i];
+    };
+
+    // direct form: chunk i of stage st into stage buffer buf; a wave's 64 lanes fill 1 KB of consecutive
+    // LDS (8 rows of 128 bytes).  Stages past the end repeat the last one into a buffer nobody reads, so
+    // that every stage issues the same number of loads (the waits below count them).
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto dma1 = [&](int st, int buf, int i) {
+        const int kb = (st < stages ? st : stages - 1) * 128;
+        __attribute__((address_space(3))) void* dst =
+            (__attribute__((address_space(3))) void*)(spk_lds + buf * CH + i * NT + wave_u * 64);
+        if (i * 32 < BM) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, goff[i], kb, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, goff[i], kb, 0, 0);
     };
 
     i32x16 acc[IM][JN];
@@ -1023,10 +1092,11 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     };
     // One 64-k sub-step = NMF = 32 slots.  Slot q: MFMA q of the current operands; slots 0..7 read
     // the packed fragments of this wave's NEXT sub-step (one fragment buffer), slots S0.. unpack
-    // them (4 instructions per slot); in a stage's first sub-step, slots 2.. also write one chunk
-    // of stage ks+1 to LDS and request the same chunk of stage ks+2.  A full scheduling barrier
-    // after every slot keeps this order.
-#define QR_SPK_SUBSTEP(CUR, NXT, RBUF, RU, DEP, SET)                                             \
+    // them (4 instructions per slot); slots 8.. of a stage's first sub-step also write one chunk
+    // of stage ks+1 to LDS each, slots 8.. of its second sub-step request the same chunks of stage
+    // ks+3 (one memory instruction per slot at most).  A full scheduling barrier after every slot
+    // keeps this order.
+#define QR_SPK_SUBSTEP(CUR, NXT, RBUF, RU, DEP, FET, SET)                                        \
     _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
         mfma1(CUR, q_);                                                                          \
         if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
@@ -1034,10 +1104,8 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
             _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
                 unpack1(pk, NXT, n_);                                                            \
         }                                                                                        \
-        if ((DEP) && q_ >= 8 && q_ < 8 + NL) {                                                   \
-            deposit1(ks_ + 1, nb_, SET, q_ - 8);                                                 \
-            fetch1(ks_ + 3, SET, q_ - 8);                                                        \
-        }                                                                                        \
+        if ((DEP) && q_ >= 8 && q_ < 8 + NL) deposit1(ks_ + 1, nb_, SET, q_ - 8);                \
+        if ((FET) && q_ >= 8 && q_ < 8 + NL) fetch1(ks_ + 3, SET, q_ - 8);                       \
         __builtin_amdgcn_sched_barrier(0);                                                       \
     }
     // one stage: KS = stage index, B = its LDS buffer (compile-time), SET = register set that holds
@@ -1046,16 +1114,74 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     {                                                                                            \
         const int ks_ = (KS);                                                                    \
         constexpr int b_ = (B), nb_ = 1 - (B);                                                   \
-        /* first sub-step: multiply (ks,u0); read + unpack (ks,u1); stage ks+1 -> LDS, request ks+3 */ \
-        QR_SPK_SUBSTEP(ops[0], ops[1], b_, 1, true, SET)                                         \
+        /* first sub-step: multiply (ks,u0); read + unpack (ks,u1); stage ks+1 -> LDS */         \
+        QR_SPK_SUBSTEP(ops[0], ops[1], b_, 1, true, false, SET)                                  \
         __syncthreads(); /* stage ks+1 visible; stage ks fully read */                           \
-        /* second sub-step: multiply (ks,u1); read + unpack (ks+1,u0) */                         \
-        QR_SPK_SUBSTEP(ops[1], ops[0], nb_, 0, false, SET)                                       \
+        /* second sub-step: multiply (ks,u1); read + unpack (ks+1,u0); request ks+3 */           \
+        QR_SPK_SUBSTEP(ops[1], ops[0], nb_, 0, false, true, SET)                                 \
     }
 
-    // prologue: stage 0 into LDS, stages 1 and 2 requested; this wave's first sub-step unpacked
     Packed pk;
     Ops ops[2];
+    if constexpr (DIRECT) {
+        // Three stage buffers.  Stage s lives in buffer s % 3; its sub-step u0 is read during the second
+        // sub-step of stage s - 1, its sub-step u1 during the first sub-step of stage s; the barrier
+        // of stage s (between its two sub-steps) is the last point at which anybody reads buffer
+        // s % 3, and the loads of stage s + 3 into it are issued right after.  A wave's loads complete
+        // in order, so "at most NL outstanding" at the barrier of stage s means its part of stage
+        // s + 1 has landed (only stage s + 2 may still be in flight); the barrier then covers the other
+        // waves' parts.  The wait is written by hand: the compiler would wait for all loads.
+#define QR_SPKD_BARRIER(ALLOWED)                                                                 \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(ALLOWED) : "memory");
+#define QR_SPKD_SUBSTEP(CUR, NXT, RBUF, RU, FET, FBUF)                                           \
+    _Pragma("unroll") for (int q_ = 0; q_ < NMF; ++q_) {                                         \
+        mfma1(CUR, q_);                                                                          \
+        if (q_ < NF) read1(RBUF, RU, q_, pk);                                                    \
+        if (q_ >= S0) {                                                                          \
+            _Pragma("unroll") for (int n_ = ((q_ - S0) * UNP) / (NMF - S0); n_ < ((q_ - S0 + 1) * UNP) / (NMF - S0); ++n_) \
+                unpack1(pk, NXT, n_);                                                            \
+        }                                                                                        \
+        if ((FET) && q_ >= 8 && q_ < 8 + NL) dma1(ks_ + 3, FBUF, q_ - 8);                        \
+        __builtin_amdgcn_sched_barrier(0);                                                       \
+    }
+#define QR_SPKD_STAGE(KS, B)                                                                     \
+    {                                                                                            \
+        const int ks_ = (KS);                                                                    \
+        constexpr int b_ = (B), nb_ = ((B) + 1) % 3;                                             \
+        /* multiply (ks,u0); read + unpack (ks,u1) */                                            \
+        QR_SPKD_SUBSTEP(ops[0], ops[1], b_, 1, false, b_)                                        \
+        QR_SPKD_BARRIER(NL) /* stage ks+1 landed; buffer b_ fully read */                        \
+        /* multiply (ks,u1); read + unpack (ks+1,u0); stage ks+3 -> buffer b_ */                 \
+        QR_SPKD_SUBSTEP(ops[1], ops[0], nb_, 0, true, b_)                                        \
+    }
+#pragma unroll
+        for (int i = 0; i < NL; ++i) dma1(0, 0, i);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) dma1(1, 1, i);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) dma1(2, 2, i);
+        QR_SPKD_BARRIER(2 * NL)
+#pragma unroll
+        for (int r = 0; r < NF; ++r) read1(0, 0, r, pk);
+#pragma unroll
+        for (int n = 0; n < UNP; ++n) unpack1(pk, ops[0], n);
+        int ks = 0;
+        for (; ks + 2 < stages; ks += 3) {
+            QR_SPKD_STAGE(ks, 0)
+            QR_SPKD_STAGE(ks + 1, 1)
+            QR_SPKD_STAGE(ks + 2, 2)
+        }
+        if (ks < stages) {
+            QR_SPKD_STAGE(ks, 0)
+            if (ks + 1 < stages) QR_SPKD_STAGE(ks + 1, 1)
+        }
+#undef QR_SPKD_STAGE
+#undef QR_SPKD_SUBSTEP
+#undef QR_SPKD_BARRIER
+        // the repeats of the last stage are still landing in the stage buffers, which the epilogue reuses
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+    // prologue: stage 0 into LDS, stages 1 and 2 requested; this wave's first sub-step unpacked
 #pragma unroll
     for (int i = 0; i < NL; ++i) fetch1(0, 0, i);
 #pragma unroll
@@ -1077,6 +1203,7 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
         QR_SPK_STAGE(ks + 1, 1, 1)
     }
     if (ks < stages) QR_SPK_STAGE(ks, 0, 0)
+    }
 #undef QR_SPK_STAGE
 #undef QR_SPK_SUBSTEP
 
@@ -1180,12 +1307,13 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
 
 int launch_spk(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st) {
-    constexpr size_t LDS = (size_t)2 * (128 + 256) * 8 * 16;
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     const bool ragged = (Kb & 127) != 0;
+    // stage buffers of 48 KB: two behind staging registers, three when loaded straight into LDS
+    const size_t LDS = (size_t)(ragged ? 2 : 3) * (128 + 256) * 8 * 16;
     if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
         return launch_ks<128, 256, 2, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
     hipError_t e;
