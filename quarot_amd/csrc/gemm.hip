@@ -1373,7 +1373,10 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
 // (SB / 16 lanes per row piece of SB bytes, PF steps ahead in a register ring) and turns them into
 // MFMA fragments (lane = row) through a wave-private LDS buffer.  Loading fragments straight from
 // global memory makes every instruction touch 32 different lines and was measured 1.5-2x slower.
-template <int MT, int SB, bool DEQ>
+// XL = load instructions per step that carry rows of X (64 / CPR rows each): with few tokens only
+// the first ceil(M / (64 / CPR)) of them are issued and staged; the remaining rows of the 32-row
+// MFMA operand keep whatever the buffer holds, and the output rows they produce are never stored.
+template <int MT, int SB, int XL, bool DEQ>
 __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
@@ -1381,7 +1384,9 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
     constexpr int CPR = SB / 16;                            // 16-byte chunks per row and step (4, 8 or 16)
     constexpr int PF = SB == 64 ? 4 : 3;                    // steps in flight
     constexpr int ROWS = (1 + MT) * 32;                     // staged rows per wave: 32 of W, then 32 MT of X
-    constexpr int NLD = ROWS * CPR / 64;                    // chunks per lane and step
+    constexpr int NLW = 32 * CPR / 64;                      // chunks per lane and step: rows of W ...
+    constexpr int NLD = NLW + XL;                           // ... plus the rows of X that exist
+    static_assert(XL >= 1 && XL <= MT * 32 * CPR / 64, "X load groups");
     constexpr int STAGE = ROWS * CPR;                       // u32x4 per wave
     constexpr int RED = MT * 4 * 64;                        // i32x4 per wave for the final sum
     extern __shared__ u32x4 dec_smem[];                     // 8 * max(STAGE, RED)
@@ -1667,27 +1672,31 @@ int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, voi
 int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                   const void* bias, hipStream_t st) {
     const unsigned grid = (unsigned)((N + 31) / 32);
-#define QR_DEC(MT, SB)                                                                                                \
+#define QR_DEC(MT, SB, XL)                                                                                            \
     do {                                                                                                              \
         constexpr int STAGE = (1 + MT) * 32 * (SB / 16), RED = MT * 4 * 64;                                           \
         constexpr size_t LDS = (size_t)8 * (STAGE > RED ? STAGE : RED) * 16;                                          \
         hipError_t e;                                                                                                 \
         if (Y) {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, true>;                                                               \
+            auto kern = decode_i4_kernel<MT, SB, XL, true>;                                                           \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr,         \
                                                      (f16*)Y, (const f16*)sA, (const f16*)sB, (const f16*)bias);      \
         } else {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, false>;                                                              \
+            auto kern = decode_i4_kernel<MT, SB, XL, false>;                                                          \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
                                                      nullptr, nullptr, nullptr, nullptr);                             \
         }                                                                                                             \
     } while (0)
-    if (M <= 32) QR_DEC(1, 128);
-    else QR_DEC(2, 128);
+    // a load instruction carries eight rows of X (128-byte pieces): issue only those that exist
+    if (M <= 8) QR_DEC(1, 128, 1);
+    else if (M <= 16) QR_DEC(1, 128, 2);
+    else if (M <= 32) QR_DEC(1, 128, 4);
+    else if (M <= 48) QR_DEC(2, 128, 6);
+    else QR_DEC(2, 128, 8);
 #undef QR_DEC
     return qr_launch_status();
 }
