@@ -134,7 +134,11 @@ GEMM_SHAPES = [(1, 1, 64), (32, 32, 64), (33, 65, 128), (64, 64, 192), (100, 200
                (8, 300, 1024), (40, 512, 512), (64, 1000, 2048), (65, 256, 320), (129, 257, 448), (256, 512, 4096),
                (300, 700, 11008), (512, 1024, 2048), (1000, 3000, 1024), (2048, 4096, 4096),
                # the pipelined kernels: whole and partly filled K stages, whole and ragged tiles
-               (2048, 4096, 320), (2050, 4100, 448), (4096, 4096, 256), (4090, 4090, 192), (2304, 8192, 64)]
+               (2048, 4096, 320), (2050, 4100, 448), (4096, 4096, 256), (4090, 4090, 192), (2304, 8192, 64),
+               # whole stages loaded straight into LDS: every remainder of the stage count modulo the
+               # buffer rotation (three buffers at 128x256 tiles, two at 256x256), ragged tiles included
+               (2048, 4096, 256), (2048, 4096, 512), (2048, 4096, 768), (2048, 4096, 1280), (2048, 4096, 1536),
+               (4096, 4096, 512), (4096, 4096, 768), (4096, 4096, 1024), (2050, 4100, 1024), (4090, 4090, 768)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -178,7 +182,9 @@ def test_sym_dequant_bit_exact(rows, cols):
 
 @pytest.mark.parametrize("m,n,k", [(1, 64, 64), (33, 65, 128), (64, 512, 1024), (100, 200, 192), (300, 700, 11008),
                                    (512, 1024, 2048), (2048, 4096, 4096), (2048, 4096, 320), (2050, 4100, 448),
-                                   (4096, 4096, 256), (4090, 4096, 192)])
+                                   (4096, 4096, 256), (4090, 4096, 192), (2048, 4096, 512), (2048, 4096, 1280),
+                                   (4096, 4096, 768), (2050, 4096, 1024), (8, 8192, 2048), (16, 8192, 1024),
+                                   (24, 8192, 512), (48, 8192, 1024)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_linear_fused_equals_staged_reference_ops(m, n, k, with_bias):
     rng = np.random.default_rng(m + n + k)
