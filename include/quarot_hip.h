@@ -131,6 +131,23 @@ int qr_linear_i4_f16(const void* A, const void* sA, const void* W, const void* s
                      void* stream);
 
 /*
+ * The same with a caller-provided scratch buffer, for shapes whose output tiles would occupy only a
+ * fraction of the CUs (decode batches of 5..64 tokens against a narrow weight, prompts of a few
+ * hundred tokens): K is then split across workgroups, each slice leaves its int32 partial sums in
+ * `workspace` and a second kernel adds and dequantises them (two launches on `stream`).  The library never
+ * allocates (the reference's bindings allocate their outputs with torch::empty,
+ * quarot/kernels/bindings.cpp:20,39,74; here the caller does).
+ *   qr_workspace_bytes: bytes that qr_linear_i4_f16_ws can use for this shape (0: none; any M, N, K).
+ *   workspace: device memory, 16-byte aligned, at least qr_workspace_bytes(M, N, K) bytes; NULL or a
+ *   smaller size selects the single-launch path of qr_linear_i4_f16.  Results are identical bit for
+ *   bit either way (integer partial sums).  Calls that share a workspace must not overlap.
+ */
+size_t qr_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void* sW,
+                        const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * KV-cache path: optional Hadamard over the head dimension, then per-vector asymmetric int4.
  * Replaces matmul_had_cuda + asym_quantize_and_pack_i4 (quarot/transformers/kv_cache.py:10-33).
  *   x fp16 [vectors, dim], dim a power of two in [16, 256].

@@ -200,7 +200,15 @@ def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
     if bias is not None and (bias.dtype != torch.float16 or bias.numel() != N):
         raise RuntimeError("linear_i4: bias must be fp16 of size out_features")
     y = torch.empty((M, N), dtype=torch.float16, device=dev)
+    L = _lib.lib()
     with torch.cuda.device(dev):
-        _lib.check(_lib.lib().qr_linear_i4_f16(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K,
-                                               _ptr(y), _lib.stream_ptr(dev)))
+        ws_bytes = L.qr_workspace_bytes(M, N, K)
+        if ws_bytes:
+            # few output tiles: the library splits K across workgroups and needs int32 scratch for the sums
+            ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+            _lib.check(L.qr_linear_i4_f16_ws(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K, _ptr(y),
+                                             _ptr(ws), ws_bytes, _lib.stream_ptr(dev)))
+        else:
+            _lib.check(L.qr_linear_i4_f16(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K, _ptr(y),
+                                          _lib.stream_ptr(dev)))
     return y.view(*lead, N)

@@ -23,6 +23,8 @@ SIGNATURES = {
     "qr_matmul_i4_i32": (_int, (_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
     "qr_sym_dequant_i32_f16": (_int, (_ptr, _ptr, _ptr, _i64, _i64, _ptr, _ptr)),
     "qr_linear_i4_f16": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
+    "qr_workspace_bytes": (_c.c_size_t, (_i64, _i64, _i64)),
+    "qr_linear_i4_f16_ws": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _c.c_size_t, _ptr)),
     "qr_kv_quant_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _ptr, _ptr, _ptr)),
     "qr_kv_dequant_i4_f16": (_int, (_ptr, _ptr, _ptr, _i64, _int, _ptr, _ptr)),
 }

@@ -356,10 +356,13 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
 __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int ksplit) {
     constexpr int NT = 128 * WAVES_M * WAVES_N;
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
     constexpr int IM = TM / 32, JN = TN / 32;
+    // ksplit > 1 (int32 output only): the stages of K are divided among ksplit workgroups per tile;
+    // slice s writes its partial sums to the s-th [M, N] slab of C, and a second kernel adds the slabs
+    // (atomic adds into one slab were measured 3-4x slower than the whole unsplit product).
     // A stage is 128 packed bytes (256 k) per row = one full cache line, eight 16-byte chunks,
     // four 64-k sub-steps; K-group g multiplies sub-steps 2g and 2g+1.
     constexpr int CH = (BM + BN) * 8;
@@ -371,8 +374,9 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 
     const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
-    int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
-    if (tile >= tiles_m * tiles_n) return;
+    const int unit = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
+    if (unit >= tiles_m * tiles_n * ksplit) return;
+    const int tile = unit / ksplit, split = unit - tile * ksplit;   // the slices of a tile are neighbours in L2
     constexpr int GROUP_M = 8;
     const int group_sz = GROUP_M * tiles_n;
     const int g = tile / group_sz;
@@ -387,7 +391,10 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     const int wxy = wave % (WAVES_M * WAVES_N);
     const int wm = wxy / WAVES_N, wn = wxy % WAVES_N;
     const int khalf = lane >> 5;
-    const int stages = (Kb + 127) / 128;
+    const int all_stages = (Kb + 127) / 128;
+    if (ksplit > 1) C += (int64_t)split * M * N;
+    const int s_first = (int)((int64_t)all_stages * split / ksplit);
+    const int stages = (int)((int64_t)all_stages * (split + 1) / ksplit) - s_first;   // >= 1: ksplit <= all_stages
     // chunk position within a row is XOR-swizzled with (row >> 1) & 7: the 16 rows a quarter-wave
     // reads at one logical chunk cover all sixteen 16-byte bank groups (row parity picks the half)
     auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
@@ -412,7 +419,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     // partly filled last stage re-read the stage's first chunk and are zeroed when written to LDS
     const bool ragged = (Kb & 127) != 0;
     auto fetch = [&](int st, u32x4(&r)[NL]) {
-        const int kb = (st < stages ? st : stages - 1) * 128;
+        const int kb = (s_first + (st < stages ? st : stages - 1)) * 128;
         const u32 off = (u32)((kb + scoff < Kb) ? kb + scoff : kb);
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
@@ -422,7 +429,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     };
     auto deposit = [&](int st, int buf, u32x4(&r)[NL]) {
         if (st < stages) {
-            if (ragged && st == stages - 1 && st * 128 + scoff >= Kb) {
+            if (ragged && (s_first + st) * 128 + scoff >= Kb) {
 #pragma unroll
                 for (int i = 0; i < NL; ++i) r[i] = u32x4{0, 0, 0, 0};
             }
@@ -658,14 +665,15 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 // ------------------------------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
-              const void* bias, hipStream_t st) {
+              const void* bias, hipStream_t st, int ksplit = 1) {
     constexpr int NT = 128 * WAVES_M * WAVES_N;
     constexpr size_t STAGES = (size_t)3 * (BM + BN) * 8 * 16;
     constexpr size_t XCH = (size_t)WAVES_M * WAVES_N * 2 * (BN / WAVES_N / 64) * 256 * 16;
     constexpr size_t LDS = STAGES > XCH ? STAGES : XCH;
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n * ksplit;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
+    if (ksplit > 1 && Y) return QR_E_UNSUPPORTED;           // partial sums exist only as int32
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     hipError_t e;
     if (Y) {
@@ -673,13 +681,13 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
-                                                (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+                                                (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, 1);
     } else {
         auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
-                                                nullptr, nullptr, nullptr, tiles_m, tiles_n);
+                                                nullptr, nullptr, nullptr, tiles_m, tiles_n, ksplit);
     }
     return qr_launch_status();
 }
@@ -1720,8 +1728,75 @@ int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void
     return qr_launch_status();
 }
 
+// ---- K split across workgroups (shapes with too few tiles to fill the CUs) ------------------------
+// y = fp16(fp16(sA[r] * sB[c]) * fp16(acc[r, c])) (+ bias[c] as a fourth rounded operation), acc = the sum
+// of `slabs` partial products: the epilogue of the fused kernels, applied to the K slices' results.
+// Four columns per thread when rows are whole groups of four.
+__global__ __launch_bounds__(256) void dequant_slabs_kernel(const int32_t* __restrict__ part, int slabs,
+                                                            const f16* __restrict__ sA, const f16* __restrict__ sB,
+                                                            const f16* __restrict__ bias, int64_t M, int64_t N,
+                                                            f16* __restrict__ Y) {
+    const int64_t cells = M * N;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    if ((N & 3) == 0) {
+        for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < cells / 4; g += stride) {
+            const int64_t i = g * 4, r = i / N, c = i - r * N;
+            i32x4 acc = *(const i32x4*)(part + i);
+            for (int s = 1; s < slabs; ++s) acc += *(const i32x4*)(part + (int64_t)s * cells + i);
+            const f16 sa = sA[r];
+            const f16x4 sb = *(const f16x4*)(sB + c);
+            f16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f16 yv = (f16)(sa * sb[e]) * (f16)(float)acc[e];
+                if (bias) yv = yv + bias[c + e];
+                o[e] = yv;
+            }
+            *(f16x4*)(Y + i) = o;
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < cells; i += stride) {
+            const int64_t r = i / N, c = i - r * N;
+            int acc = part[i];
+            for (int s = 1; s < slabs; ++s) acc += part[(int64_t)s * cells + i];
+            f16 yv = (f16)(sA[r] * sB[c]) * (f16)(float)acc;
+            if (bias) yv = yv + bias[c];
+            Y[i] = yv;
+        }
+    }
+}
+
+// Number of K slices for the 64x256-tile kernel, 1 when the shape has no use for a split.  Only
+// prompts of a few hundred tokens qualify (64 < M, fewer than 128 tiles of 128x256): decode batches
+// were measured no faster split than with the decode kernel.  A small cost model in microseconds
+// (6 for launch + prologue + epilogue, 2 more for the second launch, 1.0 per 256-k stage and round
+// of 256 workgroups, slabs written and re-read at 4 TB/s) picks the slice count, and the split is
+// used only when it promises a fifth less time.  Against a sweep of forced slice counts on
+// M = 96..768, N = 4096..12288, K = 4096..28672 the model is within 10 % and picks the measured
+// optimum or its neighbour (e.g. 256 x 4096 x 11008: 48 -> 26 us with four slices, 256 x 8192 x
+// 28672: 119 -> 78 us with two; 512 x 4096 x 4096 and 256 x 11008 x 4096 stay unsplit).
+int ks_split(int64_t M, int64_t N, int64_t Kb) {
+    if (M <= 64 || N <= 128) return 1;
+    const int64_t tn = (N + 255) / 256;
+    if (((M + 127) / 128) * tn >= 128) return 1;
+    const int64_t tiles = ((M + 63) / 64) * tn;
+    const int64_t all_stages = (Kb + 127) / 128;
+    const double t_unsplit = 6.0 + 1.0 * (double)all_stages * (double)((tiles + 255) / 256);
+    int best = 1;
+    double t_best = 0.8 * t_unsplit;
+    for (int64_t ks = 2; ks <= 16 && ks <= all_stages / 4; ++ks) {
+        const double slabs_us = 2.0 * (double)ks * (double)M * (double)N * 4.0 / 4.0e6;
+        const double t = 8.0 + 1.0 * (double)((all_stages + ks - 1) / ks) * (double)((tiles * ks + 255) / 256) + slabs_us;
+        if (t < t_best) {
+            t_best = t;
+            best = (int)ks;
+        }
+    }
+    return best;
+}
+
 int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K, void* C, void* Y, const void* sA,
-                  const void* sB, const void* bias, hipStream_t st) {
+                  const void* sB, const void* bias, hipStream_t st, void* ws = nullptr, size_t ws_bytes = 0) {
     if (M < 0 || N < 0 || K < 0) return QR_E_SHAPE;
     if (M == 0 || N == 0) return QR_OK;
     if (K == 0 || K % 64 != 0 || K > 131008 || M > 0x7fffffff || N > 0x7fffffff) return QR_E_SHAPE;
@@ -1731,6 +1806,18 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     if (M <= 4) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    // too few tiles for the CUs: split K across workgroups when the caller passed scratch for the
+    // slices' partial sums
+    const int split = ks_split(M, N, kb);
+    if (split > 1 && Y && ws && ws_bytes >= (size_t)split * (size_t)M * (size_t)N * 4 && ((uintptr_t)ws & 15) == 0) {
+        int rc = launch_ks<64, 256, 1, 4>(A, B, m, n, kb, ws, nullptr, nullptr, nullptr, nullptr, st, split);
+        if (rc != QR_OK) return rc;
+        int64_t db = (M * N / 4 + 255) / 256;
+        db = db < 1 ? 1 : (db > 4096 ? 4096 : db);
+        dequant_slabs_kernel<<<dim3((unsigned)db), dim3(256), 0, st>>>((const int32_t*)ws, split, (const f16*)sA,
+                                                                      (const f16*)sB, (const f16*)bias, M, N, (f16*)Y);
+        return qr_launch_status();
+    }
     if (M <= 64) {
         // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
         // once per tile); otherwise eight waves split K over 32 rows
@@ -1762,4 +1849,17 @@ extern "C" int qr_linear_i4_f16(const void* A, const void* sA, const void* W, co
                                 int64_t M, int64_t N, int64_t K, void* y, void* stream) {
     if (M > 0 && N > 0 && (!y || !sA || !sW)) return QR_E_NULL;
     return gemm_dispatch(A, W, M, N, K, nullptr, y, sA, sW, bias_or_null, (hipStream_t)stream);
+}
+
+extern "C" size_t qr_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 64 != 0) return 0;
+    const int split = ks_split(M, N, K / 2);
+    return split > 1 ? (size_t)split * (size_t)M * (size_t)N * 4 : 0;
+}
+
+extern "C" int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void* sW,
+                                   const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+    if (M > 0 && N > 0 && (!y || !sA || !sW)) return QR_E_NULL;
+    return gemm_dispatch(A, W, M, N, K, nullptr, y, sA, sW, bias_or_null, (hipStream_t)stream, workspace, workspace_bytes);
 }

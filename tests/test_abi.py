@@ -29,7 +29,8 @@ def test_header_declares_expected_entry_points():
     syms = declared_symbols()
     for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
                  "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
-                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror"):
+                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4",
+                 "qr_workspace_bytes", "qr_linear_i4_f16_ws"):
         assert must in syms
 
 
@@ -71,6 +72,21 @@ def test_argument_errors_are_returned_before_any_launch(lib):
     assert lib.qr_kv_quant_f16_i4(one, 4, 100, 0, one, one, one, None) == -3
     assert lib.qr_kv_quant_f16_i4(one, 4, 128, 3, one, one, one, None) == -5
     assert lib.qr_kv_dequant_i4_f16(one, one, one, 0, 128, one, None) == 0
+
+
+def test_workspace_query_needs_no_gpu(lib):
+    """qr_workspace_bytes is pure host arithmetic: non-zero exactly for prompts of a few hundred tokens
+    whose tiles would leave most CUs idle, a whole number of [M, N] int32 slabs."""
+    assert lib.qr_workspace_bytes(2048, 4096, 11008) == 0          # enough tiles
+    assert lib.qr_workspace_bytes(8, 8192, 28672) == 0             # decode batches use the decode kernel
+    assert lib.qr_workspace_bytes(512, 11008, 4096) == 0           # short K: nothing to split
+    for m, n, k in ((256, 4096, 11008), (128, 4096, 4096), (96, 8192, 8192), (256, 8192, 28672)):
+        ws = lib.qr_workspace_bytes(m, n, k)
+        assert ws > 0 and ws % (m * n * 4) == 0 and 2 <= ws // (m * n * 4) <= 16
+    assert lib.qr_workspace_bytes(0, 4096, 4096) == 0 and lib.qr_workspace_bytes(256, 4096, 100) == 0
+    one = ctypes.c_void_p(16)
+    assert lib.qr_linear_i4_f16_ws(one, None, one, one, None, 4, 4, 64, one, None, 0, None) == -1
+    assert lib.qr_linear_i4_f16_ws(one, one, one, one, None, 4, 4, 100, one, None, 0, None) == -2
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -203,6 +203,41 @@ def test_linear_fused_equals_staged_reference_ops(m, n, k, with_bias):
     assert torch.equal(staged, y)
 
 
+@pytest.mark.parametrize("m,n,k", [(128, 4096, 4096), (300, 700, 11008), (96, 512, 8192), (130, 520, 4160),
+                                   (256, 4096, 11008)])
+def test_linear_with_workspace_splits_k_and_matches_bit_for_bit(m, n, k):
+    """Shapes with few output tiles: with the scratch buffer the library splits K across workgroups
+    (int32 partial sums in slabs, then one summing dequantisation); the result must equal both the
+    oracle and the single-launch path bit for bit, with and without bias, and a missing or too small
+    workspace must silently select the single-launch path."""
+    L = _lib.lib()
+    ws_bytes = L.qr_workspace_bytes(m, n, k)
+    assert ws_bytes > 0
+    rng = np.random.default_rng(m + n + k)
+    a = o.pack_i4(rng.integers(-8, 8, (m, k)))
+    w = o.pack_i4(rng.integers(-8, 8, (n, k)))
+    sa = (np.abs(rng.standard_normal(m)) * 0.2).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01).astype(F16)
+    bias = rng.standard_normal(n).astype(F16)
+    ga, gw, gsa, gsw, gb = gpu(a), gpu(w), gpu(sa), gpu(sw), gpu(bias)
+    st = torch.cuda.current_stream().cuda_stream
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=ga.device)
+    for b_np, b_gpu in ((None, None), (bias, gb)):
+        want = o.linear4bit(a, sa, w, sw, b_np)
+        outs = []
+        for wptr, wbytes in ((ws.data_ptr(), ws_bytes), (None, 0), (ws.data_ptr(), ws_bytes - 4)):
+            y = torch.full((m, n), float("nan"), dtype=torch.float16, device=ga.device)
+            rc = L.qr_linear_i4_f16_ws(ga.data_ptr(), gsa.data_ptr(), gw.data_ptr(), gsw.data_ptr(),
+                                       None if b_gpu is None else b_gpu.data_ptr(), m, n, k, y.data_ptr(), wptr, wbytes, st)
+            assert rc == 0
+            outs.append(y.cpu().numpy())
+        for got in outs:
+            assert np.array_equal(bits(got), bits(want))
+        # the Python entry point takes the split path by itself
+        y = quarot_amd.linear_i4(ga, gsa, gw, gsw, b_gpu)
+        assert np.array_equal(bits(y.cpu().numpy()), bits(want))
+
+
 def test_linear4bit_module_from_float_and_state_dict():
     w = (torch.randn(96, 128, generator=torch.Generator().manual_seed(4)) * 0.02).half()
     s = (w.abs().amax(dim=1, keepdim=True) / 7).half()
