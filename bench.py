@@ -13,6 +13,8 @@ outlier channels that motivate the Hadamard):
     c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
     c4  down_proj 70B decode  X [64, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28
         (c4m1, c4m8: 1 / 8 tokens; c4g1, c4g8, c4g64: gate_up W int4 [57344, 8192])
+    c5  KV-cache write path of one layer: K and V [32, 4096, 8, 128] fp16 -> asymmetric int4 per head
+        vector (K through the head-dimension Hadamard first); metric GB/s of algorithmic bytes
 Decode workloads (M <= 64) rotate among several copies of the weights so that they are streamed from
 HBM rather than from the 256 MB last-level cache.
 Prints ONE JSON line on stdout (metric = TOPS of the whole step, 2.M.N.K / t).
@@ -42,6 +44,7 @@ WORKLOADS = {
     "c4g1": (1, 8192, 57344, False),        # decode, 70B gate_up (input already quantised upstream: no Hadamard)
     "c4g8": (8, 8192, 57344, False),
     "c4g64": (64, 8192, 57344, False),
+    "c5": (0, 0, 0, False),                 # KV-cache quantisation (separate code path below)
 }
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 HBM_PEAK_GBS = 8000.0
@@ -59,6 +62,7 @@ TRAFFIC_KIB = {
     "c4": (72440.1, 1024.0),
     "c4m1": (61875.4, 16.0),
     "c4g64": (115876.5, 7168.0),
+    "c5": (131104.3, 69637.5),              # kv_quant_kernel with Hadamard (K cache), per launch
 }
 
 
@@ -104,6 +108,76 @@ def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=
                       + "fp16 sym quant + int32 torch matmul + fp16 dequant"}
 
 
+def bench_kv(args, dev):
+    """Workload c5: quantise K (Hadamard over the head dimension, then asymmetric int4) and V
+    (asymmetric int4) of one layer, [32, 4096, 8, 128] fp16 each, resident in HBM."""
+    from quarot_amd.transformers import kv_cache as kv
+    shape = (32, 4096, 8, 128)
+
+    def synth(seed):
+        g = torch.Generator().manual_seed(seed)
+        t = torch.randn(shape, generator=g)
+        mask = torch.rand(shape, generator=torch.Generator().manual_seed(5)) < 0.005
+        t[mask] *= 15
+        return t.half()
+
+    k_cpu, v_cpu = synth(4), synth(6)
+    k, v = k_cpu.to(dev), v_cpu.to(dev)
+    vectors = k.numel() // 128
+    bytes_one = 2 * k.numel() + vectors * (64 + 4)          # fp16 in; codes + scale + zero out
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        kq = kv.asym_quantize_and_pack_i4(k, hadamard=True)
+        if ev is not None:
+            ev[1].record()
+        vq = kv.asym_quantize_and_pack_i4(v, hadamard=False)
+        return kq, vq
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    k_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    traffic = None
+    if TRAFFIC_KIB.get("c5"):
+        f, w = TRAFFIC_KIB["c5"]
+        traffic = round((f * FETCH_SCALE + w * WRITE_SCALE) * 1024)
+    roof = {"bound": "hbm", "achieved": round(bytes_one / (k_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "traffic": traffic}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["kernel"] = "kv_quant_kernel<128, Hadamard> (K cache)"
+    roof["kernel_ms"] = round(k_ms, 4)
+    out = {
+        "metric": "KV-cache int4 quantise GB/s (K with Hadamard + V)", "value": round(2 * bytes_one / (ms * 1e-3) / 1e9, 1),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 -> u4 (fp32 Hadamard, fp16 quantiser)",
+        "data": "synthetic",
+        "config": {"workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector",
+                   "vectors_per_tensor": vectors, "head_dim": 128},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        from oracle import quarot_oracle as o
+        n = vectors // 256                                   # 4096 vectors of each tensor
+        ks, vs = k_cpu.reshape(-1, 128)[:n].numpy(), v_cpu.reshape(-1, 128)[:n].numpy()
+        t0 = time.perf_counter()
+        o.kv_asym_quant(o.kv_hadamard(ks))
+        o.kv_asym_quant(vs)
+        t = time.perf_counter() - t0
+        sample_bytes = 2 * (2 * ks.size + n * 68)
+        out["cpu_baseline"] = {"value": round(sample_bytes / t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"first {n} of {vectors} vectors of each tensor ({t * 1e3:.0f} ms); numpy oracle "
+                                         f"(fp32 FWHT + fp16 asymmetric quantiser)"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,6 +210,8 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"launches": 20, "read_bytes": src.numel(), "written_bytes": src.numel()}}))
         return
+    if args.workload == "c5":
+        return bench_kv(args, dev)
     m, k, n, hadamard = WORKLOADS[args.workload]
     x_cpu = synth_x(m, k, seed=0, outliers=True)
     w_cpu, sw_cpu = synth_w(n, k, seed=1)
