@@ -62,7 +62,7 @@ TRAFFIC_KIB = {
     "c4": (72440.1, 1024.0),
     "c4m1": (61875.4, 16.0),
     "c4g64": (115876.5, 7168.0),
-    "c5": (131104.3, 69637.5),              # kv_quant_kernel with Hadamard (K cache), per launch
+    "c5": (131145.2, 69808.6),              # kv_had128_kernel (K cache), per launch
 }
 
 
@@ -152,7 +152,7 @@ def bench_kv(args, dev):
     roof = {"bound": "hbm", "achieved": round(bytes_one / (k_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "traffic": traffic}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = "kv_quant_kernel<128, Hadamard> (K cache)"
+    roof["kernel"] = "kv_had128_kernel (K cache: Hadamard on the matrix cores + asymmetric int4)"
     roof["kernel_ms"] = round(k_ms, 4)
     out = {
         "metric": "KV-cache int4 quantise GB/s (K with Hadamard + V)", "value": round(2 * bytes_one / (ms * 1e-3) / 1e9, 1),

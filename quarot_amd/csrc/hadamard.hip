@@ -1341,6 +1341,8 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    // head-dimension rows: the kernel whose arithmetic the K-cache quantiser shares
+    if (dtype == QR_DTYPE_F16 && K == 1 && n == 128) return qr_internal_hadamard128_f16(x, y, rows, scale, st);
     if (dtype == QR_DTYPE_F16 && K == 1 && pow2_split(n))
         return launch_hadamard_mm<true, false>(x, y, rows, n, pow2_split(n), nullptr, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && bm_applies(n, K))

@@ -203,6 +203,235 @@ __global__ __launch_bounds__(KT) void kv_dequant_kernel(const u32* __restrict__ 
     }
 }
 
+// ---- head dimension 128 with the Hadamard: the transform on the matrix cores ----------------------
+// Seven butterfly stages cost 11.5 vector instructions per element (a cross-lane stage is two
+// instructions per element however it is written) and bound the kernel above at ~3 TB/s.  Here a
+// wave takes 32 vectors at a time and computes Y^T = H_128 . X^T with v_mfma_f32_32x32x16_f16:
+//   * first operand: H_128 tiles (32 outputs j x 16 inputs k).  H[j][k] = (-1)^popcount(j & k) factors
+//     by index bits: tile (jt, ks) is a base tile that depends on ks & 1 only, times the wave-uniform
+//     sign (-1)^popcount(jt & (ks >> 1)).  Two base tiles and their negations: 16 registers.
+//   * second operand: X^T, lane (vector v = lane % 32, half h = lane / 32) supplies 8 consecutive
+//     inputs of ITS vector: 16 bytes of the vector's row.  The 8 KB block of 32 rows is fetched with
+//     coalesced 16-byte loads one block ahead, staged in a wave-private LDS region (pieces XOR-keyed by
+//     the row) and read back as fragments: no workgroup barrier anywhere in the kernel.
+//   * result: lane (v, h) holds outputs j = 32 jt + 8 q + 4 h + (0..3) of vector v, i.e. 64 of the 128
+//     outputs of one vector (lane ^ 32 holds the others).  Scaling, fp16 rounding, min / max (packed,
+//     in-lane, then one exchange with lane ^ 32) and the codes stay in the lane; four
+//     v_permlane32_swap then give lane h the 32 contiguous output bytes [32 h, 32 h + 32) of its
+//     vector, so a wave writes 2 KB of consecutive codes.
+// The fp32 sums are formed in the matrix core's order, not the butterflies': the plain transform of a
+// 128-wide row (qr_hadamard, used by matmul_had_cuda) runs through the same kernel (QUANT = false),
+// so that codes remain those of the quantiser applied to that transform's output, bit for bit.
+constexpr int KM_WAVES = 4;
+
+__device__ __forceinline__ int km_slot(int row, int piece) { return row * 16 + (piece ^ (row & 15)); }
+
+template <bool QUANT>
+__global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4* __restrict__ x, int64_t vectors,
+                                                                     float hscale, u32x4* __restrict__ q,
+                                                                     f16* __restrict__ scale, f16* __restrict__ zero,
+                                                                     u32x4* __restrict__ y) {
+    __shared__ u32x4 km_lds[KM_WAVES * 512];                       // 8 KB per wave
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int v = lane & 31, h = lane >> 5;
+    u32x4* stage = km_lds + wave * 512;
+
+    // base tiles of H_128 for ks even / odd: row j = v (jt = 0), inputs k = 16 (ks & 1) + 8 h + e
+    f16x8 hb[2], hn[2];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const bool neg = (__builtin_popcount(v & (16 * o + 8 * h + e)) & 1) != 0;
+            hb[o][e] = neg ? (f16)-1.0f : (f16)1.0f;
+            hn[o][e] = neg ? (f16)1.0f : (f16)-1.0f;
+        }
+
+    const int64_t blocks = (vectors + 31) >> 5;
+    const int64_t wstride = (int64_t)gridDim.x * KM_WAVES;
+    int64_t blk = (int64_t)blockIdx.x * KM_WAVES + wave;
+    // block of 32 rows = 512 pieces of 16 bytes; load c takes pieces 64 c + lane: row 4 c + lane / 16
+    u32x4 pre[8];
+    auto fetch = [&](int64_t b) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            int64_t row = b * 32 + 4 * c + (lane >> 4);
+            row = row < vectors ? row : vectors - 1;               // the last block may be short: repeat its last row
+            pre[c] = x[row * 16 + (lane & 15)];
+        }
+    };
+    if (blk < blocks) fetch(blk);
+    for (; blk < blocks; blk += wstride) {
+        // LDS operations of one wave execute in order: these writes follow the previous block's reads
+#pragma unroll
+        for (int c = 0; c < 8; ++c) stage[km_slot(4 * c + (lane >> 4), lane & 15)] = pre[c];
+        if (blk + wstride < blocks) fetch(blk + wstride);
+        u32x4 xf[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) xf[ks] = stage[km_slot(v, 2 * ks + h)];
+        f32x16 acc[4];
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[jt][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const bool neg = (__builtin_popcount(jt & (ks >> 1)) & 1) != 0;     // compile-time after unrolling
+                acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(neg ? hn[ks & 1] : hb[ks & 1],
+                                                                 __builtin_bit_cast(f16x8, xf[ks]), acc[jt], 0, 0, 0);
+            }
+        }
+        // scaled, rounded outputs: yq[jt][qq] = the four outputs j = 32 jt + 8 qq + 4 h + (0..3), two per word
+        u32 yw[4][4][2];
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq) {
+                yw[jt][qq][0] = narrow_f16x2(acc[jt][4 * qq] * hscale, acc[jt][4 * qq + 1] * hscale);
+                yw[jt][qq][1] = narrow_f16x2(acc[jt][4 * qq + 2] * hscale, acc[jt][4 * qq + 3] * hscale);
+            }
+        const int64_t vec = blk * 32 + v;
+        if (!QUANT) {
+            // back through the staging region (all fragment reads are done): 8-byte pieces in, rows out
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) {
+                    const int piece = 4 * jt + qq;                 // 16-byte piece of the row; this lane's half h of it
+                    ((u32x2*)stage)[km_slot(v, piece) * 2 + h] = u32x2{yw[jt][qq][0], yw[jt][qq][1]};
+                }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const int row = 4 * c + (lane >> 4);
+                const u32x4 o = stage[km_slot(row, lane & 15)];
+                if (blk * 32 + row < vectors) y[(blk * 32 + row) * 16 + (lane & 15)] = o;
+            }
+            continue;
+        }
+        // ---- quantiser on the lane's 64 values
+        u16x2 am2 = {0, 0};                                        // largest magnitude bits: >= 0x7c00 means inf or NaN
+#pragma unroll
+        for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+            for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+                for (int w = 0; w < 2; ++w)
+                    am2 = __builtin_elementwise_max(am2, __builtin_bit_cast(u16x2, yw[jt][qq][w] & 0x7fff7fffu));
+        const u32 amax = am2[0] > am2[1] ? am2[0] : am2[1];
+        const bool finite = __builtin_amdgcn_ballot_w64(amax >= 0x7c00u) == 0;
+        f16 sc, zp;
+        u32 U[8];
+        if (finite) {
+            f16x2 mn2 = as_f16x2(yw[0][0][0]), mx2 = mn2;
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        mn2 = __builtin_elementwise_min(mn2, as_f16x2(yw[jt][qq][w]));
+                        mx2 = __builtin_elementwise_max(mx2, as_f16x2(yw[jt][qq][w]));
+                    }
+            const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+            const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            f16x2 pr = {mn0, -mx0};                                // (min, -max): one packed min across the two lanes
+            const f16x2 other = as_f16x2((u32)__shfl_xor((int)__builtin_bit_cast(u32, pr), 32, 64));
+            pr = __builtin_elementwise_min(pr, other);
+            const f16 mn = pr[0], mx = -pr[1];
+            f16 rng = narrow_f16((float)mx - (float)mn);
+            const f16 floor_ = (f16)1e-5f;
+            rng = rng < floor_ ? floor_ : rng;
+            sc = narrow_f16((float)rng * (1.0f / 15.0f));
+            zp = -mn;
+            const FastRecip fr = make_fast_recip((float)sc);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                const int jt = m >> 1, q0 = (m & 1) * 2;
+                U[m] = asym_codes8_fast(u32x4{yw[jt][q0][0], yw[jt][q0][1], yw[jt][q0 + 1][0], yw[jt][q0 + 1][1]}, zp, fr);
+            }
+        } else {
+            // a NaN anywhere in a vector makes its range, scale and zero NaN and every code 0 (torch's
+            // min / max propagate it); infinities follow the IEEE operations of the reference
+            float mn = __builtin_inff(), mx = -__builtin_inff();
+            bool has_nan = false;
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq)
+#pragma unroll
+                    for (int w = 0; w < 2; ++w) {
+                        const f16x2 p = as_f16x2(yw[jt][qq][w]);
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            const float t = (float)p[e];
+                            has_nan = has_nan || (t != t);
+                            mn = t < mn ? t : mn;
+                            mx = t > mx ? t : mx;
+                        }
+                    }
+            const float omn = __shfl_xor(mn, 32, 64), omx = __shfl_xor(mx, 32, 64);
+            has_nan = has_nan || (__shfl_xor((int)has_nan, 32, 64) != 0);
+            mn = omn < mn ? omn : mn;
+            mx = omx > mx ? omx : mx;
+            if (has_nan) mn = mx = __builtin_nanf("");
+            f16 rng = (f16)(mx - mn);
+            const f16 floor_ = (f16)1e-5f;
+            rng = rng < floor_ ? floor_ : rng;                     // NaN < x is false: NaN stays
+            sc = (f16)(float)((double)(float)rng / 15.0);
+            zp = (f16)(-mn);
+            const float s = (float)sc, z = (float)zp;
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                const int jt = m >> 1, q0 = (m & 1) * 2;
+                u32 word = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f16x2 p = as_f16x2(yw[jt][q0 + (i >> 1)][i & 1]);
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const float sh = (float)(f16)((float)p[e] + z);
+                        const float r = __builtin_rintf((float)(f16)(sh / s));
+                        int code = (int)r;
+                        code = code < 0 ? 0 : (code > 15 ? 15 : code);
+                        code = (r != r) ? 0 : code;
+                        word |= (u32)code << (4 * (2 * i + e));
+                    }
+                }
+                U[m] = word;
+            }
+        }
+        // U[m] = (piece 2m, piece 2m + 1) of this lane's sixteen 2-byte pieces; pieces of the two lanes
+        // of a vector interleave.  After the swaps lane h holds both lanes' pieces of words 8 h .. 8 h + 7.
+        u32 W[8];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const auto sw = __builtin_amdgcn_permlane32_swap(U[m], U[m + 4], false, false);
+            W[2 * m] = __builtin_amdgcn_perm(sw[1], sw[0], 0x05040100u);
+            W[2 * m + 1] = __builtin_amdgcn_perm(sw[1], sw[0], 0x07060302u);
+        }
+        if (vec < vectors) {
+            q[vec * 4 + 2 * h] = u32x4{W[0], W[1], W[2], W[3]};
+            q[vec * 4 + 2 * h + 1] = u32x4{W[4], W[5], W[6], W[7]};
+            if (h == 0) {
+                scale[vec] = sc;
+                zero[vec] = zp;
+            }
+        }
+    }
+}
+
+template <bool QUANT>
+int launch_had128(const void* x, int64_t vectors, float hscale, void* q, void* scale, void* zero, void* y, hipStream_t st) {
+    auto kern = kv_had128_kernel<QUANT>;
+    const int64_t blocks = (vectors + 31) >> 5;
+    const int64_t want = (blocks + KM_WAVES - 1) / KM_WAVES;
+    const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, 64 * KM_WAVES, 0);
+    const unsigned grid = (unsigned)(want < cap ? want : cap);
+    kern<<<dim3(grid), dim3(64 * KM_WAVES), 0, st>>>((const u32x4*)x, vectors, hscale, (u32x4*)q, (f16*)scale, (f16*)zero,
+                                                    (u32x4*)y);
+    return qr_launch_status();
+}
+
 int log2_dim(int dim) {
     for (int l = 4; l <= 8; ++l)
         if ((1 << l) == dim) return l;
@@ -229,6 +458,8 @@ extern "C" int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int h
     const int64_t nchunks = vectors * (dim / 8);
     const float hs = (float)(1.0 / __builtin_sqrt((double)dim));
     hipStream_t st = (hipStream_t)stream;
+    if (dim == 128 && had_mode == 1 && (((uintptr_t)q & 15) == 0))
+        return launch_had128<true>(x, vectors, hs, q, scale, zero, nullptr, st);
     dim3 grid(grid_for(nchunks)), block(KT);
 #define QR_KV(LG)                                                                                                     \
     case LG + 3:                                                                                                      \
@@ -244,6 +475,12 @@ extern "C" int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int h
     }
 #undef QR_KV
     return qr_launch_status();
+}
+
+// The plain transform of 128-wide fp16 rows with the arithmetic of the fused kernel (see above).
+__attribute__((visibility("hidden"))) int qr_internal_hadamard128_f16(const void* x, void* y, int64_t rows, float scale,
+                                                                      hipStream_t st) {
+    return launch_had128<false>(x, rows, scale, nullptr, nullptr, nullptr, y, st);
 }
 
 extern "C" int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void* zero, int64_t vectors, int dim,

@@ -66,6 +66,9 @@ static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) 
     return blocks;
 }
 
+// kv.hip: y = x . H_128 * scale on rows of 128 halves (matrix-core kernel shared with the K-cache quantiser)
+int qr_internal_hadamard128_f16(const void* x, void* y, int64_t rows, float scale, hipStream_t st);
+
 static inline int qr_launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? QR_OK : (int)e;

@@ -438,6 +438,36 @@ def test_kv_vectors_with_infinities_take_the_ieee_path():
     assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
 
 
+def test_kv_hadamard_128_blocks_tails_and_infinities():
+    """Head dimension 128 with the Hadamard runs on the matrix cores, 32 vectors per wave step: vector
+    counts around the block size, equality of the fused codes with the quantiser applied to the plain
+    transform of the same kernel, and an infinite input (every output of that vector is +-inf: scale
+    and zero infinite, all codes 0) that must not disturb its neighbours."""
+    rng = np.random.default_rng(128)
+    for vecs in (1, 31, 32, 33, 95, 257, 4100):
+        x = rng.standard_normal((vecs, 128)).astype(F16)
+        q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=True)
+        xh = kv.matmul_had_cuda(gpu(x), torch.float16).cpu().numpy()
+        assert close(xh, o.kv_hadamard(x))
+        wq, ws, wz = o.kv_asym_quant(xh)
+        assert np.array_equal(q.cpu().numpy(), wq)
+        assert np.array_equal(bits(s.cpu().numpy()), bits(ws)) and np.array_equal(bits(z.cpu().numpy()), bits(wz))
+    x = rng.standard_normal((70, 128)).astype(F16)
+    x[40, 9] = np.inf
+    q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=True)
+    xh = kv.matmul_had_cuda(gpu(x), torch.float16).cpu().numpy()
+    q, s, z = q.cpu().numpy(), s.cpu().numpy(), z.cpu().numpy()
+    assert np.all(np.isinf(xh[40])) and np.isposinf(s[40, 0]) and np.isposinf(z[40, 0]) and np.all(q[40] == 0)
+    keep = [i for i in range(70) if i != 40]
+    wq, ws, wz = o.kv_asym_quant(xh[keep])
+    assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
+    # in place, as qr_hadamard allows
+    t = gpu(x[:50].copy())
+    rc = _lib.lib().qr_hadamard(t.data_ptr(), t.data_ptr(), 50, 128, 1, None, 0, 1.0 / np.sqrt(128.0),
+                                torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and np.array_equal(bits(t.cpu().numpy()), bits(xh[:50]))
+
+
 def test_kv_full_size_round_trip():
     """The benchmark tensor [32, 4096, 8, 128]: codes in range, extremes hit, error bound, and a
     strided sample against the oracle."""
