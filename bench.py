@@ -185,6 +185,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of the step captured in a HIP graph (decode steps are host-launch-bound when "
+                         "launched eagerly from Python); the first replay is checked against the eager result")
     ap.add_argument("--cpu-rows", type=int, default=64)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of a workload, run a plain 256 MiB device copy 20 times (known traffic: 256 MiB read, "
@@ -245,13 +248,36 @@ def main():
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(events[i])
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms = (t1 - t0) * 1e3 / args.steps
-    gemm_ms = float(np.mean([a.elapsed_time(b) for a, b in events]))
+    if args.graph:
+        # one graph per weight copy would defeat the rotation: capture a run of len(copies) steps
+        state["i"] = 0
+        want = step().clone()
+        state["i"] = 0
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [step() for _ in range(len(copies))]
+        graph.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(outs[0], want):
+            raise RuntimeError("graph replay differs from the eager step")
+        reps = max(1, args.steps // len(copies))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / (reps * len(copies))
+        for i in range(min(args.steps, 20)):                # GEMM time from eager launches (events cannot go into the graph)
+            step(events[i])
+        torch.cuda.synchronize()
+        gemm_ms = float(np.mean([a.elapsed_time(b) for a, b in events[:min(args.steps, 20)]]))
+    else:
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(events[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ms = (t1 - t0) * 1e3 / args.steps
+        gemm_ms = float(np.mean([a.elapsed_time(b) for a, b in events]))
     ops = 2.0 * m * n * k
     value = ops / (ms * 1e-3) / 1e12
 
@@ -319,7 +345,7 @@ def main():
                    "M": m, "K": k, "N": n,
                    "path": ("fused Hadamard+quantise kernel" if hadamard else "fused RMSNorm+quantise kernel" if rmsnorm
                             else "quantise kernel") + ", fused GEMM+dequant kernel",
-                   "staged_reference_api_ms": round(staged_ms, 4)},
+                   "staged_reference_api_ms": round(staged_ms, 4), "launch": "hip graph replay" if args.graph else "eager"},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:

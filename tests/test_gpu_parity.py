@@ -438,6 +438,36 @@ def test_kv_vectors_with_infinities_take_the_ieee_path():
     assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
 
 
+def test_decode_step_replays_from_a_hip_graph():
+    """A decode step (fused Hadamard+quantise, then the decode GEMM) captured into a HIP graph: every
+    replay, with fresh inputs copied into the static buffer and eager work plus synchronisation between
+    the replays, must equal the eager result bit for bit.  The library launches on the stream it is
+    given and allocates nothing, so capture needs no special path."""
+    k, n = 5120, 1024                                   # had_40 x FWHT(128), decode-size GEMM
+    w, sw = synth_w(n, k, seed=11)
+    lin = quarot_amd.nn.Linear4bit(k, n).half().cuda()
+    lin.weight.copy_(gpu(w)); lin.weight_scales.copy_(gpu(sw))
+    front = quarot_amd.nn.OnlineHadamardQuantizer(k).cuda()
+    xs = [gpu(synth_x(8, k, seed=20 + i)) for i in range(4)]
+    static_x = xs[0].clone()
+    for _ in range(2):                                  # warm-up outside capture (launch attributes are cached here)
+        lin(front(static_x))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = lin(front(static_x))
+    for i, x in enumerate(xs):
+        eager = lin(front(x))                           # eager work between replays
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, eager), f"replay {i}"
+        p = front(x)
+        wq, ws = o.quantizer(quarot_amd.nn.OnlineHadamard(k).cuda()(x).cpu().numpy())
+        assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+
+
 def test_kv_hadamard_128_blocks_tails_and_infinities():
     """Head dimension 128 with the Hadamard runs on the matrix cores, 32 vectors per wave step: vector
     counts around the block size, equality of the fused codes with the quantiser applied to the plain
