@@ -151,6 +151,32 @@ def test_matmul_int32_bit_exact(m, n, k):
     assert np.array_equal(c.cpu().numpy(), o.int4_matmul(a, b))
 
 
+def test_matmul_and_linear_random_shapes_across_every_kernel_boundary():
+    """Seeded random shapes around the dispatcher's thresholds (matrix-vector <= 4 rows, decode <= 64,
+    tile counts that select the 64x256, 128x256 and 256x256 kernels, whole and ragged K stages, the
+    workspace split): int32 product and fused fp16 output against the oracle, bit for bit."""
+    rng = np.random.default_rng(2024)
+    shapes = []
+    for _ in range(14):
+        shapes.append((int(rng.integers(1, 200)), int(rng.integers(1, 700)), 64 * int(rng.integers(1, 17))))
+    for m in (4, 5, 64, 65):
+        shapes.append((m, int(rng.integers(250, 530)), 64 * int(rng.integers(1, 9))))
+    for _ in range(6):                                   # enough tiles for the pipelined kernels
+        shapes.append((int(rng.integers(1800, 2300)), int(rng.integers(3900, 4300)), 64 * int(rng.integers(1, 13))))
+    shapes += [(70, 300, 4096), (140, 1030, 2048), (2048, 8192, 256), (4100, 4100, 512)]
+    for (m, n, k) in shapes:
+        a = o.pack_i4(rng.integers(-8, 8, (m, k)))
+        w = o.pack_i4(rng.integers(-8, 8, (n, k)))
+        want = o.int4_matmul(a, w)
+        c = quarot_amd.matmul(gpu(a), gpu(w))
+        assert np.array_equal(c.cpu().numpy(), want), (m, n, k)
+        sa = (np.abs(rng.standard_normal(m)) * 0.2 + 0.01).astype(F16)
+        sw = (np.abs(rng.standard_normal(n)) * 0.01 + 0.001).astype(F16)
+        bias = rng.standard_normal(n).astype(F16)
+        y = quarot_amd.linear_i4(gpu(a), gpu(sa), gpu(w), gpu(sw), gpu(bias))
+        assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw, bias))), (m, n, k)
+
+
 def test_matmul_known_answers_and_leading_dims():
     k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
     a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
