@@ -11,6 +11,9 @@ outlier channels that motivate the Hadamard):
     c1n the same with the RMSNorm in front of the quantiser (fused RMSNorm + Quantizer kernel)
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
     c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
+    c3  the four linears of a 7B decoder layer at 32768 tokens as ONE step: fused qkv 4096->12288, o 4096->4096,
+        gate_up 4096->22016 (Quantizer in front of each) and down 11008->4096 (Hadamard+Quantizer): 13.26 TOP
+        (c3a, c3b, c3c: the first three on their own)
     c4  down_proj 70B decode  X [64, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28
         (c4m1, c4m8: 1 / 8 tokens; c4g1, c4g8, c4g64: gate_up W int4 [57344, 8192])
     c5  KV-cache write path of one layer: K and V [32, 4096, 8, 128] fp16 -> asymmetric int4 per head
@@ -38,6 +41,12 @@ WORKLOADS = {
     "c1n": (2048, 4096, 4096, False),       # input_layernorm -> Quantizer -> q_proj
     "c2": (2048, 11008, 4096, True),
     "c3d": (32768, 11008, 4096, True),
+    "c3a": (32768, 4096, 12288, False),     # fused qkv
+    "c3b": (32768, 4096, 4096, False),      # o_proj
+    "c3c": (32768, 4096, 22016, False),     # gate_up
+    "c3": (0, 0, 0, False),                 # the whole layer set (separate code path below)
+    "c4m32": (32, 28672, 8192, True),
+    "c4g32": (32, 8192, 57344, False),
     "c4": (64, 28672, 8192, True),          # decode, 70B down_proj
     "c4m1": (1, 28672, 8192, True),
     "c4m8": (8, 28672, 8192, True),
@@ -134,7 +143,9 @@ def bench_kv(args, dev):
         if ev is not None:
             ev[1].record()
         vq = kv.asym_quantize_and_pack_i4(v, hadamard=False)
-        return kq, vq
+        kd = kv.unpack_i4_and_asym_dequantize(*kq)          # the round trip of the config
+        vd = kv.unpack_i4_and_asym_dequantize(*vq)
+        return kd, vd
 
     for _ in range(args.warmup):
         step()
@@ -155,11 +166,12 @@ def bench_kv(args, dev):
     roof["kernel"] = "kv_had128_kernel (K cache: Hadamard on the matrix cores + asymmetric int4)"
     roof["kernel_ms"] = round(k_ms, 4)
     out = {
-        "metric": "KV-cache int4 quantise GB/s (K with Hadamard + V)", "value": round(2 * bytes_one / (ms * 1e-3) / 1e9, 1),
+        "metric": "KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)", "value": round(4 * bytes_one / (ms * 1e-3) / 1e9, 1),
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 -> u4 (fp32 Hadamard, fp16 quantiser)",
         "data": "synthetic",
-        "config": {"workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector",
+        "config": {"workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector "
+                               "-> fp16 again (four launches)",
                    "vectors_per_tensor": vectors, "head_dim": 128},
         "roofline": roof,
     }
@@ -175,6 +187,65 @@ def bench_kv(args, dev):
         out["cpu_baseline"] = {"value": round(sample_bytes / t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"first {n} of {vectors} vectors of each tensor ({t * 1e3:.0f} ms); numpy oracle "
                                          f"(fp32 FWHT + fp16 asymmetric quantiser)"}
+    print(json.dumps(out))
+
+
+def bench_layer(args, dev):
+    """Workload c3: the four W4A4 linears of a Llama-2-7B decoder layer at M = 32768 tokens (prefill,
+    16 x 2048) as one step; inputs of each linear are separate seeded tensors resident in HBM."""
+    import quarot_amd
+    m = 32768
+    parts = [("qkv", 4096, 12288, False, 0), ("o", 4096, 4096, False, 10), ("gate_up", 4096, 22016, False, 20),
+             ("down", 11008, 4096, True, 30)]
+    mods = []
+    for name, k, n, had, seed in parts:
+        x = synth_x(m, k, seed=seed, outliers=True).to(dev)
+        w, sw = synth_w(n, k, seed=seed + 1)
+        lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
+        lin.weight.copy_(w.to(dev))
+        lin.weight_scales.copy_(sw.to(dev))
+        front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if had else quarot_amd.nn.Quantizer()).to(dev)
+        mods.append((x, front, lin))
+    ops = sum(2.0 * m * k * n for _, k, n, _, _ in parts)
+    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in parts]
+           for _ in range(args.steps)]
+
+    def step(ev=None):
+        for j, (x, front, lin) in enumerate(mods):
+            p = front(x)
+            if ev is not None:
+                ev[j][0].record()
+            y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None)
+            if ev is not None:
+                ev[j][1].record()
+            del y                                           # 0.8 - 1.4 GB each: returned to the pool before the next one
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(evs[i])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gemm = [float(np.mean([evs[i][j][0].elapsed_time(evs[i][j][1]) for i in range(args.steps)])) for j in range(len(parts))]
+    gemm_ms = sum(gemm)
+    roof = {"bound": "mfma", "achieved": round(ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
+            "unit": "TFLOP/s", "traffic": None}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["kernel"] = "gemm_sp256_kernel (int4 GEMM + dequant epilogue), four launches"
+    roof["kernel_ms"] = round(gemm_ms, 4)
+    roof["per_linear"] = {name: {"ms": round(t, 4), "TOPS": round(2.0 * m * k * n / (t * 1e-3) / 1e12, 1)}
+                          for (name, k, n, _, _), t in zip(parts, gemm)}
+    out = {
+        "metric": "Linear4bit TOPS (had+quant+GEMM)", "value": round(ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 scales", "data": "synthetic",
+        "config": {"workload": "c3: Llama-2-7B decoder-layer linear set at M=32768 (qkv 4096->12288, o 4096->4096, "
+                               "gate_up 4096->22016, down 11008->4096 with online Hadamard), W4A4",
+                   "M": m, "total_TOP": round(ops / 1e12, 2)},
+        "roofline": roof,
+    }
     print(json.dumps(out))
 
 
@@ -215,6 +286,8 @@ def main():
         return
     if args.workload == "c5":
         return bench_kv(args, dev)
+    if args.workload == "c3":
+        return bench_layer(args, dev)
     m, k, n, hadamard = WORKLOADS[args.workload]
     x_cpu = synth_x(m, k, seed=0, outliers=True)
     w_cpu, sw_cpu = synth_w(n, k, seed=1)
