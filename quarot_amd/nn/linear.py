@@ -3,23 +3,39 @@ import torch
 import quarot_amd
 
 
-class Linear4bit(torch.nn.Module):
-    """Symmetric W4A4 linear layer (quarot/nn/linear.py:24-79).
+def _pack_weight(weight, weight_scales):
+    """Codes round(W / scales), packed: the GPU quantiser with the given per-row scales
+    (qr_sym_quant_f16_i4 rounds and packs exactly like the reference's (W / s).round() followed by
+    pack_i4) after checking, as pack_i4 would, that no code leaves [-8, 7]."""
+    w = weight.cuda()
+    s = weight_scales.to(device=w.device, dtype=w.dtype)
+    if w.dtype == torch.float16 and w.is_contiguous():
+        ratio_max = float((w.float().abs() / s.float().abs().clamp_min(1e-30)).max()) if w.numel() else 0.0
+        if ratio_max < 7.4:                                  # every |W / s| rounds inside the grid: nothing to clamp
+            return quarot_amd.sym_quant(w, s.reshape(-1).contiguous())
+    codes = (w / s).round()
+    return quarot_amd.functional.pack_i4(codes.to(torch.int8))
 
-    Buffers (state-dict compatible with the reference): `weight` uint8 [out, in/2] packed int4,
-    `weight_scales` [out, 1], optional `bias` [out]."""
+
+class Linear4bit(torch.nn.Module):
+    """W4A4 linear layer with the interface and state-dict layout of quarot/nn/linear.py:24-79:
+    buffers `weight` (uint8 [out, in / 2], packed int4), `weight_scales` ([out, 1]) and optionally
+    `bias` ([out]).  forward() takes the PackedQuantizedTensor a Quantizer produces and runs the
+    int4 GEMM with the dequantisation (and bias) fused into its epilogue."""
 
     def __init__(self, in_features, out_features, bias=False, dtype=torch.float16):
         super().__init__()
-        self.in_features = in_features
-        self.out_features = out_features
-        self.register_buffer('weight_scales', torch.zeros((self.out_features, 1), requires_grad=False))
-        self.register_buffer('weight', torch.randint(1, 7, (self.out_features, self.in_features // 2),
-                                                     dtype=torch.uint8, requires_grad=False))
+        self.in_features, self.out_features = in_features, out_features
+        packed_shape = (out_features, in_features // 2)
+        self.register_buffer('weight_scales', torch.zeros((out_features, 1), requires_grad=False))
+        self.register_buffer('weight', torch.randint(1, 7, packed_shape, dtype=torch.uint8, requires_grad=False))
         if bias:
-            self.register_buffer('bias', torch.zeros((self.out_features), dtype=dtype))
+            self.register_buffer('bias', torch.zeros((out_features), dtype=dtype))
         else:
             self.bias = None
+
+    def extra_repr(self):
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
 
     def forward(self, x):
         assert type(x) == quarot_amd.PackedQuantizedTensor  # Quantized input is given
@@ -27,17 +43,16 @@ class Linear4bit(torch.nn.Module):
 
     @staticmethod
     def from_float(module: torch.nn.Linear, weight_scales=None):
-        """Build from an fp16 nn.Linear whose weights are already on the int4 grid times
-        `weight_scales` [out, 1]: codes = round(W / scales), packed (linear.py:58-79)."""
-        weight_matrix = module.weight.data
-        int_module = Linear4bit(module.in_features, module.out_features, bias=module.bias is not None,
-                                dtype=weight_matrix.dtype).to(weight_matrix.dtype)
-        if weight_scales is not None:
-            assert weight_scales.shape == (module.out_features, 1), 'weight_scales should have shape (out_features, 1)'
-            weight_matrix = weight_matrix.cuda()
-            int_module.weight_scales.copy_(weight_scales.to(weight_matrix.dtype))
-            int_rounded_weight = (weight_matrix / weight_scales.cuda()).round()
-            int_module.weight.copy_(quarot_amd.functional.pack_i4(int_rounded_weight.to(torch.int8)).cpu())
-            if module.bias is not None:
-                int_module.bias.copy_(module.bias)
-        return int_module
+        """A Linear4bit with module's shape; with `weight_scales` ([out, 1]) the weights, which must
+        already lie on the int4 grid times those scales, are converted to codes and packed
+        (linear.py:58-79).  Without scales only the shapes are taken over, as in the reference."""
+        w = module.weight.data
+        q4 = Linear4bit(module.in_features, module.out_features, bias=module.bias is not None, dtype=w.dtype).to(w.dtype)
+        if weight_scales is None:
+            return q4
+        assert weight_scales.shape == (module.out_features, 1), 'weight_scales should have shape (out_features, 1)'
+        q4.weight_scales.copy_(weight_scales.to(w.dtype))
+        q4.weight.copy_(_pack_weight(w, weight_scales).cpu())
+        if module.bias is not None:
+            q4.bias.copy_(module.bias)
+        return q4
