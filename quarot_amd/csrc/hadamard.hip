@@ -829,15 +829,20 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
                 for (int e = 0; e < 4; ++e) hf[t][ks][hh * 4 + e] = v[e];
             }
     }
-    // Sylvester fragments of all four column tiles: H_64[r][r'] = (-1)^popcount(r & r')
-    f16x8 b1[CT][2];
+    // Sylvester fragments of all four column tiles: H_64[r][r'] = (-1)^popcount(r & r') with
+    // r = 32 ks + 8 g + j, r' = 16 ct + l16.  The sign factors by index bits: bits 0..3 give a base
+    // fragment, bit 4 contributes (g >> 1) & (ct & 1) (lane-dependent: a second base for odd ct) and
+    // bit 5 contributes ks & (ct >> 1), the same for every lane.  Two bases and their negations
+    // (16 registers) stand for all eight fragments; which one an MFMA takes is known at compile time.
+    f16x8 sb[2][2];                                          // [ct & 1][negated]
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
+    for (int o = 0; o < 2; ++o)
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                b1[ct][ks][j] = (__builtin_popcount((ks * 32 + g * 8 + j) & (ct * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+        for (int j = 0; j < 8; ++j) {
+            const bool neg = ((__builtin_popcount(((g & 1) * 8 + j) & l16) + ((g >> 1) & o)) & 1) != 0;
+            sb[o][0][j] = neg ? (f16)-1.0f : (f16)1.0f;
+            sb[o][1][j] = neg ? (f16)1.0f : (f16)-1.0f;
+        }
 
     // staging: load c of a tile covers its rows 8 c .. 8 c + 7, lane -> (row 8 c + lane / 8, piece
     // lane % 8): 1 KB of consecutive addresses per instruction.  Pieces are XOR-keyed by the row so
@@ -893,8 +898,8 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][0]), b1[ct][0], acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][1]), b1[ct][1], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][0]), sb[ct & 1][0], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][1]), sb[ct & 1][ct >> 1], acc, 0, 0, 0);
                     float tv[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) tv[e] = acc[e] * scale;
@@ -933,6 +938,7 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             if (ct + 1 < CT) fetch(ct + 1, (ct + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);               // the next tile's reads are issued before this tile's MFMAs
             f32x4 acc[TPW];
 #pragma unroll
             for (int i = 0; i < TPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
