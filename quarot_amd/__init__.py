@@ -80,7 +80,7 @@ def sym_quant(x, scale):
     q = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().qr_sym_quant_f16_i4(_ptr(x2), _ptr(s), rows, cols, _ptr(q), _lib.stream_ptr(dev)))
-    return q.view(*lead, -1)
+    return q.view(*lead, q.shape[-1])
 
 
 def sym_dequant(q, scale_row, scale_col, bits=32):
@@ -101,7 +101,7 @@ def sym_dequant(q, scale_row, scale_col, bits=32):
     with torch.cuda.device(dev):
         _lib.check(_lib.lib().qr_sym_dequant_i32_f16(_ptr(q2), _ptr(sr), _ptr(scale_col), rows, cols, _ptr(y),
                                                      _lib.stream_ptr(dev)))
-    return y.view(*lead, -1)
+    return y.view(*lead, y.shape[-1])
 
 
 class PackedQuantizedTensor:
@@ -140,7 +140,7 @@ def quantize_rows(x, clip_ratio=1.0):
                                                       _lib.stream_ptr(dev)))
     # torch.max(dim=-1)[0].unsqueeze(1) on [..., C] gives shape lead[:1] + (1,) + lead[1:]
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
-    return q.view(*lead, -1), s.view(s_shape)
+    return q.view(*lead, q.shape[-1]), s.view(s_shape)
 
 
 def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_transformed=False):
@@ -163,7 +163,7 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
                                                           float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                           _lib.stream_ptr(dev)))
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
-    packed = PackedQuantizedTensor(q.view(*lead, -1), s.view(s_shape))
+    packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
     return (packed, y.view(x.shape)) if return_transformed else packed
 
 
@@ -182,7 +182,7 @@ def rmsnorm_quantize(x, mean_dim, eps=1e-5, clip_ratio=1.0, return_normalized=Fa
                                                          float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                          _lib.stream_ptr(dev)))
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
-    packed = PackedQuantizedTensor(q.view(*lead, -1), s.view(s_shape))
+    packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
     return (packed, y.view(x.shape)) if return_normalized else packed
 
 

@@ -464,6 +464,33 @@ def test_kv_vectors_with_infinities_take_the_ieee_path():
     assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
 
 
+def test_empty_and_leading_dimensions_through_the_python_interface():
+    """Zero rows are legal everywhere (nothing is launched, shapes follow the non-empty case); leading
+    dimensions are flattened and restored as the reference's wrappers do."""
+    e = torch.empty(0, 4096, dtype=torch.float16, device=dev())
+    q, s = quarot_amd.quantize_rows(e)
+    assert q.shape == (0, 2048) and s.numel() == 0
+    assert quarot_amd.nn.OnlineHadamard(4096).cuda()(e).shape == (0, 4096)
+    assert quarot_amd.nn.OnlineHadamardQuantizer(11008).cuda()(e.new_empty(0, 11008)).quantized_x.shape == (0, 5504)
+    assert quarot_amd.nn.RMSNormQuantizer(4096)(e).quantized_x.shape == (0, 2048)
+    w = torch.randint(0, 255, (64, 2048), dtype=torch.uint8, device=dev())
+    sw = torch.rand(64, 1, device=dev()).half()
+    assert quarot_amd.linear_i4(w.new_empty(0, 2048), sw.new_empty(0), w, sw).shape == (0, 64)
+    assert quarot_amd.matmul(w.new_empty(0, 2048), w).shape == (0, 64)
+    qk, sk, zk = kv.asym_quantize_and_pack_i4(e.new_empty(0, 8, 128), hadamard=True)
+    assert qk.shape == (0, 8, 64) and sk.shape == (0, 8, 1) and zk.shape == (0, 8, 1)
+    x3 = gpu(synth_x(10, 4096, seed=3)).view(2, 5, 4096)
+    p = quarot_amd.nn.Quantizer()(x3)
+    assert p.quantized_x.shape == (2, 5, 2048) and p.scales_x.shape == (2, 1, 5)      # the reference's unsqueeze(1) quirk
+    lin = quarot_amd.nn.Linear4bit(4096, 64).half().cuda()
+    lin.weight_scales.fill_(0.01)
+    assert lin(p).shape == (2, 5, 64)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        quarot_amd.quantize_rows(gpu(synth_x(8, 8192, seed=1))[:, ::2])
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        quarot_amd.quantize_rows(torch.zeros(8, 64, dtype=torch.float16))
+
+
 def test_decode_step_replays_from_a_hip_graph():
     """A decode step (fused Hadamard+quantise, then the decode GEMM) captured into a HIP graph: every
     replay, with fresh inputs copied into the static buffer and eager work plus synchronisation between
