@@ -352,7 +352,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
 // 0), global loads run one more stage ahead through registers, one barrier per stage.
 // (A variant in which half the waves only unpacked into int8 planes in LDS for the other half was
 // measured LDS-bound: twice the LDS bytes at ~128 B/clk/CU exceed the MFMA time.)
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int RD, bool DEQ>
 __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
@@ -423,8 +423,9 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
         const u32 off = (u32)((kb + scoff < Kb) ? kb + scoff : kb);
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
-            const uint8_t* base = (i * 64 < BM) ? A : B;
-            r[i] = *(const u32x4*)(base + (size_t)(goff[i] + off));
+            if (i * 64 < BM) r[i] = *(const u32x4*)(A + (size_t)(goff[i] + off));
+            else if (RD > 1) r[i] = __builtin_nontemporal_load((const u32x4*)(B + (size_t)(goff[i] + off)));
+            else r[i] = *(const u32x4*)(B + (size_t)(goff[i] + off));
         }
     };
     auto deposit = [&](int st, int buf, u32x4(&r)[NL]) {
@@ -437,6 +438,15 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 #pragma unroll
             for (int i = 0; i < NL; ++i) base[i * 64 * 8] = r[i];
         }
+    };
+    // the register ring's form writes stages past the end too (they repeat the last stage into a
+    // buffer nobody reads again): without a branch every wait counts exactly the loads issued after
+    // the ones it needs, with one the compiler waits for all outstanding loads
+    auto deposit_always = [&](int st, int buf, u32x4(&r)[NL]) {
+        const bool zero = ragged && (s_first + st) * 128 + scoff >= Kb;
+        u32x4* base = ks_lds + buf * CH + dst0;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) base[i * 64 * 8] = zero ? u32x4{0, 0, 0, 0} : r[i];
     };
 
     i32x16 acc[IM][JN];
@@ -488,41 +498,84 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.bhi[j], o.ahi[i], acc[i][j], 0, 0, 0);
     };
 
-    // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during iteration
-    // ks from registers requested at the end of iteration ks-1 (a second register set would spill).
-    // (the first three stages are requested together: the accumulators are not live yet, so two
-    // more register sets are free, and the prologue costs one memory round trip instead of three)
-    u32x4 regs[NL];
-    {
-        u32x4 first[NL], second[NL];
-        fetch(0, first);
-        fetch(1, second);
-        fetch(2, regs);
-        deposit(0, 0, first);
-        deposit(1, 1, second);
-    }
-    __syncthreads();                                        // stages 0 and 1 visible
     Ops ops;
-    if (kg == 1) load_ops(0, 0, ops);                       // group 1 starts one unpack ahead
     int bcur = 0;
-    for (int ks = 0; ks < stages; ++ks) {
-        const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
-        const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
-        if (kg == 0) {
-            load_ops(bcur, 0, ops);
-            multiply(ops);
-            load_ops(bcur, 1, ops);
-            multiply(ops);
-        } else {
-            multiply(ops);                                  // sub-step 2 of this stage (unpacked earlier)
-            load_ops(bcur, 1, ops);
-            multiply(ops);                                  // sub-step 3
-            if (ks + 1 < stages) load_ops(bnext, 0, ops);   // next stage's sub-step 2
+    if constexpr (RD == 1) {
+        // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during
+        // iteration ks from registers requested at the end of iteration ks-1.  The first three stages
+        // are requested together: the accumulators are not live yet, so two more register sets are
+        // free, and the prologue costs one memory round trip instead of three.
+        u32x4 regs[NL];
+        {
+            u32x4 first[NL], second[NL];
+            fetch(0, first);
+            fetch(1, second);
+            fetch(2, regs);
+            deposit(0, 0, first);
+            deposit(1, 1, second);
         }
-        deposit(ks + 2, bfill, regs);
-        fetch(ks + 3, regs);
-        __syncthreads();
-        bcur = bnext;
+        __syncthreads();                                    // stages 0 and 1 visible
+        if (kg == 1) load_ops(0, 0, ops);                   // group 1 starts one unpack ahead
+        for (int ks = 0; ks < stages; ++ks) {
+            const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+            const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
+            if (kg == 0) {
+                load_ops(bcur, 0, ops);
+                multiply(ops);
+                load_ops(bcur, 1, ops);
+                multiply(ops);
+            } else {
+                multiply(ops);                              // sub-step 2 of this stage (unpacked earlier)
+                load_ops(bcur, 1, ops);
+                multiply(ops);                              // sub-step 3
+                if (ks + 1 < stages) load_ops(bnext, 0, ops);   // next stage's sub-step 2
+            }
+            deposit(ks + 2, bfill, regs);
+            fetch(ks + 3, regs);
+            __syncthreads();
+            bcur = bnext;
+        }
+    } else {
+        // Weight streaming (few tokens): an iteration is far shorter than the memory latency, so RD
+        // register sets rotate, set (st % RD) carrying stage st, requested RD iterations before it
+        // is written to LDS.  The first two stages pass through the ring like all others.  Whole
+        // turns of the ring run without a branch around the loads.
+        u32x4 regs[RD][NL];
+#pragma unroll
+        for (int r = 0; r < RD; ++r) fetch(r, regs[r]);
+        deposit_always(0, 0, regs[0]);
+        fetch(RD, regs[0]);
+        deposit_always(1, 1, regs[1 % RD]);
+        fetch(RD + 1, regs[1 % RD]);
+        __syncthreads();                                    // stages 0 and 1 visible
+        if (kg == 1) load_ops(0, 0, ops);                   // group 1 starts one unpack ahead
+        auto iteration = [&](int ks, u32x4(&r)[NL]) {
+            const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+            const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
+            if (kg == 0) {
+                load_ops(bcur, 0, ops);
+                multiply(ops);
+                load_ops(bcur, 1, ops);
+                multiply(ops);
+            } else {
+                multiply(ops);
+                load_ops(bcur, 1, ops);
+                multiply(ops);
+                if (ks + 1 < stages) load_ops(bnext, 0, ops);
+            }
+            deposit_always(ks + 2, bfill, r);
+            fetch(ks + 2 + RD, r);
+            __syncthreads();
+            bcur = bnext;
+        };
+        int ks0 = 0;
+        for (; ks0 + RD <= stages; ks0 += RD) {
+#pragma unroll
+            for (int r = 0; r < RD; ++r) iteration(ks0 + r, regs[(r + 2) % RD]);
+        }
+#pragma unroll
+        for (int r = 0; r < RD - 1; ++r)
+            if (ks0 + r < stages) iteration(ks0 + r, regs[(r + 2) % RD]);
     }
 
     // K-split: group 0 finalises the lower half of the j tiles and group 1 the upper half; each sends
@@ -663,7 +716,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int RD = 1>
 int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
               const void* bias, hipStream_t st, int ksplit = 1) {
     constexpr int NT = 128 * WAVES_M * WAVES_N;
@@ -677,13 +730,13 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     hipError_t e;
     if (Y) {
-        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, true>;
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, RD, true>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, 1);
     } else {
-        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, RD, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
@@ -1384,13 +1437,12 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
 // XL = load instructions per step that carry rows of X (64 / CPR rows each): with few tokens only
 // the first ceil(M / (64 / CPR)) of them are issued and staged; the remaining rows of the 32-row
 // MFMA operand keep whatever the buffer holds, and the output rows they produce are never stored.
-template <int MT, int SB, int XL, bool DEQ>
+template <int MT, int SB, int XL, int PF, bool DEQ>
 __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
                                                         const f16* __restrict__ sB, const f16* __restrict__ bias) {
     constexpr int CPR = SB / 16;                            // 16-byte chunks per row and step (4, 8 or 16)
-    constexpr int PF = SB == 64 ? 4 : 3;                    // steps in flight
     constexpr int ROWS = (1 + MT) * 32;                     // staged rows per wave: 32 of W, then 32 MT of X
     constexpr int NLW = 32 * CPR / 64;                      // chunks per lane and step: rows of W ...
     constexpr int NLD = NLW + XL;                           // ... plus the rows of X that exist
@@ -1439,18 +1491,25 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
         const bool dead = sc * SB + piece * 16 >= Kb;
         const int off = sc * SB + (dead ? (piece & 1) : piece) * 16;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i) st.v[i] = *(const u32x4*)(src[i] + off);
+        for (int i = 0; i < NLD; ++i) {
+            // weights are used once: streaming loads keep the tokens' codes, which every workgroup
+            // re-reads, in the caches
+            if (i < NLW) st.v[i] = __builtin_nontemporal_load((const u32x4*)(src[i] + off));
+            else st.v[i] = *(const u32x4*)(src[i] + off);
+        }
     };
     i32x16 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[t][v] = 0;
-    auto consume = [&](int sidx, const Step& st) {
+    auto deposit = [&](int sidx, const Step& st) {
         const bool dead = sidx * SB + piece * 16 >= Kb;
         // LDS operations of one wave execute in order: these writes follow the previous step's reads
 #pragma unroll
         for (int i = 0; i < NLD; ++i) stage[dst[i]] = dead ? u32x4{0, 0, 0, 0} : st.v[i];
+    };
+    auto multiply = [&]() {
 #pragma unroll
         for (int c = 0; c < CPR / 2; ++c) {                 // lane half h takes pieces 2c + h of both operands
             const u32x4 wq = stage[slot(r, 2 * c + h)];
@@ -1467,15 +1526,28 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
     Step ring[PF];
 #pragma unroll
     for (int p = 0; p < PF; ++p) fetch(s_begin + p, ring[p]);
-    for (int s = s_begin; s < s_end; s += PF) {
+    // whole turns of the ring run without a branch, so that every wait inside them counts exactly the
+    // loads issued after the step it needs (a branch in the loop body makes the compiler wait for all
+    // outstanding loads once per turn)
+    // The loads that refill a ring slot are issued as soon as the slot has been written to LDS, before
+    // the step's multiplications; the scheduling barriers keep the compiler from moving them later.
+    int s = s_begin;
+    for (; s + PF <= s_end; s += PF) {
 #pragma unroll
         for (int p = 0; p < PF; ++p) {
-            if (s + p < s_end) {
-                consume(s + p, ring[p]);
-                fetch(s + p + PF, ring[p]);                 // indices past the end re-read the last step (unused)
-            }
+            deposit(s + p, ring[p]);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(s + p + PF, ring[p]);                     // indices past the end re-read the last step (unused)
+            __builtin_amdgcn_sched_barrier(0);
+            multiply();
         }
     }
+#pragma unroll
+    for (int p = 0; p < PF - 1; ++p)
+        if (s + p < s_end) {
+            deposit(s + p, ring[p]);
+            multiply();
+        }
     __syncthreads();                                        // the staging buffers become the reduction buffer
     // ---- sum the eight partial tiles
 #pragma unroll
@@ -1680,19 +1752,19 @@ int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, voi
 int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                   const void* bias, hipStream_t st) {
     const unsigned grid = (unsigned)((N + 31) / 32);
-#define QR_DEC(MT, SB, XL)                                                                                            \
+#define QR_DEC(MT, SB, XL, PF)                                                                                          \
     do {                                                                                                              \
         constexpr int STAGE = (1 + MT) * 32 * (SB / 16), RED = MT * 4 * 64;                                           \
         constexpr size_t LDS = (size_t)8 * (STAGE > RED ? STAGE : RED) * 16;                                          \
         hipError_t e;                                                                                                 \
         if (Y) {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, XL, true>;                                                           \
+            auto kern = decode_i4_kernel<MT, SB, XL, PF, true>;                                                        \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr,         \
                                                      (f16*)Y, (const f16*)sA, (const f16*)sB, (const f16*)bias);      \
         } else {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, XL, false>;                                                          \
+            auto kern = decode_i4_kernel<MT, SB, XL, PF, false>;                                                       \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
@@ -1700,11 +1772,11 @@ int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, v
         }                                                                                                             \
     } while (0)
     // a load instruction carries eight rows of X (128-byte pieces): issue only those that exist
-    if (M <= 8) QR_DEC(1, 128, 1);
-    else if (M <= 16) QR_DEC(1, 128, 2);
-    else if (M <= 32) QR_DEC(1, 128, 4);
-    else if (M <= 48) QR_DEC(2, 128, 6);
-    else QR_DEC(2, 128, 8);
+    if (M <= 8) QR_DEC(1, 128, 1, 3);
+    else if (M <= 16) QR_DEC(1, 128, 2, 3);
+    else if (M <= 32) QR_DEC(1, 128, 4, 3);
+    else if (M <= 48) QR_DEC(2, 128, 6, 3);
+    else QR_DEC(2, 128, 8, 3);
 #undef QR_DEC
     return qr_launch_status();
 }
@@ -1821,7 +1893,7 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (M <= 64) {
         // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
         // once per tile); otherwise eight waves split K over 32 rows
-        if ((N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        if ((N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
