@@ -1628,8 +1628,16 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
         const int mr = m < M ? m : M - 1;
         xp[m] = A + (int64_t)mr * Kb + lane * 16;
     }
+    // which of a group's NV sums this lane stores at the end of the exchange below (log2(NV) lane
+    // bits from bit 5 downwards), and its token's scale
+    constexpr int LV = NV == 4 ? 2 : NV == 8 ? 3 : NV == 16 ? 4 : 5;
+    const int vidx = lane >> (6 - LV);
+    const int my_m = vidx / R, my_r = vidx % R;
+    f16 my_sa = (f16)0;
+    if (DEQ) my_sa = sA[my_m < M ? my_m : M - 1];
     struct Seg {
         u32x4 w[R], x[MB];
+        f16 sb, bi;                                         // column scale and bias of the lane's output
     };
     // fetch side: position (fg, fs) runs ahead of the consume side
     int fg = 0, fs = 0;
@@ -1645,6 +1653,14 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
         }
 #pragma unroll
         for (int m = 0; m < MB; ++m) g.x[m] = *(const u32x4*)(xp[m] - lane * 16 + off);
+        // every segment carries its group's scale along: loading it at the group's end would make
+        // the wave wait for everything it has in flight
+        if (DEQ) {
+            int col = (g0 + fg) * R + my_r;
+            col = col < N ? col : N - 1;
+            g.sb = sB[col];
+            g.bi = (bias ? bias : sB)[col];                 // (no bias: a harmless second read of the scale)
+        }
         if (fs + 1 < nseg) ++fs;
         else if (fg + 1 < gcount) { ++fg; fs = 0; }
     };
@@ -1653,15 +1669,18 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
     for (int v = 0; v < NV; ++v) acc[v] = 0;
     int cg = 0, cs = 0;
     auto consume = [&](const Seg& g) {
-        if (cs * 1024 + lane * 16 < Kb) {
+        // lanes beyond the row end multiply by zero (no branch around the products: a branch here
+        // makes the compiler wait for every outstanding load once per turn of the ring)
+        const bool live = cs * 1024 + lane * 16 < Kb;
 #pragma unroll
-            for (int m = 0; m < MB; ++m)
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int xv = live ? (int)g.x[m][d] : 0;
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int d = 0; d < 4; ++d)
-                        acc[m * R + r] = __builtin_amdgcn_sdot8((int)g.w[r][d], (int)g.x[m][d], acc[m * R + r], false);
-        }
+                    acc[m * R + r] = __builtin_amdgcn_sdot8((int)g.w[r][d], xv, acc[m * R + r], false);
+            }
         if (++cs < nseg) return;
         // ---- end of a row group: halving exchange.  After the steps with offsets 32, 16, ... a lane
         // holds the sum of value index (bits of its lane id, most significant first) over the lanes
@@ -1683,19 +1702,15 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
         }
         int sum = vals[0];
         for (; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
-        // which value this lane ended up with: log2(NV) lane bits from bit 5 downwards
-        constexpr int LV = NV == 4 ? 2 : NV == 8 ? 3 : NV == 16 ? 4 : 5;
-        const int vidx = lane >> (6 - LV);
         if ((lane & ((1 << (6 - LV)) - 1)) == 0) {
-            const int m = vidx / R, r = vidx % R;
-            const int col = (g0 + cg) * R + r;
-            if (m < M && col < N) {
+            const int col = (g0 + cg) * R + my_r;
+            if (my_m < M && col < N) {
                 if (DEQ) {
-                    f16 yv = (f16)(sA[m] * sB[col]) * (f16)(float)sum;
-                    if (bias) yv = yv + bias[col];
-                    Y[(int64_t)m * N + col] = yv;
+                    f16 yv = (f16)(my_sa * g.sb) * (f16)(float)sum;
+                    if (bias) yv = yv + g.bi;
+                    Y[(int64_t)my_m * N + col] = yv;
                 } else {
-                    C[(int64_t)m * N + col] = sum;
+                    C[(int64_t)my_m * N + col] = sum;
                 }
             }
         }
@@ -1708,26 +1723,50 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
     fetch(ga);
     fetch(gb);
     fetch(gc);
-    for (int it = 0; it < total; it += 3) {
+    int it = 0;
+    for (; it + 3 <= total; it += 3) {                      // whole turns of the ring: no branch around the loads
         consume(ga);
         fetch(ga);
-        if (it + 1 < total) {
-            consume(gb);
-            fetch(gb);
-        }
-        if (it + 2 < total) {
-            consume(gc);
-            fetch(gc);
-        }
+        consume(gb);
+        fetch(gb);
+        consume(gc);
+        fetch(gc);
     }
+    if (it < total) consume(ga);
+    if (it + 1 < total) consume(gb);
 }
 
 int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                 const void* bias, hipStream_t st) {
     const int groups = (N + 3) / 4;
-    // row groups per wave: at least ~64 KB of weights per wave, but keep >= 2048 waves when N allows
+    // row groups per wave: about 64 KB of weights per wave, but keep >= 2048 waves when N allows ...
     int ng = (65536 + 4 * Kb - 1) / (4 * Kb);
     while (ng > 1 && groups / ng < 2048) --ng;
+    // ... and, when all workgroups are resident at once (up to five per CU), a count that spreads
+    // evenly over the 256 CUs: 3.5 workgroups per CU run as long as 4.  Among ng / 2 ... 2 ng the
+    // value nearest to ng whose last round of 256 is at least 97 % full, else the fullest.
+    {
+        auto fill = [&](int g) {
+            const int wgs = ((groups + g - 1) / g + 3) / 4;
+            if (wgs > 1280) return 1.0;
+            return (double)wgs / (double)(((wgs + 255) / 256) * 256);
+        };
+        int best = ng;
+        double best_fill = fill(ng);
+        for (int d = 1; d <= ng && best_fill < 0.97; ++d) {
+            const int cand[2] = {ng - d, ng + d};
+            for (int c = 0; c < 2; ++c) {
+                const int g = cand[c];
+                if (g < 1 || 2 * g < ng || g > 2 * ng) continue;
+                const double f = fill(g);
+                if (f >= 0.97 ? best_fill < 0.97 : f > best_fill) {
+                    best = g;
+                    best_fill = f;
+                }
+            }
+        }
+        ng = best;
+    }
     const int waves = (groups + ng - 1) / ng;
     const unsigned grid = (unsigned)((waves + 3) / 4);
 #define QR_GEMV(MB)                                                                                                   \
