@@ -68,9 +68,9 @@ TRAFFIC_KIB = {
     "c1": (16551.0, 16384.0),
     "c2": (44210.0, 16384.0),
     "c3d": (528791.7, 262144.0),
-    "c4": (72440.1, 1024.0),
-    "c4m1": (61875.4, 16.0),
-    "c4g64": (115876.5, 7168.0),
+    "c4": (62375.6, 1024.0),
+    "c4m1": (57494.0, 16.0),
+    "c4g64": (124423.7, 7168.0),
     "c5": (131145.2, 69808.6),              # kv_had128_kernel (K cache), per launch
 }
 
