@@ -399,7 +399,7 @@ def main():
     if m <= 4:
         kern = "gemv_i4_kernel"
     elif decode:
-        kern = "gemm_ks_kernel<64,256>" if (n + 255) // 256 >= 128 else "decode_i4_kernel"
+        kern = "gemm_ks_kernel<64,256>" if m > 16 and (n + 255) // 256 >= 128 else "decode_i4_kernel"
     elif t128 >= 128:       # the library's choice between its two pipelined kernels, by rounds of tiles
         kern = "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
     else:

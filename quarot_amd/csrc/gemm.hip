@@ -1427,9 +1427,10 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decode (M <= 64) with too few column tiles for the tiled kernels.  A workgroup of eight waves owns
-// 32 weight rows; the waves split K into eight contiguous ranges and the eight partial 32 x M tiles
-// are summed through LDS and dequantised.  Nothing is shared between waves in the main loop, so there
+// Decode (M <= 64) with too few column tiles for the tiled kernels, or few tokens.  A workgroup of
+// eight waves owns 8 / KW groups of 32 weight rows; the KW waves of a group split K into contiguous
+// ranges and their partial 32 x M tiles are summed through LDS and dequantised (KW = 8 when K is
+// long and N small, 2 or 4 when a wave would otherwise get only a handful of steps).  Nothing is shared between waves in the main loop, so there
 // are no barriers in it: every wave streams its own slices of W and X with coalesced 16-byte loads
 // (SB / 16 lanes per row piece of SB bytes, PF steps ahead in a register ring) and turns them into
 // MFMA fragments (lane = row) through a wave-private LDS buffer.  Loading fragments straight from
@@ -1437,7 +1438,7 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
 // XL = load instructions per step that carry rows of X (64 / CPR rows each): with few tokens only
 // the first ceil(M / (64 / CPR)) of them are issued and staged; the remaining rows of the 32-row
 // MFMA operand keep whatever the buffer holds, and the output rows they produce are never stored.
-template <int MT, int SB, int XL, int PF, bool DEQ>
+template <int MT, int SB, int XL, int PF, int KW, bool DEQ>
 __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
@@ -1453,9 +1454,11 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
     i32x4* red = (i32x4*)dec_smem;                          // [wave][m tile][4-register group][lane]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
-    const int n0 = blockIdx.x * 32;
+    constexpr int RG = 8 / KW;                              // groups of 32 weight rows per workgroup
+    const int kw = wave % KW;                               // this wave's share of K within its row group
+    const int n0 = (blockIdx.x * RG + wave / KW) * 32;
     const int steps = (Kb + SB - 1) / SB;
-    const int s_begin = (int)((int64_t)steps * wave / 8), s_end = (int)((int64_t)steps * (wave + 1) / 8);
+    const int s_begin = (int)((int64_t)steps * kw / KW), s_end = (int)((int64_t)steps * (kw + 1) / KW);
     u32x4* stage = dec_smem + wave * STAGE;
     // chunk position XOR-keyed by the row: the 16 rows of a fragment read spread over all bank groups
     auto slot = [](int row, int chunk) {
@@ -1556,14 +1559,14 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
         for (int gq = 0; gq < 4; ++gq)
             red[((wave * MT + t) * 4 + gq) * 64 + lane] = i32x4{acc[t][gq * 4], acc[t][gq * 4 + 1], acc[t][gq * 4 + 2], acc[t][gq * 4 + 3]};
     __syncthreads();
-    // unit u = (m tile, register group): one wave each
-    if (wave < MT * 4) {
-        const int t = wave >> 2, gq = wave & 3;
+    // unit u = (row group, m tile, register group): the waves take them in turn
+    for (int u = wave; u < RG * MT * 4; u += 8) {
+        const int g = u / (MT * 4), t = (u >> 2) % MT, gq = u & 3;
         i32x4 sum = {0, 0, 0, 0};
 #pragma unroll
-        for (int w = 0; w < 8; ++w) sum += red[((w * MT + t) * 4 + gq) * 64 + lane];
+        for (int w = 0; w < KW; ++w) sum += red[(((g * KW + w) * MT + t) * 4 + gq) * 64 + lane];
         const int row = t * 32 + r;
-        const int col = n0 + gq * 8 + h * 4;
+        const int col = (blockIdx.x * RG + g) * 32 + gq * 8 + h * 4;
         if (row < M && col < N) {
             const bool whole = (col + 4 <= N) && ((N & 3) == 0);
             if (DEQ) {
@@ -1789,33 +1792,61 @@ int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, voi
 }
 
 int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
-                  const void* bias, hipStream_t st) {
-    const unsigned grid = (unsigned)((N + 31) / 32);
-#define QR_DEC(MT, SB, XL, PF)                                                                                          \
+                  const void* bias, hipStream_t st, int kw = 0) {
+#define QR_DEC(MT, SB, XL, PF, KW)                                                                                          \
     do {                                                                                                              \
         constexpr int STAGE = (1 + MT) * 32 * (SB / 16), RED = MT * 4 * 64;                                           \
         constexpr size_t LDS = (size_t)8 * (STAGE > RED ? STAGE : RED) * 16;                                          \
         hipError_t e;                                                                                                 \
         if (Y) {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, XL, PF, true>;                                                        \
+            auto kern = decode_i4_kernel<MT, SB, XL, PF, KW, true>;                                                       \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
-            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr,         \
+            kern<<<dim3((unsigned)((N + 32 * (8 / KW) - 1) / (32 * (8 / KW)))), dim3(512), LDS, st>>>(                \
+                (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr,                                              \
                                                      (f16*)Y, (const f16*)sA, (const f16*)sB, (const f16*)bias);      \
         } else {                                                                                                      \
-            auto kern = decode_i4_kernel<MT, SB, XL, PF, false>;                                                       \
+            auto kern = decode_i4_kernel<MT, SB, XL, PF, KW, false>;                                                      \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
-            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
+            kern<<<dim3((unsigned)((N + 32 * (8 / KW) - 1) / (32 * (8 / KW)))), dim3(512), LDS, st>>>(                \
+                (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,                                          \
                                                      nullptr, nullptr, nullptr, nullptr);                             \
         }                                                                                                             \
     } while (0)
     // a load instruction carries eight rows of X (128-byte pieces): issue only those that exist
-    if (M <= 8) QR_DEC(1, 128, 1, 3);
-    else if (M <= 16) QR_DEC(1, 128, 2, 3);
-    else if (M <= 32) QR_DEC(1, 128, 4, 3);
-    else if (M <= 48) QR_DEC(2, 128, 6, 3);
-    else QR_DEC(2, 128, 8, 3);
+    // K is split KW ways within a row group (8 / KW row groups per workgroup).  One workgroup is
+    // resident per CU, so the launch takes rounds(workgroups / 256) times a workgroup's time, which
+    // is a fixed part (start, first loads, final sum: about six steps' worth) plus its steps per wave.
+    if (kw == 0) {
+        kw = 8;
+        if (M <= 32) {
+            const int steps = (Kb + 127) / 128;
+            double best = 0;
+            for (int c = 8; c >= 2; c >>= 1) {
+                const int wgs = (N + 32 * (8 / c) - 1) / (32 * (8 / c));
+                const double cost = (double)((wgs + 255) / 256) * (6.0 + (double)steps / c);
+                if (c == 8 || cost < best) {
+                    best = cost;
+                    kw = c;
+                }
+            }
+        }
+    }
+    if (M <= 8) {
+        if (kw == 2) QR_DEC(1, 128, 1, 3, 2);
+        else if (kw == 4) QR_DEC(1, 128, 1, 3, 4);
+        else QR_DEC(1, 128, 1, 3, 8);
+    } else if (M <= 16) {
+        if (kw == 2) QR_DEC(1, 128, 2, 3, 2);
+        else if (kw == 4) QR_DEC(1, 128, 2, 3, 4);
+        else QR_DEC(1, 128, 2, 3, 8);
+    } else if (M <= 32) {
+        if (kw == 2) QR_DEC(1, 128, 4, 3, 2);
+        else if (kw == 4) QR_DEC(1, 128, 4, 3, 4);
+        else QR_DEC(1, 128, 4, 3, 8);
+    } else if (M <= 48) QR_DEC(2, 128, 6, 3, 8);
+    else QR_DEC(2, 128, 8, 3, 8);
 #undef QR_DEC
     return qr_launch_status();
 }
@@ -1930,9 +1961,10 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         return qr_launch_status();
     }
     if (M <= 64) {
-        // weight streaming: with enough 256-row tiles to fill the CUs the tiled kernel wins (X is read
-        // once per tile); otherwise eight waves split K over 32 rows
-        if ((N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        // weight streaming: above 16 tokens and with enough 256-row tiles to fill the CUs the tiled
+        // kernel wins (X is read once per tile); otherwise the barrier-free kernel in which the waves
+        // of a workgroup split K over groups of 32 rows
+        if (M > 16 && (N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);

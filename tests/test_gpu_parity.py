@@ -164,6 +164,10 @@ def test_matmul_and_linear_random_shapes_across_every_kernel_boundary():
     for _ in range(6):                                   # enough tiles for the pipelined kernels
         shapes.append((int(rng.integers(1800, 2300)), int(rng.integers(3900, 4300)), 64 * int(rng.integers(1, 13))))
     shapes += [(70, 300, 4096), (140, 1030, 2048), (2048, 8192, 256), (4100, 4100, 512)]
+    # few tokens and many weight rows: the decode kernel with K split four ways (N > 8192) and two ways
+    # (N > 16384) within a row group, every token-count variant, ragged N and a ragged last K step
+    shapes += [(5, 8207, 320), (16, 8450, 1024), (17, 9001, 192), (32, 8333, 576),
+               (8, 16531, 192), (9, 16700, 768), (24, 17001, 320), (32, 16385, 128)]
     for (m, n, k) in shapes:
         a = o.pack_i4(rng.integers(-8, 8, (m, k)))
         w = o.pack_i4(rng.integers(-8, 8, (n, k)))
