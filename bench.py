@@ -9,6 +9,8 @@ HBM.  Workloads (shapes of Llama-2; inputs as in the reference's qlinear benchma
 outlier channels that motivate the Hadamard):
     c1  q_proj 7B      X [2048, 4096]   W int4 [4096, 4096]     no online Hadamard
     c1n the same with the RMSNorm in front of the quantiser (fused RMSNorm + Quantizer kernel)
+    c1o o_proj 7B      attention output [2048, 32, 128] -> Hadamard across the 32 heads -> Quantizer
+        (one fused kernel) -> W int4 [4096, 4096]
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
     c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
     c3  the four linears of a 7B decoder layer at 32768 tokens as ONE step: fused qkv 4096->12288, o 4096->4096,
@@ -39,6 +41,7 @@ WORKLOADS = {
     #        M      K      N     hadamard
     "c1": (2048, 4096, 4096, False),
     "c1n": (2048, 4096, 4096, False),       # input_layernorm -> Quantizer -> q_proj
+    "c1o": (2048, 4096, 4096, False),       # attention output -> Hadamard over heads -> Quantizer -> o_proj
     "c2": (2048, 11008, 4096, True),
     "c3d": (32768, 11008, 4096, True),
     "c3a": (32768, 4096, 12288, False),     # fused qkv
@@ -94,7 +97,7 @@ def synth_w(n, k, seed=1):
     return pack_i4(codes), s
 
 
-def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=False):
+def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=False, heads=0):
     """The reference's CPU path (torch Hadamard + quant + integer matmul + dequant) on a bounded
     row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
     from oracle import cpu_baseline as cb
@@ -103,17 +106,18 @@ def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=
     wc = cb.unpacked_codes(w_packed.numpy())
     ws = w_scales.view(-1)
     torch.set_num_threads(os.cpu_count() or 1)
-    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm)          # warm-up
+    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
-        cb.linear4bit_path(xs, wc, ws, hadamard, rmsnorm)
+        cb.linear4bit_path(xs, wc, ws, hadamard, rmsnorm, heads)
         times.append(time.perf_counter() - t0)
     t = float(np.median(times))
     return {"value": round(2.0 * rows * n * k / t / 1e12, 5), "unit": "TOPS", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"first {rows} of {m} rows, full N and K, median of 3 ({t * 1e3:.0f} ms); torch "
-                      + ("fp32 RMSNorm + " if rmsnorm else "fp32 matmul_hadU + " if hadamard else "")
+                      + ("fp32 RMSNorm + " if rmsnorm else "fp32 matmul_hadU + " if hadamard
+                         else "fp32 matmul_hadU over heads + " if heads else "")
                       + "fp16 sym quant + int32 torch matmul + fp16 dequant"}
 
 
@@ -296,8 +300,11 @@ def main():
     lin.weight.copy_(w_cpu.to(dev))
     lin.weight_scales.copy_(sw_cpu.to(dev))
     rmsnorm = args.workload == "c1n"
+    heads = 32 if args.workload == "c1o" else 0
+    if heads:
+        x = x.view(m, heads, k // heads)                    # as attention writes it: [tokens, heads, head_dim]
     front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if hadamard else quarot_amd.nn.RMSNormQuantizer(k) if rmsnorm
-             else quarot_amd.nn.Quantizer()).to(dev)
+             else quarot_amd.nn.HeadsHadamardQuantizer(heads) if heads else quarot_amd.nn.Quantizer()).to(dev)
     # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
     copies = [lin.weight]
     if m <= 64:
@@ -358,6 +365,10 @@ def main():
     staged_front = (torch.nn.Sequential(quarot_amd.nn.OnlineHadamard(k), quarot_amd.nn.Quantizer()) if hadamard
                     else torch.nn.Sequential(quarot_amd.nn.RMSNorm(k), quarot_amd.nn.Quantizer()) if rmsnorm
                     else quarot_amd.nn.Quantizer()).to(dev)
+    if heads:
+        # the reference's sequence: transform on the transposed view, transpose back, reshape, quantise
+        had_heads, quant = quarot_amd.nn.OnlineHadamard(heads).to(dev), quarot_amd.nn.Quantizer()
+        staged_front = lambda t: quant(had_heads(t.transpose(-1, -2)).transpose(-1, -2).reshape(m, k).contiguous())
     for _ in range(3):
         lin(staged_front(x))
     torch.cuda.synchronize()
@@ -414,15 +425,17 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 scales",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: Linear4bit X[{m},{k}] fp16 (1% outlier channels x20) . W int4[{n},{k}]"
-                               + (" with online Hadamard" if hadamard else " behind RMSNorm" if rmsnorm else ""),
+                               + (" with online Hadamard" if hadamard else " behind RMSNorm" if rmsnorm
+                                  else f" behind the Hadamard across {heads} heads" if heads else ""),
                    "M": m, "K": k, "N": n,
                    "path": ("fused Hadamard+quantise kernel" if hadamard else "fused RMSNorm+quantise kernel" if rmsnorm
-                            else "quantise kernel") + ", fused GEMM+dequant kernel",
+                            else "fused heads-Hadamard+quantise kernel" if heads else "quantise kernel")
+                           + ", fused GEMM+dequant kernel",
                    "staged_reference_api_ms": round(staged_ms, 4), "launch": "hip graph replay" if args.graph else "eager"},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(x_cpu, w_cpu, sw_cpu, hadamard, m, n, k, args.cpu_rows, rmsnorm)
+        out["cpu_baseline"] = cpu_baseline(x_cpu, w_cpu, sw_cpu, hadamard, m, n, k, args.cpu_rows, rmsnorm, heads)
     print(json.dumps(out))
 
 

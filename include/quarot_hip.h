@@ -104,6 +104,23 @@ int qr_rmsnorm_quantize_f16_i4(const void* x, int64_t rows, int64_t cols, int me
                                float clip, void* q, void* scales, void* y_or_null, void* stream);
 
 /*
+ * Fused Hadamard across attention heads + Quantizer: the chain in front of o_proj
+ * (e2e/quantized_llama/modeling_llama.py:108-110: quarot.nn.OnlineHadamard(num_heads) applied to
+ * attn_output.transpose(-1, -2), transposed back and reshaped to [.., hidden], then o_proj's
+ * quarot.nn.Quantizer; the transform itself is quarot/nn/hadamard.py:17-23 with K = 1, i.e.
+ * quarot/functional/hadamard.py:92-101 on a last axis of length num_heads).
+ *   x fp16 [rows, heads * head_dim], a row being [heads, head_dim] as attention writes it;
+ *   y[r, g, d] = fp16( (1 / sqrt(heads)) * sum_h Had[g, h] * x[r, h, d] ), Had the Sylvester matrix of
+ *   size heads, summed in fp32 and rounded to fp16 once; q and scales as qr_quantize_rows_f16_i4(y)
+ *   over the whole row.  No transposed copies are made.
+ *   head_dim == 128 and heads in {16, 32, 64} (else QR_E_UNSUPPORTED: use qr_hadamard on a transposed
+ *   copy and qr_quantize_rows_f16_i4); y_or_null: optional fp16 copy of the transformed rows.
+ *   x and y 16-byte aligned, q 4-byte aligned.
+ */
+int qr_heads_hadamard_quantize_f16_i4(const void* x, int64_t rows, int heads, int head_dim, float clip,
+                                      void* q, void* scales, void* y_or_null, void* stream);
+
+/*
  * int4 x int4 -> int32 GEMM:  C[M, N] = unpack(A)[M, K] . unpack(B)[N, K]^T.
  * Replaces matmul_host (quarot/kernels/gemm.cu:7-46), bound as quarot._CUDA.matmul
  * (quarot/kernels/bindings.cpp:9-25).

@@ -42,10 +42,15 @@ def rmsnorm(x16, eps=1e-5):
     return (xf * torch.rsqrt(var + eps)).to(torch.float16)
 
 
-def linear4bit_path(x16, w_codes_i32, w_scales16, hadamard=True, norm=False):
-    """x fp16 [M, K] -> fp16 [M, N]: (RMSNorm ->) Hadamard (fp32) -> quantise -> int32 matmul -> dequant."""
+def linear4bit_path(x16, w_codes_i32, w_scales16, hadamard=True, norm=False, heads=0):
+    """x fp16 [M, K] -> fp16 [M, N]: (RMSNorm ->) Hadamard (fp32) -> quantise -> int32 matmul -> dequant.
+    heads > 0: the Hadamard runs over the head axis of rows seen as [heads, K / heads], on the
+    transposed view as in e2e/quantized_llama/modeling_llama.py:108-109."""
     if norm:
         x16 = rmsnorm(x16)
+    if heads:
+        v = x16.float().view(x16.shape[0], heads, -1).transpose(-1, -2).contiguous()
+        x16 = matmul_hadU(v).transpose(-1, -2).reshape(x16.shape).contiguous().to(torch.float16)
     xh = matmul_hadU(x16.float()).to(torch.float16) if hadamard else x16
     q, sx = quantize(xh)
     acc = q @ w_codes_i32.t()

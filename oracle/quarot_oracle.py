@@ -22,6 +22,8 @@ How each function is pinned (see tests/test_oracle.py):
   int4_matmul          int64 brute force, closed-form all-7 x all-(-8) = -56.K, one-hot rows
   sym_dequant          exact rational rounding of each of the three operations
   kv_asym_*            range/extreme-code invariants and exact rational spot checks
+  heads_hadamard       float64 einsum with scipy.linalg.hadamard over the head axis, a row constant
+                       across heads (only head 0 survives, times sqrt(H)), one-hot heads (sign columns)
   rmsnorm              float64 closed form x / sqrt(sum(x^2) / mean_dim + eps) rounded once,
                        constant rows, mean_dim different from the row length, sign symmetry
 """
@@ -177,6 +179,16 @@ def online_hadamard(x, force_fp32=False):
     hadk, k = get_hadK(x.shape[-1])
     io = F32 if force_fp32 else x.dtype
     return hadamard_staged(x.astype(io), hadk, k, io).astype(x.dtype)
+
+
+def heads_hadamard(x, num_heads):
+    """The transform in front of o_proj (e2e/quantized_llama/modeling_llama.py:108-109):
+    OnlineHadamard(num_heads) applied to attn_output.transpose(-1, -2), transposed back and reshaped
+    to [..., hidden].  x fp16 [..., num_heads, head_dim] -> fp16 [..., num_heads * head_dim]."""
+    x = np.asarray(x)
+    assert x.shape[-2] == num_heads
+    y = np.swapaxes(online_hadamard(np.swapaxes(x, -1, -2)), -1, -2)
+    return np.ascontiguousarray(y).reshape(*x.shape[:-2], x.shape[-2] * x.shape[-1])
 
 
 # ----------------------------------------------------------------------------------------------

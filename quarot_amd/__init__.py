@@ -15,7 +15,7 @@ from . import nn
 
 __all__ = [
     "matmul", "sym_quant", "sym_dequant", "PackedQuantizedTensor",      # the reference's names
-    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "linear_i4",   # fused entry points
+    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "heads_hadamard_quantize", "linear_i4",   # fused entry points
 ]
 
 
@@ -184,6 +184,29 @@ def rmsnorm_quantize(x, mean_dim, eps=1e-5, clip_ratio=1.0, return_normalized=Fa
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
     return (packed, y.view(x.shape)) if return_normalized else packed
+
+
+def heads_hadamard_quantize(x, num_heads, clip_ratio=1.0, return_transformed=False):
+    """The chain in front of o_proj in one kernel (e2e/quantized_llama/modeling_llama.py:108-110):
+    OnlineHadamard(num_heads) over the head axis of attention's output, then Quantizer.forward on the
+    rows reshaped to [..., hidden].  x is [..., num_heads, head_dim], contiguous, as attention writes
+    it; no transposed copies are made.  head_dim 128 and 16, 32 or 64 heads."""
+    assert x.dtype == torch.float16
+    if x.dim() < 2 or x.shape[-2] != num_heads:
+        raise RuntimeError("heads_hadamard_quantize: x must be [..., num_heads, head_dim]")
+    x2, lead = _flat2d(x.view(*x.shape[:-2], x.shape[-2] * x.shape[-1]))
+    dev = _require_gpu_contiguous("heads_hadamard_quantize", x=x2)
+    rows, cols = x2.shape
+    q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
+    s = torch.empty((rows,), dtype=torch.float16, device=dev)
+    y = torch.empty_like(x2) if return_transformed else None
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().qr_heads_hadamard_quantize_f16_i4(_ptr(x2), rows, int(num_heads), cols // int(num_heads),
+                                                                float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
+                                                                _lib.stream_ptr(dev)))
+    s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
+    packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
+    return (packed, y.view(*lead, cols)) if return_transformed else packed
 
 
 def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):

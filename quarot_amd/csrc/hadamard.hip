@@ -1328,6 +1328,74 @@ int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const vo
     return qr_launch_status();
 }
 
+// Short power-of-two rows (8 ... 64 elements, e.g. the transform across 32 or 64 attention heads on
+// a transposed copy, e2e/quantized_llama/modeling_llama.py:108): many rows per workgroup.  A lane
+// holds 8 consecutive elements of a row (one 16-byte load, consecutive lanes = consecutive memory),
+// n / 8 neighbouring lanes hold a row; three butterfly stages run in the lane, the others between
+// lanes (DPP quad permutes for lane distance 1 and 2, a cross-lane read for 4).  fp32 inside, the
+// scale applied at the end, rounded to fp16 once.
+template <int LPR>
+__global__ __launch_bounds__(256) void hadamard_small_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ y,
+                                                             int64_t chunks, float scale) {
+    const int lane = threadIdx.x & 63;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    // every lane of a wave runs the same number of turns: chunks beyond the end are zeros, not stored
+    const int64_t turns = (chunks + stride - 1) / stride;
+    int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    for (int64_t t = 0; t < turns; ++t, idx += stride) {
+        const bool live = idx < chunks;
+        const u32x4 v = live ? __builtin_nontemporal_load(x + idx) : u32x4{0, 0, 0, 0};
+        float f[8];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const f16x2 h = as_f16x2(v[w]);
+            f[2 * w] = (float)h[0];
+            f[2 * w + 1] = (float)h[1];
+        }
+#pragma unroll
+        for (int b = 1; b < 8; b <<= 1)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if ((e & b) == 0) {
+                    const float lo = f[e], hi = f[e | b];
+                    f[e] = lo + hi;
+                    f[e | b] = lo - hi;
+                }
+#pragma unroll
+        for (int d = 1; d < LPR; d <<= 1) {
+            const bool upper = (lane & d) != 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int own = __builtin_bit_cast(int, f[e]);
+                int other;
+                if (d == 1) other = __builtin_amdgcn_update_dpp(0, own, 0xB1, 0xF, 0xF, true);        // quad_perm [1,0,3,2]
+                else if (d == 2) other = __builtin_amdgcn_update_dpp(0, own, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+                else other = __shfl_xor(own, d, QR_WAVE);
+                const float p = __builtin_bit_cast(float, other);
+                f[e] = upper ? p - f[e] : f[e] + p;
+            }
+        }
+        if (live) {
+            u32x4 o;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) o[w] = narrow_f16x2(f[2 * w] * scale, f[2 * w + 1] * scale);
+            __builtin_nontemporal_store(o, y + idx);
+        }
+    }
+}
+
+int launch_hadamard_small(const void* x, void* y, int64_t rows, int n, float scale, hipStream_t st) {
+    const int64_t chunks = rows * (n / 8);
+    int64_t blocks = (chunks + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    const dim3 grid((unsigned)blocks), block(256);
+    if (n == 8) hadamard_small_kernel<1><<<grid, block, 0, st>>>((const u32x4*)x, (u32x4*)y, chunks, scale);
+    else if (n == 16) hadamard_small_kernel<2><<<grid, block, 0, st>>>((const u32x4*)x, (u32x4*)y, chunks, scale);
+    else if (n == 32) hadamard_small_kernel<4><<<grid, block, 0, st>>>((const u32x4*)x, (u32x4*)y, chunks, scale);
+    else hadamard_small_kernel<8><<<grid, block, 0, st>>>((const u32x4*)x, (u32x4*)y, chunks, scale);
+    return qr_launch_status();
+}
+
 int check_shape(int64_t rows, int n, int K) {
     if (rows < 0 || n <= 0 || K <= 0) return QR_E_SHAPE;
     if (n % K != 0) return QR_E_SHAPE;
@@ -1349,6 +1417,7 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     hipStream_t st = (hipStream_t)stream;
     // head-dimension rows: the kernel whose arithmetic the K-cache quantiser shares
     if (dtype == QR_DTYPE_F16 && K == 1 && n == 128) return qr_internal_hadamard128_f16(x, y, rows, scale, st);
+    if (dtype == QR_DTYPE_F16 && K == 1 && n <= 64) return launch_hadamard_small(x, y, rows, n, scale, st);
     if (dtype == QR_DTYPE_F16 && K == 1 && pow2_split(n))
         return launch_hadamard_mm<true, false>(x, y, rows, n, pow2_split(n), nullptr, scale, 1.f, nullptr, nullptr, st);
     if (dtype == QR_DTYPE_F16 && bm_applies(n, K))

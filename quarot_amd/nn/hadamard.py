@@ -44,3 +44,28 @@ class OnlineHadamardQuantizer(torch.nn.Module):
     def forward(self, x):
         return quarot_amd.hadamard_quantize(x, self.had_rem_dim, self.rem_dim, self.input_clip_ratio,
                                             force_fp32=self.fp32_had)
+
+
+class HeadsHadamardQuantizer(torch.nn.Module):
+    """The three steps in front of o_proj (e2e/quantized_llama/modeling_llama.py:108-110) in one
+    kernel: OnlineHadamard(num_heads) over the head axis of attention's output [..., heads, head_dim]
+    (the reference applies it to a transposed view and transposes back), the reshape to
+    [..., hidden], and o_proj's Quantizer(input_clip_ratio).  Neither the transposed copies nor the
+    transformed fp16 tensor go through HBM.  Shapes the fused kernel does not take (head_dim other
+    than 128, a head count other than 16, 32 or 64, a dtype other than fp16, a strided input) run as
+    the separate steps."""
+
+    def __init__(self, num_heads, input_clip_ratio=1.0):
+        super().__init__()
+        self.num_heads = num_heads
+        self.input_clip_ratio = input_clip_ratio
+        self.had = OnlineHadamard(num_heads)
+
+    def forward(self, x):
+        assert x.shape[-2] == self.num_heads
+        if (x.dtype == torch.float16 and x.shape[-1] == 128 and self.num_heads in (16, 32, 64)
+                and x.is_contiguous()):
+            return quarot_amd.heads_hadamard_quantize(x, self.num_heads, self.input_clip_ratio)
+        y = self.had(x.transpose(-1, -2)).transpose(-1, -2)
+        y = y.reshape(*x.shape[:-2], x.shape[-2] * x.shape[-1]).contiguous()
+        return quarot_amd.PackedQuantizedTensor(*quarot_amd.quantize_rows(y, self.input_clip_ratio))

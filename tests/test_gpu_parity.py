@@ -289,7 +289,7 @@ def test_linear4bit_module_from_float_and_state_dict():
 
 # ------------------------------------------------------------------------------ Hadamard
 
-HAD_SIZES = [8, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
+HAD_SIZES = [8, 16, 32, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
 
 
 def close(got, want):
@@ -311,6 +311,25 @@ def test_hadamard_within_tolerance(n, dtype):
     cf = o.hadamard_closed_form(x.astype(np.float64))
     tol = 3e-3 if dtype == F16 else 1e-5
     assert np.all(np.abs(got - cf) <= tol * (1 + np.abs(cf)))
+
+
+@pytest.mark.parametrize("n", [8, 16, 32, 64])
+def test_hadamard_short_rows_many_per_workgroup(n):
+    """Short rows (the transform across attention heads on a transposed copy): row counts that leave
+    a partly filled last wave and more chunks than one pass of the grid covers, out of place and in
+    place, against the oracle and through the involution H(H(x)) = x."""
+    for rows in (1, 37, 1000, 262144 + 3):
+        x = gpu(synth_x(min(rows, 4096), n, seed=n + rows))
+        if rows > 4096:
+            x = x.repeat((rows + 4095) // 4096, 1)[:rows].contiguous()
+        y = quarot_amd.functional.matmul_hadU_cuda(x, None, 1)
+        sl = slice(None, None, max(1, rows // 500))
+        assert close(y[sl].cpu().numpy(), o.online_hadamard(x[sl].cpu().numpy()))
+        assert close(y[-3:].cpu().numpy(), o.online_hadamard(x[-3:].cpu().numpy()))
+        # two fp16 roundings, each relative to the largest element of the row (outlier channels)
+        back = quarot_amd.functional.matmul_hadU_cuda(y, None, 1)
+        err = (back.float() - x.float()).abs().amax(dim=1)
+        assert bool((err <= 2e-3 * x.float().abs().amax(dim=1) + 1e-3).all())
 
 
 @pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 224, 3840, 6912, 8960, 11008, 28672, 13824])
@@ -389,6 +408,69 @@ def test_fused_rmsnorm_quantize_full_size_and_errors():
     assert L.qr_rmsnorm_quantize_f16_i4(x.data_ptr() + 2, 8, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) == -4
     assert L.qr_rmsnorm_quantize_f16_i4(x.data_ptr(), 0, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) == 0
     assert L.qr_rmsnorm_quantize_f16_i4(None, 8, 4096, 4096, 1e-5, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+
+
+@pytest.mark.parametrize("heads,rows,clip", [(32, 37, 1.0), (64, 19, 0.9), (16, 64, 1.0), (32, 1, 1.0)])
+def test_fused_heads_hadamard_quantize(heads, rows, clip):
+    """Hadamard across attention heads + Quantizer in one kernel (the chain in front of o_proj).  The
+    transformed rows (returned on request) against the oracle to the floating-point tolerance (the
+    sums are formed in a different order, so nearly every element is identical), codes and scales
+    equal to the oracle quantiser applied to the kernel's OWN rows bit for bit, and the module
+    against the three separate steps of the reference's model code."""
+    x = gpu(synth_x(rows, heads * 128, seed=heads + rows)).view(rows, heads, 128)
+    mod = quarot_amd.nn.HeadsHadamardQuantizer(heads, input_clip_ratio=clip)
+    p = mod(x)
+    p2, y = quarot_amd.heads_hadamard_quantize(x, heads, clip, return_transformed=True)
+    assert torch.equal(p.quantized_x, p2.quantized_x) and torch.equal(p.scales_x, p2.scales_x)
+    assert p.quantized_x.shape == (rows, heads * 64) and y.shape == (rows, heads * 128)
+    yk = y.cpu().numpy()
+    want_y = o.heads_hadamard(x.cpu().numpy(), heads)
+    assert close(yk, want_y) and np.mean(yk == want_y) > 0.995
+    wq, ws = o.quantizer(yk, clip)
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    assert np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+    # the reference's own sequence: transform on the transposed view, transpose back, reshape, quantise
+    had = quarot_amd.nn.OnlineHadamard(heads)
+    staged_y = had(x.transpose(-1, -2)).transpose(-1, -2).reshape(rows, heads * 128).contiguous()
+    assert close(staged_y.cpu().numpy(), want_y)
+    staged = quarot_amd.nn.Quantizer(clip)(staged_y)
+    assert p.scales_x.shape == staged.scales_x.shape
+    assert float((p.quantized_x == staged.quantized_x).float().mean()) > 0.99
+
+
+def test_fused_heads_hadamard_quantize_full_size_fallback_and_errors():
+    """Prefill-size input ([2, 1024, 32, 128]) checked on strided rows and through norm preservation;
+    shapes the fused kernel does not take go through the separate steps; argument errors of the C
+    entry point."""
+    x = gpu(synth_x(2048, 4096, seed=9)).view(2, 1024, 32, 128)
+    p, y = quarot_amd.heads_hadamard_quantize(x, 32, 1.0, return_transformed=True)
+    assert p.quantized_x.shape == (2, 1024, 2048) and p.scales_x.shape == (2, 1, 1024)
+    y2 = y.view(2048, 4096)
+    rows = slice(None, None, 131)
+    xs = x.view(2048, 32, 128)[rows].cpu().numpy()
+    assert close(y2[rows].cpu().numpy(), o.heads_hadamard(xs, 32))
+    wq, ws = o.quantizer(y2[rows].cpu().numpy(), 1.0)
+    assert np.array_equal(p.quantized_x.view(2048, -1)[rows].cpu().numpy(), wq)
+    assert np.array_equal(p.scales_x.reshape(-1)[rows].cpu().numpy(), ws)
+    assert torch.allclose(y2.float().norm(dim=1), x.view(2048, 4096).float().norm(dim=1), rtol=2e-3)
+    # 8 heads of 64: the module runs the separate steps
+    xs = gpu(synth_x(5, 512, seed=3)).view(5, 8, 64)
+    pf = quarot_amd.nn.HeadsHadamardQuantizer(8)(xs)
+    yf = o.heads_hadamard(xs.cpu().numpy(), 8)
+    wq, _ = o.quantizer(yf, 1.0)
+    assert pf.quantized_x.shape == (5, 256) and np.mean(pf.quantized_x.cpu().numpy() == wq) > 0.99
+    L = _lib.lib()
+    xf = x.view(2048, 4096)
+    q = torch.empty(8, 2048, dtype=torch.uint8, device=x.device)
+    s = torch.empty(8, dtype=torch.float16, device=x.device)
+    st = torch.cuda.current_stream().cuda_stream
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 8, 64, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 40, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr() + 2, 8, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) == -4
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 0, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) == 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(None, 8, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    with pytest.raises(RuntimeError):
+        quarot_amd.heads_hadamard_quantize(xf, 32)
 
 
 def test_hadamard_full_size_properties():

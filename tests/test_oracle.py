@@ -397,3 +397,31 @@ def test_cpu_baseline_port_agrees_with_oracle():
     y = cb.linear4bit_path(torch.from_numpy(x), torch.from_numpy(wq.astype(np.int32)), torch.from_numpy(ws))
     want = o.linear4bit(o.pack_i4(q.numpy()), sx.numpy().reshape(-1), o.pack_i4(wq), ws)
     assert np.array_equal(y.numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_heads_hadamard_is_the_transform_over_the_head_axis():
+    """The composition transpose -> OnlineHadamard(num_heads) -> transpose -> reshape against an
+    independent float64 einsum with scipy's Sylvester matrix, and cases that a transform over the
+    wrong axis, a missing 1/sqrt(H) or a transposed result would fail."""
+    import scipy.linalg
+    rng = np.random.default_rng(21)
+    for heads, dim in ((32, 128), (64, 128), (16, 8), (8, 4)):
+        x = rng.standard_normal((3, heads, dim)).astype(F16)
+        got = o.heads_hadamard(x, heads)
+        assert got.shape == (3, heads * dim) and got.dtype == F16
+        H = scipy.linalg.hadamard(heads).astype(np.float64)
+        want = np.einsum("gh,rhd->rgd", H, x.astype(np.float64)) / np.sqrt(np.float64(heads))
+        # the oracle multiplies by the float32 scale 1/sqrt(H) before its single rounding: one fp16 ulp
+        assert np.allclose(got.astype(np.float64), want.reshape(3, -1), rtol=2e-3, atol=2e-3)
+        assert np.mean(got == want.reshape(3, -1).astype(F16)) > 0.99
+    # constant across heads: everything lands in head 0, scaled by sqrt(H) (exact for H = 16, 64)
+    c = np.broadcast_to(rng.standard_normal((1, 1, 128)).astype(F16), (1, 64, 128)).copy()
+    y = o.heads_hadamard(c, 64).reshape(64, 128)
+    assert np.array_equal(y[0], (c[0, 0].astype(F32) * F32(8)).astype(F16)) and not y[1:].any()
+    # a single non-zero head h: output head g is Had[g, h] / sqrt(H) times that head's vector
+    e = np.zeros((1, 16, 128), F16)
+    e[0, 5] = rng.standard_normal(128).astype(F16)
+    y = o.heads_hadamard(e, 16).reshape(16, 128)
+    H16 = scipy.linalg.hadamard(16)
+    for g in range(16):
+        assert np.array_equal(y[g], (e[0, 5].astype(F32) * F32(0.25 * H16[g, 5])).astype(F16))
