@@ -156,30 +156,28 @@ __global__ __launch_bounds__(QT) void rmsnorm_quant_rows_kernel(const u32x4* __r
 
 // Hadamard across the heads of an attention output row, then the quantiser, in one pass
 // (e2e/quantized_llama/modeling_llama.py:108-110: OnlineHadamard(num_heads) on the transposed view,
-// transpose back, reshape, then o_proj's Quantizer).  A row is [H, 128] fp16, H = 16 NC heads; the
+// transpose back, reshape, then o_proj's Quantizer).  A row is [H, 128] fp16, H = 4 NC heads; the
 // transform is the Walsh-Hadamard transform of size H over the head index for each of the 128
 // positions, scaled by 1/sqrt(H) and rounded to fp16 once (quarot/nn/hadamard.py:17-23 with K = 1).
-// One workgroup of 256 threads per row; thread t holds the 16-byte chunks t + 256 i, i.e. heads
-// (t >> 4) + 16 i at positions 8 (t & 15) ...: head bits 4.. are the chunk index i (butterflies in
-// the thread), bits 0 and 1 are lane bits 4 and 5 (one v_permlane16_swap / v_permlane32_swap per
-// value: after swapping a register with its own copy, both partners hold (lower, upper) and take the
-// sum or the difference), bits 2 and 3 are the wave index (a four-point transform through LDS).
+// One WAVE per row, four rows per workgroup, no LDS and no barrier: lane l holds the 16-byte chunks
+// l + 64 i, i.e. heads (l >> 4) + 4 i at positions 8 (l & 15) ...: head bits 2.. are the chunk index
+// i (butterflies in the lane), bits 0 and 1 are lane bits 4 and 5 (one v_permlane16_swap /
+// v_permlane32_swap per value: after swapping a register with its own copy, both partners hold
+// (lower, upper) and take the sum or the difference).  The row maximum is a wave reduction.
 template <int NC>
-__global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32x4* __restrict__ x, float hscale,
-                                                                       float clip, u32* __restrict__ q,
+__global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32x4* __restrict__ x, int64_t rows,
+                                                                       float hscale, float clip, u32* __restrict__ q,
                                                                        f16* __restrict__ scale_out,
                                                                        u32x4* __restrict__ y) {
-    static_assert(QT == 256, "the head-to-thread mapping assumes four waves");
-    constexpr int cols8 = NC * QT;
-    __shared__ f32x4 xch[4][NC * 2][QR_WAVE];                // [wave][chunk, half][lane]
-    __shared__ u32 red[QT / QR_WAVE];
-    const int64_t row = blockIdx.x;
+    constexpr int cols8 = NC * QR_WAVE;
     const int lane = threadIdx.x & (QR_WAVE - 1), wave = threadIdx.x / QR_WAVE;
+    const int64_t row = (int64_t)blockIdx.x * (QT / QR_WAVE) + wave;
+    if (row >= rows) return;                                // a whole wave: nothing below synchronises waves
     const u32x4* xr = x + row * (int64_t)cols8;
     float f[NC][8];
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-        const u32x4 v = xr[threadIdx.x + i * QT];
+        const u32x4 v = xr[lane + i * QR_WAVE];
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const f16x2 h = as_f16x2(v[w]);
@@ -187,7 +185,7 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
             f[i][2 * w + 1] = (float)h[1];
         }
     }
-    // head bits 4..: pairs of chunks of this thread
+    // head bits 2..: pairs of chunks of this lane
 #pragma unroll
     for (int b = 1; b < NC; b <<= 1)
 #pragma unroll
@@ -200,10 +198,12 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
                     f[i | b][e] = lo - hi;
                 }
             }
-    // head bits 0 and 1: lanes 16 and 32 apart
+    // head bits 0 and 1: lanes 16 and 32 apart; then scale and round to fp16
     const bool up16 = (lane & 16) != 0, up32 = (lane & 32) != 0;
+    u32x4 v[NC];
+    u32 m = 0;
 #pragma unroll
-    for (int i = 0; i < NC; ++i)
+    for (int i = 0; i < NC; ++i) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const u32 a = __builtin_bit_cast(u32, f[i][e]);
@@ -215,58 +215,30 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
             const float lo2 = __builtin_bit_cast(float, (u32)s32[0]), hi2 = __builtin_bit_cast(float, (u32)s32[1]);
             f[i][e] = up32 ? lo2 - hi2 : lo2 + hi2;
         }
-    // head bits 2 and 3: the four waves
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-        xch[wave][2 * i][lane] = f32x4{f[i][0], f[i][1], f[i][2], f[i][3]};
-        xch[wave][2 * i + 1][lane] = f32x4{f[i][4], f[i][5], f[i][6], f[i][7]};
-    }
-    __syncthreads();
-    u32x4 v[NC];
-    u32 m = 0;
-#pragma unroll
-    for (int i = 0; i < NC; ++i) {
-        float o[8];
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            const f32x4 w0 = xch[0][2 * i + hf][lane], w1 = xch[1][2 * i + hf][lane];
-            const f32x4 w2 = xch[2][2 * i + hf][lane], w3 = xch[3][2 * i + hf][lane];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                // two butterfly stages: wave bit 0 (waves 0,1 and 2,3), then wave bit 1
-                const float s01 = (wave & 1) ? w0[e] - w1[e] : w0[e] + w1[e];
-                const float s23 = (wave & 1) ? w2[e] - w3[e] : w2[e] + w3[e];
-                o[4 * hf + e] = (wave & 2) ? s01 - s23 : s01 + s23;
-            }
-        }
-#pragma unroll
-        for (int w = 0; w < 4; ++w) v[i][w] = narrow_f16x2(o[2 * w] * hscale, o[2 * w + 1] * hscale);
+        for (int w = 0; w < 4; ++w) v[i][w] = narrow_f16x2(f[i][2 * w] * hscale, f[i][2 * w + 1] * hscale);
         const u32 mi = absmax_bits8(v[i]);
         m = m > mi ? m : mi;
     }
     m = wave_max_u32_dpp(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
     const f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
-    if (threadIdx.x == 0) scale_out[row] = sh;
+    if (lane == 0) scale_out[row] = sh;
     const float s = (float)sh;
     u32* qr = q + row * (int64_t)cols8;
     if (y) {
 #pragma unroll
-        for (int i = 0; i < NC; ++i) y[row * (int64_t)cols8 + threadIdx.x + i * QT] = v[i];
+        for (int i = 0; i < NC; ++i) y[row * (int64_t)cols8 + lane + i * QR_WAVE] = v[i];
     }
-    if (fast_quant_ok(m, s)) {       // workgroup-uniform
+    if (fast_quant_ok(m, s)) {       // wave-uniform
         const FastRecip fr = make_fast_recip(s);
 #pragma unroll
-        for (int i = 0; i < NC; ++i) qr[threadIdx.x + i * QT] = sym_codes8_fast(v[i], fr);
+        for (int i = 0; i < NC; ++i) qr[lane + i * QR_WAVE] = sym_codes8_fast(v[i], fr);
         return;
     }
     const bool fast = scale_fast_ok(s);
     const float rs = fast ? 1.0f / s : 0.0f;
 #pragma unroll
-    for (int i = 0; i < NC; ++i) qr[threadIdx.x + i * QT] = sym_codes8(v[i], s, rs, fast);
+    for (int i = 0; i < NC; ++i) qr[lane + i * QR_WAVE] = sym_codes8(v[i], s, rs, fast);
 }
 
 // Any column count (odd included), any alignment: one workgroup per row, scalar accesses, the row
@@ -414,15 +386,15 @@ extern "C" int qr_heads_hadamard_quantize_f16_i4(const void* x, int64_t rows, in
     if (!x || !q || !scales) return QR_E_NULL;
     if (head_dim != 128 || (heads != 16 && heads != 32 && heads != 64)) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
-    dim3 grid((unsigned)rows), block(QT);
+    dim3 grid((unsigned)((rows + QT / QR_WAVE - 1) / (QT / QR_WAVE))), block(QT);
     hipStream_t st = (hipStream_t)stream;
     const float hscale = 1.0f / __builtin_sqrtf((float)heads);
 #define QR_LAUNCH(NC)                                                                                                 \
-    heads_hadamard_quant_rows_kernel<NC><<<grid, block, 0, st>>>((const u32x4*)x, hscale, clip, (u32*)q, (f16*)scales, \
-                                                                 (u32x4*)y_or_null)
-    if (heads == 16) QR_LAUNCH(1);
-    else if (heads == 32) QR_LAUNCH(2);
-    else QR_LAUNCH(4);
+    heads_hadamard_quant_rows_kernel<NC><<<grid, block, 0, st>>>((const u32x4*)x, rows, hscale, clip, (u32*)q,        \
+                                                                 (f16*)scales, (u32x4*)y_or_null)
+    if (heads == 16) QR_LAUNCH(4);
+    else if (heads == 32) QR_LAUNCH(8);
+    else QR_LAUNCH(16);
 #undef QR_LAUNCH
     return qr_launch_status();
 }
