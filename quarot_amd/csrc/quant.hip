@@ -161,9 +161,8 @@ __global__ __launch_bounds__(QT) void rmsnorm_quant_rows_kernel(const u32x4* __r
 // positions, scaled by 1/sqrt(H) and rounded to fp16 once (quarot/nn/hadamard.py:17-23 with K = 1).
 // One WAVE per row, four rows per workgroup, no LDS and no barrier: lane l holds the 16-byte chunks
 // l + 64 i, i.e. heads (l >> 4) + 4 i at positions 8 (l & 15) ...: head bits 2.. are the chunk index
-// i (butterflies in the lane), bits 0 and 1 are lane bits 4 and 5 (one v_permlane16_swap /
-// v_permlane32_swap per value: after swapping a register with its own copy, both partners hold
-// (lower, upper) and take the sum or the difference).  The row maximum is a wave reduction.
+// i (butterflies in the lane), bits 0 and 1 are lane bits 4 and 5 (v_permlane16_swap /
+// v_permlane32_swap, one swap per butterfly).  The row maximum is a wave reduction.
 template <int NC>
 __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32x4* __restrict__ x, int64_t rows,
                                                                        float hscale, float clip, u32* __restrict__ q,
@@ -174,20 +173,27 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
     const int64_t row = (int64_t)blockIdx.x * (QT / QR_WAVE) + wave;
     if (row >= rows) return;                                // a whole wave: nothing below synchronises waves
     const u32x4* xr = x + row * (int64_t)cols8;
-    float f[NC][8];
+    u32x4 raw[NC];
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-        const u32x4 v = xr[lane + i * QR_WAVE];
+    for (int i = 0; i < NC; ++i) raw[i] = xr[lane + i * QR_WAVE];
+    // head bits 2..: pairs of chunks of this lane.  The first stage reads the fp16 pairs directly
+    // (fused multiply-adds by +-1 with fp16 sources: one instruction converts and adds).
+    float f[NC][8];
+    float one = 1.0f, minus_one = -1.0f;
+    asm volatile("" : "+v"(one), "+v"(minus_one));           // opaque, or the compiler splits the fma into convert + add
+#pragma unroll
+    for (int i = 0; i < NC; i += 2)
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const f16x2 h = as_f16x2(v[w]);
-            f[i][2 * w] = (float)h[0];
-            f[i][2 * w + 1] = (float)h[1];
-        }
-    }
-    // head bits 2..: pairs of chunks of this lane
+            const f16x2 lo = as_f16x2(raw[i][w]), hi = as_f16x2(raw[i + 1][w]);
 #pragma unroll
-    for (int b = 1; b < NC; b <<= 1)
+            for (int k = 0; k < 2; ++k) {
+                f[i][2 * w + k] = __builtin_fmaf((float)hi[k], one, (float)lo[k]);
+                f[i + 1][2 * w + k] = __builtin_fmaf((float)hi[k], minus_one, (float)lo[k]);
+            }
+        }
+#pragma unroll
+    for (int b = 2; b < NC; b <<= 1)
 #pragma unroll
         for (int i = 0; i < NC; ++i)
             if ((i & b) == 0) {
@@ -198,22 +204,36 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
                     f[i | b][e] = lo - hi;
                 }
             }
-    // head bits 0 and 1: lanes 16 and 32 apart; then scale and round to fp16
-    const bool up16 = (lane & 16) != 0, up32 = (lane & 32) != 0;
+    // head bits 0 and 1: lanes 16 and 32 apart.  Two values A, B of a lane go through a stage together:
+    // swapping A with B across the lane pair leaves (A_lower, A_upper) in the lower lane and
+    // (B_lower, B_upper) in the upper one; each forms sum and difference of what it holds, and a second
+    // swap hands the lower lane both sums and the upper lane both differences -- two swaps, one add
+    // and one subtract for two butterflies.  Then scale and round to fp16.
     u32x4 v[NC];
     u32 m = 0;
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const u32 a = __builtin_bit_cast(u32, f[i][e]);
-            const auto s16 = __builtin_amdgcn_permlane16_swap(a, a, false, false);
-            const float lo = __builtin_bit_cast(float, (u32)s16[0]), hi = __builtin_bit_cast(float, (u32)s16[1]);
-            const float g = up16 ? lo - hi : lo + hi;
-            const u32 c = __builtin_bit_cast(u32, g);
-            const auto s32 = __builtin_amdgcn_permlane32_swap(c, c, false, false);
-            const float lo2 = __builtin_bit_cast(float, (u32)s32[0]), hi2 = __builtin_bit_cast(float, (u32)s32[1]);
-            f[i][e] = up32 ? lo2 - hi2 : lo2 + hi2;
+        for (int e = 0; e < 8; e += 2) {
+            u32 a = __builtin_bit_cast(u32, f[i][e]), c = __builtin_bit_cast(u32, f[i][e + 1]);
+            {
+                const auto s1 = __builtin_amdgcn_permlane16_swap(a, c, false, false);
+                const float lo = __builtin_bit_cast(float, (u32)s1[0]), hi = __builtin_bit_cast(float, (u32)s1[1]);
+                const auto s2 = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(u32, lo + hi),
+                                                                 __builtin_bit_cast(u32, lo - hi), false, false);
+                a = s2[0];
+                c = s2[1];
+            }
+            {
+                const auto s1 = __builtin_amdgcn_permlane32_swap(a, c, false, false);
+                const float lo = __builtin_bit_cast(float, (u32)s1[0]), hi = __builtin_bit_cast(float, (u32)s1[1]);
+                const auto s2 = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(u32, lo + hi),
+                                                                 __builtin_bit_cast(u32, lo - hi), false, false);
+                a = s2[0];
+                c = s2[1];
+            }
+            f[i][e] = __builtin_bit_cast(float, a);
+            f[i][e + 1] = __builtin_bit_cast(float, c);
         }
 #pragma unroll
         for (int w = 0; w < 4; ++w) v[i][w] = narrow_f16x2(f[i][2 * w] * hscale, f[i][2 * w + 1] * hscale);
