@@ -1,7 +1,7 @@
 """The reference's CPU-capable statement of the path, in torch, for TIMING on host cores.
 TEST/BENCHMARK INFRASTRUCTURE ONLY (never imported by the shipped package).
 
-It is the chain BASELINE names: the repo's PyTorch Hadamard (matmul_hadU,
+It chains the reference's CPU-capable pieces: its PyTorch Hadamard (matmul_hadU,
 fake_quant/hadamard_utils.py:58-79), per-token symmetric quantisation
 (fake_quant/quant_utils.py:30-33 with the scale of quarot/nn/quantization.py:10), a torch integer
 matmul on unpacked int32 codes (what quarot/kernels/gemm.cu:7-46 computes), and the fp16 dequant of
