@@ -76,11 +76,20 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
                                                       u32* __restrict__ q, f16* __restrict__ scale,
                                                       f16* __restrict__ zero) {
     const int lane = threadIdx.x & 63;
-    const int64_t stride = (int64_t)gridDim.x * KT;      // multiple of 64 > lanes per vector
-    for (int64_t c0 = (int64_t)blockIdx.x * KT; c0 < nchunks; c0 += stride) {
-        const int64_t c = c0 + threadIdx.x;
-        const bool live = c < nchunks;                   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
-        u32x4 hp = live ? *(x + c) : u32x4{0, 0, 0, 0};  // the 8 fp16 values to quantise, packed
+    constexpr int U = 4;                                 // chunks per thread and turn: their loads are all issued first
+    const int64_t stride = (int64_t)gridDim.x * KT * U;  // multiple of 64 > lanes per vector
+    for (int64_t c0 = (int64_t)blockIdx.x * KT * U; c0 < nchunks; c0 += stride) {
+      u32x4 hps[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+          const int64_t c = c0 + u * KT + threadIdx.x;
+          hps[u] = c < nchunks ? __builtin_nontemporal_load(x + c) : u32x4{0, 0, 0, 0};
+      }
+      u32 outws[U];
+      f16 scs[U], zps[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        u32x4 hp = hps[u];                               // the 8 fp16 values to quantise, packed
         if (HAD) {
             float v[8];
 #pragma unroll
@@ -174,13 +183,21 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
                 outw |= (u32)code << (4 * e);
             }
         }
-        if (live) {
-            q[c] = outw;
-            if ((lane & ((1 << LG) - 1)) == 0) {
-                scale[c >> LG] = sc;
-                zero[c >> LG] = zp;
-            }
-        }
+        outws[u] = outw;
+        scs[u] = sc;
+        zps[u] = zp;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+          const int64_t c = c0 + u * KT + threadIdx.x;   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
+          if (c < nchunks) {
+              q[c] = outws[u];
+              if ((lane & ((1 << LG) - 1)) == 0) {
+                  scale[c >> LG] = scs[u];
+                  zero[c >> LG] = zps[u];
+              }
+          }
+      }
     }
 }
 
@@ -438,8 +455,8 @@ int log2_dim(int dim) {
     return -1;
 }
 
-unsigned grid_for(int64_t nchunks) {
-    int64_t b = (nchunks + KT - 1) / KT;
+unsigned grid_for(int64_t nchunks, int per_block = KT) {
+    int64_t b = (nchunks + per_block - 1) / per_block;
     const int64_t cap = 256 * 32;
     return (unsigned)(b < cap ? b : cap);
 }
@@ -460,7 +477,7 @@ extern "C" int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int h
     hipStream_t st = (hipStream_t)stream;
     if (dim == 128 && had_mode == 1 && (((uintptr_t)q & 15) == 0))
         return launch_had128<true>(x, vectors, hs, q, scale, zero, nullptr, st);
-    dim3 grid(grid_for(nchunks)), block(KT);
+    dim3 grid(grid_for(nchunks, 4 * KT)), block(KT);
 #define QR_KV(LG)                                                                                                     \
     case LG + 3:                                                                                                      \
         if (had_mode)                                                                                                 \
