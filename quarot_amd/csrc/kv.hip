@@ -205,18 +205,33 @@ template <int LG>
 __global__ __launch_bounds__(KT) void kv_dequant_kernel(const u32* __restrict__ q, const f16* __restrict__ scale,
                                                         const f16* __restrict__ zero, int64_t nchunks,
                                                         u32x4* __restrict__ y) {
-    const int64_t stride = (int64_t)gridDim.x * KT;
-    for (int64_t c = (int64_t)blockIdx.x * KT + threadIdx.x; c < nchunks; c += stride) {
-        const u32 w = *(q + c);
-        const f16 sc = scale[c >> LG], zp = zero[c >> LG];
-        u32x4 o;
+    constexpr int U = 4;                                 // chunks per thread and turn: their loads are all issued first
+    const int64_t stride = (int64_t)gridDim.x * KT * U;
+    for (int64_t c0 = (int64_t)blockIdx.x * KT * U + threadIdx.x; c0 < nchunks; c0 += stride) {
+        u32 ws[U];
+        f16 scs[U], zps[U];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const f16 a = (f16)((f16)(float)((w >> (8 * i)) & 0xfu) * sc) - zp;
-            const f16 b = (f16)((f16)(float)((w >> (8 * i + 4)) & 0xfu) * sc) - zp;
-            o[i] = (u32)f16_bits(a) | ((u32)f16_bits(b) << 16);
+        for (int u = 0; u < U; ++u) {
+            const int64_t c = c0 + u * KT;
+            const int64_t cc = c < nchunks ? c : nchunks - 1;
+            ws[u] = *(q + cc);
+            scs[u] = scale[cc >> LG];
+            zps[u] = zero[cc >> LG];
         }
-        __builtin_nontemporal_store(o, y + c);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t c = c0 + u * KT;
+            const u32 w = ws[u];
+            const f16 sc = scs[u], zp = zps[u];
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16 a = (f16)((f16)(float)((w >> (8 * i)) & 0xfu) * sc) - zp;
+                const f16 b = (f16)((f16)(float)((w >> (8 * i + 4)) & 0xfu) * sc) - zp;
+                o[i] = (u32)f16_bits(a) | ((u32)f16_bits(b) << 16);
+            }
+            if (c < nchunks) __builtin_nontemporal_store(o, y + c);
+        }
     }
 }
 
@@ -510,7 +525,7 @@ extern "C" int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void
     if (((uintptr_t)y & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
     const int64_t nchunks = vectors * (dim / 8);
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(grid_for(nchunks)), block(KT);
+    dim3 grid(grid_for(nchunks, 4 * KT)), block(KT);
     switch (l2 - 3) {
         case 1: kv_dequant_kernel<1><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
         case 2: kv_dequant_kernel<2><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
