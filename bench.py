@@ -74,7 +74,7 @@ TRAFFIC_KIB = {
     "c4": (62375.6, 1024.0),
     "c4m1": (57494.0, 16.0),
     "c4g64": (124423.7, 7168.0),
-    "c5": (131145.2, 69808.6),              # kv_had128_kernel (K cache), per launch
+    "c5": (131145.3, 69774.2),              # kv_had128_kernel (K cache), per launch
 }
 
 
