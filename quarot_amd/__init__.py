@@ -7,6 +7,8 @@ its C ABI.  Extras that fuse adjacent steps are listed after the reference's nam
 
     import quarot_amd as quarot
 """
+import functools
+
 import torch
 
 from . import _lib
@@ -62,7 +64,7 @@ def matmul(A, B):
         raise RuntimeError(f"matmul: inner sizes differ ({A2.shape[1]} vs {B2.shape[1]} packed bytes)")
     M, N, K = A2.shape[0], B2.shape[0], A2.shape[1] * 2
     C = torch.empty((M, N), dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_matmul_i4_i32(_ptr(A2), _ptr(B2), M, N, K, _ptr(C), _lib.stream_ptr(dev)))
     return C.view(*a_lead, *b_lead)
 
@@ -78,7 +80,7 @@ def sym_quant(x, scale):
         raise RuntimeError(f"sym_quant: expected scale of size {x2.shape[0]}, got {s.shape[0]}")
     rows, cols = x2.shape
     q = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_sym_quant_f16_i4(_ptr(x2), _ptr(s), rows, cols, _ptr(q), _lib.stream_ptr(dev)))
     return q.view(*lead, q.shape[-1])
 
@@ -98,7 +100,7 @@ def sym_dequant(q, scale_row, scale_col, bits=32):
     if bits != 32:
         raise RuntimeError("Unsupported data type")       # quarot/kernels/bindings.cpp:76-84
     y = torch.empty((rows, cols), dtype=torch.float16, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_sym_dequant_i32_f16(_ptr(q2), _ptr(sr), _ptr(scale_col), rows, cols, _ptr(y),
                                                      _lib.stream_ptr(dev)))
     return y.view(*lead, y.shape[-1])
@@ -135,7 +137,7 @@ def quantize_rows(x, clip_ratio=1.0):
     rows, cols = x2.shape
     q = torch.empty((rows, (cols + 1) // 2), dtype=torch.uint8, device=dev)
     s = torch.empty((rows,), dtype=torch.float16, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_quantize_rows_f16_i4(_ptr(x2), float(clip_ratio), rows, cols, _ptr(q), _ptr(s),
                                                       _lib.stream_ptr(dev)))
     # torch.max(dim=-1)[0].unsqueeze(1) on [..., C] gives shape lead[:1] + (1,) + lead[1:]
@@ -156,9 +158,9 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
     q = torch.empty((rows, n // 2), dtype=torch.uint8, device=dev)
     s = torch.empty((rows,), dtype=torch.float16, device=dev)
     y = torch.empty_like(x2) if return_transformed else None
-    scale = float(1.0 / torch.tensor(n).sqrt())
+    scale = functional.hadamard.had_scale(n)
     mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
                                                           float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                           _lib.stream_ptr(dev)))
@@ -177,7 +179,7 @@ def rmsnorm_quantize(x, mean_dim, eps=1e-5, clip_ratio=1.0, return_normalized=Fa
     q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
     s = torch.empty((rows,), dtype=torch.float16, device=dev)
     y = torch.empty_like(x2) if return_normalized else None
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_rmsnorm_quantize_f16_i4(_ptr(x2), rows, cols, int(mean_dim), float(eps),
                                                          float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                          _lib.stream_ptr(dev)))
@@ -200,13 +202,18 @@ def heads_hadamard_quantize(x, num_heads, clip_ratio=1.0, return_transformed=Fal
     q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
     s = torch.empty((rows,), dtype=torch.float16, device=dev)
     y = torch.empty_like(x2) if return_transformed else None
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_heads_hadamard_quantize_f16_i4(_ptr(x2), rows, int(num_heads), cols // int(num_heads),
                                                                 float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                                 _lib.stream_ptr(dev)))
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
     return (packed, y.view(*lead, cols)) if return_transformed else packed
+
+
+@functools.lru_cache(maxsize=4096)
+def _workspace_bytes(M, N, K):
+    return _lib.lib().qr_workspace_bytes(M, N, K)
 
 
 def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
@@ -224,8 +231,8 @@ def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
         raise RuntimeError("linear_i4: bias must be fp16 of size out_features")
     y = torch.empty((M, N), dtype=torch.float16, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
-        ws_bytes = L.qr_workspace_bytes(M, N, K)
+    with _lib.on_device(dev):
+        ws_bytes = _workspace_bytes(M, N, K)
         if ws_bytes:
             # few output tiles: the library splits K across workgroups and needs int32 scratch for the sums
             ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)

@@ -58,5 +58,29 @@ def check(code):
 
 
 def stream_ptr(device):
+    """Raw handle of torch's current stream on `device` (the library launches there)."""
     import torch
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None and device.index is not None:
+        return raw(device.index)                 # same value, without building a Stream object
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def on_device(device):
+    """Context that makes `device` current for the launch; nothing to do (and nothing to pay) when
+    it already is."""
+    import torch
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)

@@ -108,17 +108,23 @@ def _run(x, hadK, K, scale):
         hadK = hadK.to(device=xc.device, dtype=xc.dtype).contiguous()
     y = torch.empty_like(xc)
     code = _lib.QR_DTYPE_F16 if xc.dtype == torch.float16 else _lib.QR_DTYPE_F32
-    with torch.cuda.device(xc.device):
+    with _lib.on_device(xc.device):
         _lib.check(_lib.lib().qr_hadamard(xc.data_ptr(), y.data_ptr(), rows, n, int(K),
                                           None if hadK is None else hadK.data_ptr(), code, scale,
                                           _lib.stream_ptr(xc.device)))
     return y
 
 
+@functools.lru_cache(maxsize=None)
+def had_scale(n):
+    """The reference's scale, 1.0 / torch.tensor(n).sqrt() (a float32; hadamard.py:95,99), as a Python float."""
+    return float(1.0 / torch.tensor(n).sqrt())
+
+
 def matmul_hadU_cuda(X, hadK, K):
     """X . (hadK (x) H_{n/K})^T / sqrt(n) on the GPU (hadamard.py:92-101); output in X's dtype and shape."""
     n = X.shape[-1]
-    scale = float(1.0 / torch.tensor(n).sqrt())
+    scale = had_scale(n)
     return _run(X, hadK if K > 1 else None, K, scale).reshape(X.shape)
 
 

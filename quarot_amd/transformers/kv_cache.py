@@ -28,7 +28,7 @@ def asym_quantize_and_pack_i4(x: torch.Tensor, hadamard: bool = False):
     q = torch.empty((*lead, dim // 2), dtype=torch.uint8, device=xc.device)
     scale = torch.empty((*lead, 1), dtype=torch.float16, device=xc.device)
     zero = torch.empty((*lead, 1), dtype=torch.float16, device=xc.device)
-    with torch.cuda.device(xc.device):
+    with _lib.on_device(xc.device):
         _lib.check(_lib.lib().qr_kv_quant_f16_i4(xc.data_ptr(), vecs, dim, 1 if hadamard else 0, q.data_ptr(),
                                                  scale.data_ptr(), zero.data_ptr(), _lib.stream_ptr(xc.device)))
     return q, scale, zero
@@ -47,7 +47,7 @@ def unpack_i4_and_asym_dequantize(q, scale, zero):
     if sc.numel() != vecs or zc.numel() != vecs:
         raise RuntimeError("unpack_i4_and_asym_dequantize: one scale and zero per vector expected")
     y = torch.empty((*qc.shape[:-1], half_dim * 2), dtype=torch.float16, device=qc.device)
-    with torch.cuda.device(qc.device):
+    with _lib.on_device(qc.device):
         _lib.check(_lib.lib().qr_kv_dequant_i4_f16(qc.data_ptr(), sc.data_ptr(), zc.data_ptr(), vecs, half_dim * 2,
                                                    y.data_ptr(), _lib.stream_ptr(qc.device)))
     return y
