@@ -69,6 +69,7 @@ FETCH_SCALE, WRITE_SCALE = 262144.0 / 131083.8, 262144.0 / 262144.0
 TRAFFIC_KIB = {
     #        FETCH_SIZE   WRITE_SIZE
     "c1": (16551.0, 16384.0),
+    "c1o": (16590.5, 16384.0),
     "c2": (44210.0, 16384.0),
     "c3d": (528791.7, 262144.0),
     "c4": (62375.6, 1024.0),
