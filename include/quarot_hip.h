@@ -31,6 +31,7 @@ extern "C" {
 #define QR_E_UNSUPPORTED -3  /* valid for the reference but outside what this build implements */
 #define QR_E_ALIGN      -4   /* a pointer is not aligned as the entry point requires */
 #define QR_E_DTYPE      -5   /* unknown dtype / mode code */
+#define QR_E_WORKSPACE  -6   /* the workspace is NULL, misaligned or smaller than the entry point needs */
 
 #define QR_DTYPE_F16 0
 #define QR_DTYPE_F32 1
@@ -163,6 +164,26 @@ size_t qr_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void* sW,
                         const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * A whole quantised linear layer in one host call: the module chain
+ *   torch.nn.Sequential(OnlineHadamard(K), Quantizer(clip), Linear4bit)        (had_K >= 1)
+ *   torch.nn.Sequential(Quantizer(clip), Linear4bit)                           (had_K == 0)
+ * of e2e/quantized_llama/modeling_llama.py:99-102,111-115 (quarot/nn/hadamard.py:17-23,
+ * quarot/nn/quantization.py:9-13, quarot/nn/linear.py:42-56).  It enqueues exactly the launches of
+ * qr_hadamard_quantize_f16_i4 (or qr_quantize_rows_f16_i4) and qr_linear_i4_f16_ws on `stream`, with
+ * the codes and scales between them in `workspace`: same results bit for bit, one call instead of
+ * two for hosts whose per-call cost matters (a decode step launched from Python).
+ *   x fp16 [M, K]; had_K, hadK, mode, scale as in qr_hadamard_quantize_f16_i4; W uint8 [N, K/2],
+ *   sW fp16 [N], bias fp16 [N] or NULL -> y fp16 [M, N].
+ *   workspace: device memory, 16-byte aligned, at least qr_quantized_linear_workspace_bytes(M, N, K)
+ *   bytes (never 0 for M > 0), else QR_E_WORKSPACE.  Calls that share a workspace must not overlap.
+ */
+size_t qr_quantized_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int had_K, const void* hadK, int mode,
+                            float scale, float clip, const void* W, const void* sW,
+                            const void* bias_or_null, int64_t N, void* y, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /*
  * KV-cache path: optional Hadamard over the head dimension, then per-vector asymmetric int4.

@@ -17,7 +17,7 @@ from . import nn
 
 __all__ = [
     "matmul", "sym_quant", "sym_dequant", "PackedQuantizedTensor",      # the reference's names
-    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "heads_hadamard_quantize", "linear_i4",   # fused entry points
+    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "heads_hadamard_quantize", "linear_i4", "quantized_linear",   # fused entry points
 ]
 
 
@@ -241,4 +241,40 @@ def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
         else:
             _lib.check(L.qr_linear_i4_f16(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K, _ptr(y),
                                           _lib.stream_ptr(dev)))
+    return y.view(*lead, N)
+
+
+@functools.lru_cache(maxsize=4096)
+def _quantized_linear_workspace_bytes(M, N, K):
+    return _lib.lib().qr_quantized_linear_workspace_bytes(M, N, K)
+
+
+def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_ratio=1.0, force_fp32=False):
+    """Sequential(OnlineHadamard, Quantizer, Linear4bit) -- or, with K == 0, Sequential(Quantizer,
+    Linear4bit) -- in ONE call into the library (e2e/quantized_llama/modeling_llama.py:99-102,111-115):
+    the same two launches as hadamard_quantize / quantize_rows followed by linear_i4, same results bit
+    for bit, half the host-side cost.  x fp16 [..., in_features] -> fp16 [..., out_features]."""
+    assert x.dtype == torch.float16
+    assert x.shape[-1] % 64 == 0, "in_features: {} must be a multiple of 64".format(x.shape[-1])
+    x2, lead = _flat2d(x)
+    sw = weight_scales.view(-1)
+    dev = _require_gpu_contiguous("quantized_linear", x=x2, weight=weight, weight_scales=sw, bias=bias, hadK=hadK)
+    M, n = x2.shape
+    N = weight.shape[0]
+    if weight.shape[1] * 2 != n or sw.shape[0] != N or sw.dtype != torch.float16 or weight.dtype != torch.uint8:
+        raise RuntimeError("quantized_linear: inconsistent operand sizes or dtypes")
+    if bias is not None and (bias.dtype != torch.float16 or bias.numel() != N):
+        raise RuntimeError("quantized_linear: bias must be fp16 of size out_features")
+    want = torch.float32 if force_fp32 else torch.float16
+    if hadK is not None and hadK.dtype != want:
+        hadK = hadK.to(want)
+    y = torch.empty((M, N), dtype=torch.float16, device=dev)
+    ws_bytes = _quantized_linear_workspace_bytes(M, N, n)
+    ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
+    mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_quantized_linear_f16(_ptr(x2), M, n, int(K), _ptr(hadK), mode,
+                                                      functional.hadamard.had_scale(n), float(clip_ratio), _ptr(weight),
+                                                      _ptr(sw), _ptr(bias), N, _ptr(y), _ptr(ws), ws_bytes,
+                                                      _lib.stream_ptr(dev)))
     return y.view(*lead, N)

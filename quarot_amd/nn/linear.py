@@ -56,3 +56,37 @@ class Linear4bit(torch.nn.Module):
         if module.bias is not None:
             q4.bias.copy_(module.bias)
         return q4
+
+
+class Linear4bitSequential(torch.nn.Sequential):
+    """torch.nn.Sequential for the module chains the reference builds around Linear4bit
+    (e2e/quantized_llama/modeling_llama.py:99-102,111-115):
+        Linear4bitSequential(OnlineHadamard(n), Quantizer(), Linear4bit.from_float(...))
+        Linear4bitSequential(Quantizer(), Linear4bit.from_float(...))
+    Same constructor, same state-dict keys ("0.had_rem_dim", "2.weight", ...) and same results; when
+    the chain has one of these two shapes and the input is a contiguous fp16 GPU tensor the forward
+    pass is ONE call into the library instead of one per module.  Anything else runs module by
+    module like the base class."""
+
+    def _plan(self):
+        from .hadamard import OnlineHadamard
+        from .quantization import Quantizer
+        mods = list(self)
+        had = None
+        if len(mods) == 3 and isinstance(mods[0], OnlineHadamard):
+            had, mods = mods[0], mods[1:]
+        if len(mods) == 2 and isinstance(mods[0], Quantizer) and isinstance(mods[1], Linear4bit):
+            return had, mods[0], mods[1]
+        return None
+
+    def forward(self, x):
+        plan = self._plan()
+        if (plan is None or not isinstance(x, torch.Tensor) or x.dtype != torch.float16 or not x.is_cuda
+                or not x.is_contiguous() or x.shape[-1] % 64 != 0):
+            return super().forward(x)
+        had, quantizer, lin = plan
+        if had is None:
+            return quarot_amd.quantized_linear(x, lin.weight, lin.weight_scales, lin.bias,
+                                               clip_ratio=quantizer.input_clip_ratio)
+        return quarot_amd.quantized_linear(x, lin.weight, lin.weight_scales, lin.bias, had.had_rem_dim, had.rem_dim,
+                                           quantizer.input_clip_ratio, force_fp32=had.fp32_had)

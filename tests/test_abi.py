@@ -29,7 +29,7 @@ def test_header_declares_expected_entry_points():
     syms = declared_symbols()
     for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
                  "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
-                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4",
+                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4", "qr_quantized_linear_workspace_bytes", "qr_quantized_linear_f16",
                  "qr_workspace_bytes", "qr_linear_i4_f16_ws"):
         assert must in syms
 
@@ -87,6 +87,26 @@ def test_workspace_query_needs_no_gpu(lib):
     one = ctypes.c_void_p(16)
     assert lib.qr_linear_i4_f16_ws(one, None, one, one, None, 4, 4, 64, one, None, 0, None) == -1
     assert lib.qr_linear_i4_f16_ws(one, one, one, one, None, 4, 4, 100, one, None, 0, None) == -2
+
+
+def test_quantized_linear_workspace_and_argument_errors_need_no_gpu(lib):
+    """The single-call layer entry point: its workspace holds the codes (M K / 2 bytes), the scales
+    (2 M bytes), each rounded up to 16 bytes, and the GEMM's own scratch; argument errors are
+    reported before anything is launched."""
+    assert lib.qr_quantized_linear_workspace_bytes(1, 8192, 28672) == 14336 + 16
+    assert lib.qr_quantized_linear_workspace_bytes(2048, 4096, 11008) == 2048 * 5504 + 4096
+    m, n, k = 256, 4096, 11008
+    assert lib.qr_quantized_linear_workspace_bytes(m, n, k) == m * k // 2 + 512 + lib.qr_workspace_bytes(m, n, k)
+    assert lib.qr_quantized_linear_workspace_bytes(0, n, k) == 0
+    one = ctypes.c_void_p(16)
+    args = (one, 4, 64, 0, None, 0, 1.0, 1.0, one, one, None, 4, one)
+    assert lib.qr_quantized_linear_f16(*args, None, 0, None) == -6                 # no workspace
+    assert lib.qr_quantized_linear_f16(*args, one, 100, None) == -6                # too small (needs 128 + 16)
+    assert lib.qr_quantized_linear_f16(*args, ctypes.c_void_p(24), 4096, None) == -6   # misaligned
+    assert lib.qr_quantized_linear_f16(one, 4, 100, 0, None, 0, 1.0, 1.0, one, one, None, 4, one, one, 4096, None) == -2
+    assert lib.qr_quantized_linear_f16(None, 4, 64, 0, None, 0, 1.0, 1.0, one, one, None, 4, one, one, 4096, None) == -1
+    assert lib.qr_quantized_linear_f16(one, 0, 64, 0, None, 0, 1.0, 1.0, one, one, None, 4, one, None, 0, None) == 0
+    assert b"workspace" in lib.qr_strerror(-6)
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

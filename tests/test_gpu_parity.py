@@ -711,6 +711,49 @@ def test_decode_shapes_bit_exact(m, k, n):
     assert np.array_equal(bits(y[:, cols].cpu().numpy()), bits(want))
 
 
+def test_linear4bit_sequential_is_one_call_with_the_same_results_and_state_dict():
+    """Linear4bitSequential against torch.nn.Sequential of the same modules: identical output bits
+    (the same two kernels run), identical state-dict keys, and the oracle on a small case; chains
+    and inputs it does not recognise run module by module."""
+    rng = np.random.default_rng(77)
+    nn_ = quarot_amd.nn
+
+    def make(k, n, bias, had, clip=1.0, fp32=False):
+        lin = nn_.Linear4bit(k, n, bias=bias).half().cuda()
+        lin.weight.copy_(gpu(rng.integers(0, 256, (n, k // 2), dtype=np.uint8)))
+        lin.weight_scales.copy_(gpu((np.abs(rng.standard_normal((n, 1))) * 0.01 + 0.001).astype(F16)))
+        if bias:
+            lin.bias.copy_(gpu(rng.standard_normal(n).astype(F16)))
+        front = ([nn_.OnlineHadamard(k, force_fp32=fp32).cuda()] if had else []) + [nn_.Quantizer(clip)]
+        return torch.nn.Sequential(*front, lin), nn_.Linear4bitSequential(*front, lin)
+
+    for (m, k, n, bias, had, clip, fp32) in [(37, 11008, 256, True, True, 0.9, False), (1, 28672, 512, False, True, 1.0, False),
+                                             (5, 4096, 512, False, False, 1.0, False), (64, 4096, 128, True, True, 1.0, True),
+                                             (200, 8192, 320, False, False, 0.95, False)]:
+        ref, fused = make(k, n, bias, had, clip, fp32)
+        x = gpu(synth_x(m, k, seed=m + k))
+        assert torch.equal(fused(x), ref(x)), (m, k, n)
+        assert list(fused.state_dict().keys()) == list(ref.state_dict().keys())
+    ref, fused = make(4096, 256, True, False)
+    x3 = gpu(synth_x(6, 4096, seed=1)).view(2, 3, 4096)
+    y3 = fused(x3)
+    assert y3.shape == (2, 3, 256) and torch.equal(y3, ref(x3))
+    lin = fused[1]
+    wq, ws = o.quantizer(x3.view(6, 4096).cpu().numpy())
+    want = o.linear4bit(wq, ws, lin.weight.cpu().numpy(), lin.weight_scales.cpu().numpy().reshape(-1), lin.bias.cpu().numpy())
+    assert np.array_equal(bits(y3.view(6, 256).cpu().numpy()), bits(want))
+    # not one of the two chains, or not a contiguous fp16 tensor: module by module
+    plain = nn_.Linear4bitSequential(nn_.Quantizer())
+    p = plain(x3.view(6, 4096))
+    assert isinstance(p, quarot_amd.PackedQuantizedTensor) and np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    xs = gpu(synth_x(6, 8192, seed=2))[:, ::2]
+    with pytest.raises(RuntimeError):
+        fused(xs)                                            # the reference's modules reject a strided input as well
+    fused2 = nn_.Linear4bitSequential(*list(ref))
+    fused2.load_state_dict(ref.state_dict())
+    assert torch.equal(fused2(x3), y3)
+
+
 def test_runs_on_the_current_stream():
     s = torch.cuda.Stream()
     x = gpu(synth_x(64, 4096, seed=8))
