@@ -48,7 +48,8 @@ const char* qr_strerror(int code);
  * matmul_hadU_cuda (quarot/functional/hadamard.py:92-101) and matmul_had_cuda
  * (quarot/transformers/kv_cache.py:30-33).
  *   x, y    [rows, n] of `dtype` (QR_DTYPE_F16 or QR_DTYPE_F32); y may alias x.
- *   K       1, or the order of hadK; n % K == 0 and n / K a power of two, 8 <= n/K, n <= 32768.
+ *   K       1, or the order of hadK; n % K == 0 and n / K a power of two; n <= 32768, and n <= 128
+ *           when n / K < 8 (e.g. had_40 alone across the 40 attention heads of Llama-2-13B).
  *   hadK    [K, K] row-major of `dtype` (the module's had_rem_dim buffer), ignored when K == 1.
  *           Entries must be exactly representable in fp16 (the reference's tables are +-1).
  *   scale   applied in fp32 after the butterflies (the reference passes 1/sqrt(n)).

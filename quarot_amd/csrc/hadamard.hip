@@ -1396,12 +1396,85 @@ int launch_hadamard_small(const void* x, void* y, int64_t rows, int n, float sca
     return qr_launch_status();
 }
 
+// Rows whose power-of-two factor is 1, 2 or 4 (e.g. OnlineHadamard(40) across the 40 attention heads
+// of Llama-2-13B on a transposed copy: had_40 alone), n <= 128.  A workgroup takes 64 consecutive rows:
+// they are staged in LDS as floats, the m-point butterflies run in place with the scale applied (and,
+// for fp16 I/O, the rounding to fp16 that the reference's two-step form has between its steps,
+// quarot/functional/hadamard.py:99-100), then thread (row, part) forms outputs part, part + 4, ... as
+// dot products of hadK rows (LDS broadcast reads) with the staged row, and the results leave through
+// LDS as one contiguous block.  fp32 accumulation, one rounding at the end.
+template <typename IO>
+__global__ __launch_bounds__(256) void hadamard_tiny_kernel(const IO* __restrict__ x, IO* __restrict__ y, int64_t rows,
+                                                            int n, int K, const IO* __restrict__ hadK, float scale) {
+    constexpr int RW = 64;
+    extern __shared__ float tiny_lds[];
+    const int m = n / K, ld = n + 1;                        // odd row stride in floats: lanes = rows hit distinct banks
+    float* T = tiny_lds;                                    // [RW][ld]
+    float* Y = T + RW * ld;                                 // [RW][ld]
+    float* H = Y + RW * ld;                                 // [K][K]
+    const int tid = threadIdx.x;
+    const int64_t row0 = (int64_t)blockIdx.x * RW;
+    const int live = (int)((rows - row0) < RW ? (rows - row0) : RW);
+    for (int i = tid; i < K * K; i += 256) H[i] = K > 1 ? (float)hadK[i] : 1.0f;
+    const IO* xb = x + row0 * n;
+    for (int i = tid; i < live * n; i += 256) T[(i / n) * ld + i % n] = (float)xb[i];
+    __syncthreads();
+    // m-point Walsh-Hadamard transform of every (row, k) group, scaled
+    for (int u = tid; u < live * K; u += 256) {
+        float* t = T + (u / K) * ld + (u % K) * m;
+        float v[4] = {t[0], m > 1 ? t[1] : 0.f, m > 2 ? t[2] : 0.f, m > 2 ? t[3] : 0.f};
+        if (m > 1) {
+            const float a = v[0] + v[1], b = v[0] - v[1], c = v[2] + v[3], d = v[2] - v[3];
+            v[0] = a; v[1] = b; v[2] = c; v[3] = d;
+        }
+        if (m > 2) {
+            const float a = v[0] + v[2], b = v[1] + v[3], c = v[0] - v[2], d = v[1] - v[3];
+            v[0] = a; v[1] = b; v[2] = c; v[3] = d;
+        }
+        for (int e = 0; e < m; ++e) {
+            const float sv = v[e] * scale;
+            t[e] = sizeof(IO) == 2 ? (float)narrow_f16(sv) : sv;
+        }
+    }
+    __syncthreads();
+    const int r = tid & 63, part = tid >> 6;
+    if (r < live) {
+        const float* t = T + r * ld;
+        for (int j = part; j < n; j += 4) {
+            const int kp = j / m, rr = j - kp * m;
+            const float* h = H + kp * K;
+            float acc = 0.f;
+            for (int k = 0; k < K; ++k) acc = __builtin_fmaf(h[k], t[k * m + rr], acc);
+            Y[r * ld + j] = acc;
+        }
+    }
+    __syncthreads();
+    IO* yb = y + row0 * n;
+    for (int i = tid; i < live * n; i += 256) yb[i] = (IO)Y[(i / n) * ld + i % n];
+}
+
+template <typename IO>
+int launch_hadamard_tiny(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, hipStream_t st) {
+    const size_t lds = ((size_t)2 * 64 * (n + 1) + (size_t)K * K) * sizeof(float);
+    auto kern = hadamard_tiny_kernel<IO>;
+    if (lds > 48 * 1024) {
+        hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    const int64_t grid = (rows + 63) / 64;
+    if (grid > 0x7fffffffLL) return QR_E_SHAPE;
+    kern<<<dim3((unsigned)grid), dim3(256), lds, st>>>((const IO*)x, (IO*)y, rows, n, K, (const IO*)hadK, scale);
+    return qr_launch_status();
+}
+
+bool tiny_applies(int n, int K) { return n / K < 8 && n <= 128; }
+
 int check_shape(int64_t rows, int n, int K) {
     if (rows < 0 || n <= 0 || K <= 0) return QR_E_SHAPE;
     if (n % K != 0) return QR_E_SHAPE;
     const int m = n / K;
     if ((m & (m - 1)) != 0) return QR_E_SHAPE;
-    if (m < 8 || n > 32768 || K > 32 * KS_MAX) return QR_E_UNSUPPORTED;
+    if ((m < 8 && n > 128) || n > 32768 || K > 32 * KS_MAX) return QR_E_UNSUPPORTED;
     return QR_OK;
 }
 
@@ -1415,6 +1488,11 @@ extern "C" int qr_hadamard(const void* x, void* y, int64_t rows, int n, int K, c
     if (!x || !y || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y & 15)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    if (tiny_applies(n, K)) {
+        if (dtype == QR_DTYPE_F16) return launch_hadamard_tiny<f16>(x, y, rows, n, K, hadK, scale, st);
+        if (dtype == QR_DTYPE_F32) return launch_hadamard_tiny<float>(x, y, rows, n, K, hadK, scale, st);
+        return QR_E_DTYPE;
+    }
     // head-dimension rows: the kernel whose arithmetic the K-cache quantiser shares
     if (dtype == QR_DTYPE_F16 && K == 1 && n == 128) return qr_internal_hadamard128_f16(x, y, rows, scale, st);
     if (dtype == QR_DTYPE_F16 && K == 1 && n <= 64) return launch_hadamard_small(x, y, rows, n, scale, st);
@@ -1444,6 +1522,7 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 7)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (tiny_applies(n, K)) return QR_E_UNSUPPORTED;       // rows this short: qr_hadamard, then qr_quantize_rows_f16_i4
     if (K == 1 && pow2_split(n))
         return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, pow2_split(n), nullptr, scale, clip, q, scales, st);
     if (mode == QR_DTYPE_F16 && bm_applies(n, K))

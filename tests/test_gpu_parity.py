@@ -289,7 +289,7 @@ def test_linear4bit_module_from_float_and_state_dict():
 
 # ------------------------------------------------------------------------------ Hadamard
 
-HAD_SIZES = [8, 16, 32, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
+HAD_SIZES = [4, 12, 24, 40, 112, 120, 8, 16, 32, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
 
 
 def close(got, want):
@@ -311,6 +311,27 @@ def test_hadamard_within_tolerance(n, dtype):
     cf = o.hadamard_closed_form(x.astype(np.float64))
     tol = 3e-3 if dtype == F16 else 1e-5
     assert np.all(np.abs(got - cf) <= tol * (1 + np.abs(cf)))
+
+
+def test_hadamard_across_forty_heads():
+    """Llama-2-13B has 40 attention heads: OnlineHadamard(40) is had_40 alone (power-of-two factor 1),
+    applied by the reference to a transposed view.  Row counts that leave a partly filled last block of
+    64, fp16 and fp32, and the module that chains it with the quantiser (separate steps for this head
+    count) against the oracle."""
+    hadk, k = quarot_amd.functional.hadamard.get_hadK(40)
+    assert k == 40
+    for rows in (1, 63, 1000):
+        x = synth_x(rows, 40, seed=rows)
+        y = quarot_amd.functional.matmul_hadU_cuda(gpu(x), hadk.cuda(), k)
+        assert close(y.cpu().numpy(), o.online_hadamard(x))
+        xf = x.astype(F32) * F32(1.003)
+        yf = quarot_amd.functional.matmul_hadU_cuda(gpu(xf), hadk.cuda(), k)
+        assert np.allclose(yf.cpu().numpy(), o.hadamard_closed_form(xf.astype(np.float64)), rtol=1e-5, atol=1e-5)
+    xa = gpu(synth_x(7, 40 * 128, seed=4)).view(7, 40, 128)
+    p = quarot_amd.nn.HeadsHadamardQuantizer(40)(xa)
+    want_y = o.heads_hadamard(xa.cpu().numpy(), 40)
+    wq, _ = o.quantizer(want_y, 1.0)
+    assert p.quantized_x.shape == (7, 20 * 128) and np.mean(p.quantized_x.cpu().numpy() == wq) > 0.99
 
 
 @pytest.mark.parametrize("n", [8, 16, 32, 64])
