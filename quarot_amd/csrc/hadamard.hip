@@ -1415,7 +1415,14 @@ __global__ __launch_bounds__(256) void hadamard_tiny_kernel(const IO* __restrict
     const int tid = threadIdx.x;
     const int64_t row0 = (int64_t)blockIdx.x * RW;
     const int live = (int)((rows - row0) < RW ? (rows - row0) : RW);
-    for (int i = tid; i < K * K; i += 256) H[i] = K > 1 ? (float)hadK[i] : 1.0f;
+    // m == 1: hadK is kept transposed, so that four consecutive outputs read their four coefficients
+    // of one k with a single 16-byte broadcast (K % 4 == 0 for every table of the reference)
+    const bool blocked = m == 1 && (K & 3) == 0;
+    for (int i = tid; i < K * K; i += 256) {
+        const float hv = K > 1 ? (float)hadK[i] : 1.0f;
+        if (blocked) H[(i % K) * K + i / K] = hv;
+        else H[i] = hv;
+    }
     const IO* xb = x + row0 * n;
     for (int i = tid; i < live * n; i += 256) T[(i / n) * ld + i % n] = (float)xb[i];
     __syncthreads();
@@ -1438,7 +1445,20 @@ __global__ __launch_bounds__(256) void hadamard_tiny_kernel(const IO* __restrict
     }
     __syncthreads();
     const int r = tid & 63, part = tid >> 6;
-    if (r < live) {
+    if (r < live && blocked) {
+        const float* t = T + r * ld;
+        for (int j0 = part * 4; j0 < n; j0 += 16) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < K; ++k) {
+                const f32x4 h4 = *(const f32x4*)(H + k * K + j0);
+                const float tv = t[k];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(h4[e], tv, acc[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Y[r * ld + j0 + e] = acc[e];
+        }
+    } else if (r < live) {
         const float* t = T + r * ld;
         for (int j = part; j < n; j += 4) {
             const int kp = j / m, rr = j - kp * m;
