@@ -115,12 +115,17 @@ int qr_rmsnorm_quantize_f16_i4(const void* x, int64_t rows, int64_t cols, int me
  *   y[r, g, d] = fp16( (1 / sqrt(heads)) * sum_h Had[g, h] * x[r, h, d] ), Had the Sylvester matrix of
  *   size heads, summed in fp32 and rounded to fp16 once; q and scales as qr_quantize_rows_f16_i4(y)
  *   over the whole row.  No transposed copies are made.
- *   head_dim == 128 and heads in {16, 32, 64} (else QR_E_UNSUPPORTED: use qr_hadamard on a transposed
- *   copy and qr_quantize_rows_f16_i4); y_or_null: optional fp16 copy of the transformed rows.
- *   x and y 16-byte aligned, q 4-byte aligned.
+ *   head_dim == 128 and heads in {16, 32, 64}, hadK_or_null ignored; or heads the order of one of
+ *   the reference's tables (12, 20, 28, 36, 40, 52, 60: Llama-2-13B has 40 heads, Llama-30B 52) with
+ *   hadK_or_null = that table, fp16 [heads, heads] (the module's had_rem_dim buffer): OnlineHadamard
+ *   is then hadK alone and y[r, g, d] = fp16( sum_h hadK[g, h] * fp16(x[r, h, d] / sqrt(heads)) ), the
+ *   reference's two-step rounding (quarot/functional/hadamard.py:99-100).  Anything else returns
+ *   QR_E_UNSUPPORTED (use qr_hadamard on a transposed copy and qr_quantize_rows_f16_i4).
+ *   y_or_null: optional fp16 copy of the transformed rows.  x and y 16-byte aligned, q 4-byte aligned.
  */
-int qr_heads_hadamard_quantize_f16_i4(const void* x, int64_t rows, int heads, int head_dim, float clip,
-                                      void* q, void* scales, void* y_or_null, void* stream);
+int qr_heads_hadamard_quantize_f16_i4(const void* x, int64_t rows, int heads, int head_dim,
+                                      const void* hadK_or_null, float clip, void* q, void* scales,
+                                      void* y_or_null, void* stream);
 
 /*
  * int4 x int4 -> int32 GEMM:  C[M, N] = unpack(A)[M, K] . unpack(B)[N, K]^T.

@@ -188,23 +188,30 @@ def rmsnorm_quantize(x, mean_dim, eps=1e-5, clip_ratio=1.0, return_normalized=Fa
     return (packed, y.view(x.shape)) if return_normalized else packed
 
 
-def heads_hadamard_quantize(x, num_heads, clip_ratio=1.0, return_transformed=False):
+def heads_hadamard_quantize(x, num_heads, clip_ratio=1.0, return_transformed=False, hadK=None):
     """The chain in front of o_proj in one kernel (e2e/quantized_llama/modeling_llama.py:108-110):
     OnlineHadamard(num_heads) over the head axis of attention's output, then Quantizer.forward on the
     rows reshaped to [..., hidden].  x is [..., num_heads, head_dim], contiguous, as attention writes
-    it; no transposed copies are made.  head_dim 128 and 16, 32 or 64 heads."""
+    it; no transposed copies are made.  head_dim 128 and 16, 32 or 64 heads; or a head count that is
+    the order of one of the reference's tables (40 for Llama-2-13B, 52 for Llama-30B, ...) with hadK =
+    that table (OnlineHadamard's had_rem_dim buffer)."""
     assert x.dtype == torch.float16
     if x.dim() < 2 or x.shape[-2] != num_heads:
         raise RuntimeError("heads_hadamard_quantize: x must be [..., num_heads, head_dim]")
     x2, lead = _flat2d(x.view(*x.shape[:-2], x.shape[-2] * x.shape[-1]))
-    dev = _require_gpu_contiguous("heads_hadamard_quantize", x=x2)
+    if hadK is not None:
+        if hadK.shape != (num_heads, num_heads):
+            raise RuntimeError("heads_hadamard_quantize: hadK must be [num_heads, num_heads]")
+        if hadK.dtype != torch.float16 or hadK.device != x2.device:     # (a module left on the CPU: as matmul_hadU_cuda does)
+            hadK = hadK.to(device=x2.device, dtype=torch.float16)
+    dev = _require_gpu_contiguous("heads_hadamard_quantize", x=x2, hadK=hadK)
     rows, cols = x2.shape
     q = torch.empty((rows, cols // 2), dtype=torch.uint8, device=dev)
     s = torch.empty((rows,), dtype=torch.float16, device=dev)
     y = torch.empty_like(x2) if return_transformed else None
     with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_heads_hadamard_quantize_f16_i4(_ptr(x2), rows, int(num_heads), cols // int(num_heads),
-                                                                float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
+                                                                _ptr(hadK), float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
                                                                 _lib.stream_ptr(dev)))
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))

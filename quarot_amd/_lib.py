@@ -20,7 +20,7 @@ SIGNATURES = {
     "qr_quantize_rows_f16_i4": (_int, (_ptr, _f32, _i64, _i64, _ptr, _ptr, _ptr)),
     "qr_hadamard_quantize_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _int, _f32, _f32, _ptr, _ptr, _ptr, _ptr)),
     "qr_rmsnorm_quantize_f16_i4": (_int, (_ptr, _i64, _i64, _int, _f32, _f32, _ptr, _ptr, _ptr, _ptr)),
-    "qr_heads_hadamard_quantize_f16_i4": (_int, (_ptr, _i64, _int, _int, _f32, _ptr, _ptr, _ptr, _ptr)),
+    "qr_heads_hadamard_quantize_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _f32, _ptr, _ptr, _ptr, _ptr)),
     "qr_matmul_i4_i32": (_int, (_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
     "qr_sym_dequant_i32_f16": (_int, (_ptr, _ptr, _ptr, _i64, _i64, _ptr, _ptr)),
     "qr_linear_i4_f16": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),

@@ -51,9 +51,9 @@ class HeadsHadamardQuantizer(torch.nn.Module):
     kernel: OnlineHadamard(num_heads) over the head axis of attention's output [..., heads, head_dim]
     (the reference applies it to a transposed view and transposes back), the reshape to
     [..., hidden], and o_proj's Quantizer(input_clip_ratio).  Neither the transposed copies nor the
-    transformed fp16 tensor go through HBM.  Shapes the fused kernel does not take (head_dim other
-    than 128, a head count other than 16, 32 or 64, a dtype other than fp16, a strided input) run as
-    the separate steps."""
+    transformed fp16 tensor go through HBM.  Shapes the fused kernels do not take (head_dim other
+    than 128, a head count that is neither 16, 32, 64 nor the order of one of the reference's tables
+    up to 60, a dtype other than fp16, a strided input) run as the separate steps."""
 
     def __init__(self, num_heads, input_clip_ratio=1.0):
         super().__init__()
@@ -63,9 +63,12 @@ class HeadsHadamardQuantizer(torch.nn.Module):
 
     def forward(self, x):
         assert x.shape[-2] == self.num_heads
-        if (x.dtype == torch.float16 and x.shape[-1] == 128 and self.num_heads in (16, 32, 64)
-                and x.is_contiguous()):
-            return quarot_amd.heads_hadamard_quantize(x, self.num_heads, self.input_clip_ratio)
+        if x.dtype == torch.float16 and x.shape[-1] == 128 and x.is_contiguous() and x.is_cuda:
+            if self.num_heads in (16, 32, 64):
+                return quarot_amd.heads_hadamard_quantize(x, self.num_heads, self.input_clip_ratio)
+            if self.had.rem_dim == self.num_heads and self.num_heads <= 64:      # hadK alone (40, 52, ... heads)
+                return quarot_amd.heads_hadamard_quantize(x, self.num_heads, self.input_clip_ratio,
+                                                          hadK=self.had.had_rem_dim)
         y = self.had(x.transpose(-1, -2)).transpose(-1, -2)
         y = y.reshape(*x.shape[:-2], x.shape[-2] * x.shape[-1]).contiguous()
         return quarot_amd.PackedQuantizedTensor(*quarot_amd.quantize_rows(y, self.input_clip_ratio))

@@ -327,11 +327,27 @@ def test_hadamard_across_forty_heads():
         xf = x.astype(F32) * F32(1.003)
         yf = quarot_amd.functional.matmul_hadU_cuda(gpu(xf), hadk.cuda(), k)
         assert np.allclose(yf.cpu().numpy(), o.hadamard_closed_form(xf.astype(np.float64)), rtol=1e-5, atol=1e-5)
-    xa = gpu(synth_x(7, 40 * 128, seed=4)).view(7, 40, 128)
-    p = quarot_amd.nn.HeadsHadamardQuantizer(40)(xa)
-    want_y = o.heads_hadamard(xa.cpu().numpy(), 40)
-    wq, _ = o.quantizer(want_y, 1.0)
-    assert p.quantized_x.shape == (7, 20 * 128) and np.mean(p.quantized_x.cpu().numpy() == wq) > 0.99
+    # the module for 40 and 52 heads (Llama-2-13B, Llama-30B): one kernel with the table as a matrix;
+    # its own fp16 rows within tolerance of the oracle, codes and scales bit-exact on those rows
+    for heads, rows in ((40, 7), (52, 70), (12, 3)):
+        xa = gpu(synth_x(rows, heads * 128, seed=heads)).view(rows, heads, 128)
+        mod = quarot_amd.nn.HeadsHadamardQuantizer(heads, input_clip_ratio=0.95).cuda()
+        p = mod(xa)
+        p2, y = quarot_amd.heads_hadamard_quantize(xa, heads, 0.95, return_transformed=True, hadK=mod.had.had_rem_dim)
+        assert torch.equal(p.quantized_x, p2.quantized_x) and torch.equal(p.scales_x, p2.scales_x)
+        yk = y.cpu().numpy()
+        want_y = o.heads_hadamard(xa.cpu().numpy(), heads)
+        assert close(yk, want_y) and np.mean(yk == want_y) > 0.99
+        wq, ws = o.quantizer(yk, 0.95)
+        assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+        assert np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+        staged = mod.had(xa.transpose(-1, -2)).transpose(-1, -2).reshape(rows, heads * 128).contiguous()
+        assert close(staged.cpu().numpy(), want_y)
+    # 24 heads = had_12 (x) H_2: neither form of the fused kernel, the module runs the separate steps
+    xb = gpu(synth_x(5, 24 * 128, seed=6)).view(5, 24, 128)
+    pb = quarot_amd.nn.HeadsHadamardQuantizer(24).cuda()(xb)
+    wq, _ = o.quantizer(o.heads_hadamard(xb.cpu().numpy(), 24), 1.0)
+    assert pb.quantized_x.shape == (5, 12 * 128) and np.mean(pb.quantized_x.cpu().numpy() == wq) > 0.99
 
 
 @pytest.mark.parametrize("n", [8, 16, 32, 64])
@@ -485,11 +501,11 @@ def test_fused_heads_hadamard_quantize_full_size_fallback_and_errors():
     q = torch.empty(8, 2048, dtype=torch.uint8, device=x.device)
     s = torch.empty(8, dtype=torch.float16, device=x.device)
     st = torch.cuda.current_stream().cuda_stream
-    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 8, 64, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
-    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 40, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
-    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr() + 2, 8, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) == -4
-    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 0, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) == 0
-    assert L.qr_heads_hadamard_quantize_f16_i4(None, 8, 32, 128, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 8, 64, None, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 8, 40, 128, None, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr() + 2, 8, 32, 128, None, 1.0, q.data_ptr(), s.data_ptr(), None, st) == -4
+    assert L.qr_heads_hadamard_quantize_f16_i4(xf.data_ptr(), 0, 32, 128, None, 1.0, q.data_ptr(), s.data_ptr(), None, st) == 0
+    assert L.qr_heads_hadamard_quantize_f16_i4(None, 8, 32, 128, None, 1.0, q.data_ptr(), s.data_ptr(), None, st) < 0
     with pytest.raises(RuntimeError):
         quarot_amd.heads_hadamard_quantize(xf, 32)
 
