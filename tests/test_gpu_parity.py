@@ -475,6 +475,26 @@ def test_fused_heads_hadamard_quantize(heads, rows, clip):
     assert float((p.quantized_x == staged.quantized_x).float().mean()) > 0.99
 
 
+@pytest.mark.parametrize("heads", [32, 64, 40])
+def test_fused_heads_hadamard_quantize_infinite_nan_zero_huge_and_tiny_rows(heads):
+    """Rows holding an infinity, a NaN, only zeros, a value near the fp16 maximum, and values near the
+    subnormal range: codes and scales of both kernel forms must still equal the oracle quantiser applied
+    to the kernel's own transformed rows, bit for bit (the quantiser's slow paths)."""
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((6, heads, 128)).astype(F16)
+    x[1, 3, 5] = np.inf
+    x[2, 0, 0] = np.nan
+    x[3] = 0
+    x[4, 7, 9] = 60000.0
+    x[5] *= F16(1e-4)
+    mod = quarot_amd.nn.HeadsHadamardQuantizer(heads).cuda()
+    p, y = quarot_amd.heads_hadamard_quantize(gpu(x), heads, 1.0, return_transformed=True, hadK=mod.had.had_rem_dim)
+    with np.errstate(all="ignore"):
+        wq, ws = o.quantizer(y.cpu().numpy(), 1.0)
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    assert np.array_equal(bits(p.scales_x.cpu().numpy().reshape(-1)), bits(ws))
+
+
 def test_fused_heads_hadamard_quantize_full_size_fallback_and_errors():
     """Prefill-size input ([2, 1024, 32, 128]) checked on strided rows and through norm preservation;
     shapes the fused kernel does not take go through the separate steps; argument errors of the C
