@@ -152,19 +152,23 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
                 v[2 * i + 1] = (float)f16_from_bits((unsigned short)(hp[i] >> 16));
             }
             float mn = v[0], mx = v[0];
+            float nan_seen = amax > 0x7c00u ? 1.0f : 0.0f;       // magnitude bits above infinity's: a NaN in this lane
 #pragma unroll
             for (int e = 1; e < 8; ++e) {
                 mn = v[e] < mn ? v[e] : mn;
                 mx = v[e] > mx ? v[e] : mx;
             }
-            if (LG > 0) kv_minmax<1>(mn, mx);
-            if (LG > 1) kv_minmax<2>(mn, mx);
-            if (LG > 2) kv_minmax<4>(mn, mx);
-            if (LG > 3) kv_minmax<8>(mn, mx);
-            if (LG > 4) kv_minmax<16>(mn, mx);
+            float nan_lo = 0.0f;                                 // (unused minimum of the flag; the maximum is the "any")
+            if (LG > 0) { kv_minmax<1>(mn, mx); kv_minmax<1>(nan_lo, nan_seen); }
+            if (LG > 1) { kv_minmax<2>(mn, mx); kv_minmax<2>(nan_lo, nan_seen); }
+            if (LG > 2) { kv_minmax<4>(mn, mx); kv_minmax<4>(nan_lo, nan_seen); }
+            if (LG > 3) { kv_minmax<8>(mn, mx); kv_minmax<8>(nan_lo, nan_seen); }
+            if (LG > 4) { kv_minmax<16>(mn, mx); kv_minmax<16>(nan_lo, nan_seen); }
+            // torch.amax / amin propagate a NaN: range, scale and zero of that vector are NaN, every code 0
+            if (nan_seen != 0.0f) mn = mx = __builtin_nanf("");
             f16 rng = (f16)(mx - mn);
             const f16 floor_ = (f16)1e-5f;
-            rng = rng < floor_ ? floor_ : rng;
+            rng = rng < floor_ ? floor_ : rng;                   // NaN < x is false: NaN stays
             sc = (f16)(float)((double)(float)rng / 15.0);
             zp = (f16)(-mn);
             const float s = (float)sc, z = (float)zp;

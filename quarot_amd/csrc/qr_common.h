@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <mutex>
+#include <vector>
 #include <stdint.h>
 #include "../../include/quarot_hip.h"
 
@@ -28,17 +29,21 @@ static inline hipError_t qr_allow_dynamic_lds(const void* kernel, size_t bytes) 
         int dev;
         size_t bytes;
     };
-    static Entry table[64];
-    static int used = 0;
+    static std::vector<Entry> table;            // grows with the kernel instantiations in use (never shrinks)
     static std::mutex guard;                    // entry points may be called from several host threads
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     std::lock_guard<std::mutex> lock(guard);
-    for (int i = 0; i < used; ++i)
-        if (table[i].fn == kernel && table[i].dev == dev && table[i].bytes >= bytes) return hipSuccess;
+    for (Entry& t : table)
+        if (t.fn == kernel && t.dev == dev) {
+            if (t.bytes >= bytes) return hipSuccess;
+            e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+            if (e == hipSuccess) t.bytes = bytes;
+            return e;
+        }
     e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e == hipSuccess && used < 64) table[used++] = Entry{kernel, dev, bytes};
+    if (e == hipSuccess) table.push_back(Entry{kernel, dev, bytes});
     return e;
 }
 
@@ -51,18 +56,16 @@ static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) 
         size_t lds;
         int blocks;
     };
-    static Entry table[64];
-    static int used = 0;
+    static std::vector<Entry> table;
     static std::mutex guard;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 1;
     std::lock_guard<std::mutex> lock(guard);
-    for (int i = 0; i < used; ++i)
-        if (table[i].fn == kernel && table[i].dev == dev && table[i].threads == threads && table[i].lds == lds)
-            return table[i].blocks;
+    for (const Entry& t : table)
+        if (t.fn == kernel && t.dev == dev && t.threads == threads && t.lds == lds) return t.blocks;
     int blocks = 1;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, threads, lds) != hipSuccess || blocks < 1) blocks = 1;
-    if (used < 64) table[used++] = Entry{kernel, dev, threads, lds, blocks};
+    table.push_back(Entry{kernel, dev, threads, lds, blocks});
     return blocks;
 }
 

@@ -289,7 +289,7 @@ def test_linear4bit_module_from_float_and_state_dict():
 
 # ------------------------------------------------------------------------------ Hadamard
 
-HAD_SIZES = [4, 12, 24, 40, 112, 120, 8, 16, 32, 64, 128, 512, 1024, 2048, 4096, 8192, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
+HAD_SIZES = [4, 12, 24, 40, 112, 120, 8, 16, 32, 64, 128, 512, 1024, 2048, 4096, 8192, 16384, 32768, 96, 224, 320, 1376, 2304, 3840, 5120, 6912, 8960, 9984, 11008, 13824, 14336, 28672]
 
 
 def close(got, want):
@@ -369,7 +369,7 @@ def test_hadamard_short_rows_many_per_workgroup(n):
         assert bool((err <= 2e-3 * x.float().abs().amax(dim=1) + 1e-3).all())
 
 
-@pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 224, 3840, 6912, 8960, 11008, 28672, 13824])
+@pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 16384, 224, 3840, 6912, 8960, 11008, 28672, 13824, 5120])
 @pytest.mark.parametrize("fp32", [False, True])
 def test_fused_hadamard_quantize_equals_staged(n, fp32):
     """Codes of the fused kernel are judged on the kernel's OWN fp16 Hadamard output (returned on
@@ -605,6 +605,28 @@ def test_kv_vectors_with_infinities_take_the_ieee_path():
     keep = [i for i in range(64) if i not in (5, 9)]
     wq, ws, wz = o.kv_asym_quant(x[keep])
     assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
+
+
+@pytest.mark.parametrize("dim,hadamard", [(128, False), (64, False), (64, True), (16, False), (256, True), (128, True)])
+def test_kv_vector_with_nan_gets_nan_scale_and_zero(dim, hadamard):
+    """torch.amax / torch.amin propagate a NaN (kv_cache.py:13-14): the vector's scale and zero are NaN
+    and its codes 0 (NaN converts to 0), wherever in the vector the NaN sits; the other vectors of the
+    same wave keep the oracle's codes."""
+    rng = np.random.default_rng(dim)
+    x = rng.standard_normal((70, dim)).astype(F16)
+    where = {3: 0, 20: dim - 1, 41: dim // 2 + 1, 69: 9}
+    for vec, el in where.items():
+        x[vec, el] = np.nan
+    x[50, 2] = np.inf                                              # an infinity next to them still takes the IEEE path
+    q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=hadamard)
+    q, s, z = q.cpu().numpy(), s.cpu().numpy(), z.cpu().numpy()
+    for vec in where:
+        assert np.isnan(s[vec, 0]) and np.isnan(z[vec, 0]) and not q[vec].any(), vec
+    keep = [i for i in range(70) if i not in where and i != 50]
+    xin = kv.matmul_had_cuda(gpu(x), torch.float16).cpu().numpy() if hadamard else x
+    wq, ws, wz = o.kv_asym_quant(xin[keep])
+    assert np.array_equal(q[keep], wq) and np.array_equal(bits(s[keep]), bits(ws)) and np.array_equal(bits(z[keep]), bits(wz))
+    assert np.isposinf(s[50, 0])
 
 
 def test_empty_and_leading_dimensions_through_the_python_interface():
