@@ -32,6 +32,7 @@ extern "C" {
 #define QR_E_ALIGN      -4   /* a pointer is not aligned as the entry point requires */
 #define QR_E_DTYPE      -5   /* unknown dtype / mode code */
 #define QR_E_WORKSPACE  -6   /* the workspace is NULL, misaligned or smaller than the entry point needs */
+#define QR_E_SCRATCH_LIMIT -7 /* the shape needs more scratch than the library's built-in buffer holds */
 
 #define QR_DTYPE_F16 0
 #define QR_DTYPE_F32 1
@@ -170,6 +171,26 @@ size_t qr_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void* sW,
                         const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y,
                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * qr_linear_i4_f16_ws without a workspace argument and without any allocation.  It has NO counterpart
+ * in the reference (whose bindings allocate with torch::empty on every call); it exists for callers
+ * that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The K-split slabs live in a buffer of QR_STATIC_SCRATCH_BYTES that is part
+ * of the library's device image (one copy per GPU, held until the process ends); the call itself
+ * performs no hipMalloc / hipFree and no allocating library call.
+ *   Same operands and bit-identical results as qr_linear_i4_f16_ws with a sufficient workspace.
+ *   A shape whose qr_workspace_bytes(M, N, K) exceeds QR_STATIC_SCRATCH_BYTES returns
+ *   QR_E_SCRATCH_LIMIT and launches nothing (use qr_linear_i4_f16 or the _ws form); shapes that need
+ *   no scratch run the single-launch kernels.
+ *   All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
+ *   streams or host threads) race.  The first call on a device looks the buffer's address up
+ *   (hipGetSymbolAddress); make that call outside graph capture.
+ */
+#define QR_STATIC_SCRATCH_BYTES (32u << 20)
+int qr_linear_i4_f16_static(const void* A, const void* sA, const void* W, const void* sW,
+                            const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y,
+                            void* stream);
 
 /*
  * A whole quantised linear layer in one host call: the module chain

@@ -29,6 +29,7 @@ SIGNATURES = {
     "qr_quantized_linear_f16": (_int, (_ptr, _i64, _i64, _int, _ptr, _int, _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _ptr,
                                        _c.c_size_t, _ptr)),
     "qr_linear_i4_f16_ws": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _c.c_size_t, _ptr)),
+    "qr_linear_i4_f16_static": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
     "qr_kv_quant_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _ptr, _ptr, _ptr)),
     "qr_kv_dequant_i4_f16": (_int, (_ptr, _ptr, _ptr, _i64, _int, _ptr, _ptr)),
 }

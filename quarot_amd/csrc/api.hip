@@ -13,6 +13,7 @@ extern "C" const char* qr_strerror(int code) {
         case QR_E_ALIGN: return "pointer not aligned as required";
         case QR_E_DTYPE: return "unknown dtype or mode code";
         case QR_E_WORKSPACE: return "workspace missing, misaligned or too small";
+        case QR_E_SCRATCH_LIMIT: return "the shape needs more scratch than the library's built-in buffer (QR_STATIC_SCRATCH_BYTES) holds";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

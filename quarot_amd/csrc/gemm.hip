@@ -2000,6 +2000,50 @@ extern "C" size_t qr_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return split > 1 ? (size_t)split * (size_t)M * (size_t)N * 4 : 0;
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------------
+// Slabs of int32 partial sums for the K split, held by the library itself: one array per GPU, alive
+// until the process ends.  Host code must never hand the array's NAME to a kernel (in host code it is a
+// stand-in, not a device address): the per-device address comes from hipGetSymbolAddress, once per
+// device, and only that pointer is used afterwards.
+static __device__ __align__(256) unsigned char scratch[QR_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* scratch_ptr[kMaxDevices];                 // per device: its own copy of `scratch`, at its own address
+std::mutex scratch_guard;
+
+// Address of `scratch` on the current device (looked up on the first call on that device).
+int static_scratch(void** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return QR_E_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(scratch_guard);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return QR_OK;
+}
+}  // namespace
+
+extern "C" int qr_linear_i4_f16_static(const void* A, const void* sA, const void* W, const void* sW,
+                                       const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y, void* stream) {
+    if (M > 0 && N > 0 && (!y || !sA || !sW)) return QR_E_NULL;
+    const size_t need = qr_workspace_bytes(M, N, K);
+    if (need > (size_t)QR_STATIC_SCRATCH_BYTES) return QR_E_SCRATCH_LIMIT;
+    void* ws = nullptr;
+    if (need) {                                  // every slab cell is written before it is read: nothing to clear
+        const int rc = static_scratch(&ws);
+        if (rc != QR_OK) return rc;
+    }
+    return gemm_dispatch(A, W, M, N, K, nullptr, y, sA, sW, bias_or_null, (hipStream_t)stream, ws, need);
+}
+
 extern "C" int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void* sW,
                                    const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y, void* workspace,
                                    size_t workspace_bytes, void* stream) {

@@ -30,7 +30,7 @@ def test_header_declares_expected_entry_points():
     for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
                  "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
                  "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4", "qr_quantized_linear_workspace_bytes", "qr_quantized_linear_f16",
-                 "qr_workspace_bytes", "qr_linear_i4_f16_ws"):
+                 "qr_workspace_bytes", "qr_linear_i4_f16_ws", "qr_linear_i4_f16_static"):
         assert must in syms
 
 
@@ -44,7 +44,7 @@ def test_library_exports_every_declared_symbol(lib):
 def test_version_and_error_text(lib):
     assert lib.qr_version() >= 100
     assert lib.qr_strerror(0) == b"success"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert len(lib.qr_strerror(code)) > 5
     assert b"unknown" in lib.qr_strerror(-99)
 
@@ -72,6 +72,10 @@ def test_argument_errors_are_returned_before_any_launch(lib):
     assert lib.qr_kv_quant_f16_i4(one, 4, 100, 0, one, one, one, None) == -3
     assert lib.qr_kv_quant_f16_i4(one, 4, 128, 3, one, one, one, None) == -5
     assert lib.qr_kv_dequant_i4_f16(one, one, one, 0, 128, one, None) == 0
+    # the entry point with the built-in scratch buffer: a shape beyond the buffer is refused by size alone
+    assert lib.qr_workspace_bytes(768, 3072, 65536) > (32 << 20)
+    assert lib.qr_linear_i4_f16_static(one, one, one, one, None, 768, 3072, 65536, one, None) == -7
+    assert lib.qr_linear_i4_f16_static(one, one, one, one, None, 128, 4096, 100, one, None) == -2
 
 
 def test_workspace_query_needs_no_gpu(lib):
