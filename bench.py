@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--workload c2]
+                    [--no-cpu-baseline] [--no-per-config] [--graph]
 
 A step is one pass of  OnlineHadamard -> Quantizer -> Linear4bit  (Hadamard + per-token int4
 quantise + int4 GEMM + fp16 dequant) over one batch of seeded synthetic tokens already resident in
@@ -12,21 +13,31 @@ outlier channels that motivate the Hadamard):
     c1o o_proj 7B      attention output [2048, 32, 128] -> Hadamard across the 32 heads -> Quantizer
         (one fused kernel) -> W int4 [4096, 4096]
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
-    c3d down_proj 7B, prefill 16 x 2048 tokens  X [32768, 11008]
     c3  the four linears of a 7B decoder layer at 32768 tokens as ONE step: fused qkv 4096->12288, o 4096->4096,
         gate_up 4096->22016 (Quantizer in front of each) and down 11008->4096 (Hadamard+Quantizer): 13.26 TOP
-        (c3a, c3b, c3c: the first three on their own)
-    c4  down_proj 70B decode  X [64, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28
-        (c4m1, c4m8: 1 / 8 tokens; c4g1, c4g8, c4g64: gate_up W int4 [57344, 8192])
+        (c3a, c3b, c3c, c3d: each of them on its own)
+    c4mT  down_proj 70B decode  X [T, 28672]  W int4 [8192, 28672]  Hadamard FWHT(1024) (x) had_28, T in 1, 8, 32, 64
+    c4gT  gate_up 70B decode    X [T, 8192]   W int4 [57344, 8192]
     c5  KV-cache write path of one layer: K and V [32, 4096, 8, 128] fp16 -> asymmetric int4 per head
-        vector (K through the head-dimension Hadamard first); metric GB/s of algorithmic bytes
+        vector (K through the head-dimension Hadamard first) -> fp16 again; metric GB/s of algorithmic bytes
+    b13v, b70v, b13d, b70d  the other sizes of the reference's benchmarks/qlinear_benchmark.py:8-18 at 2048 tokens
+        (5120->5120, 8192->8192 with the Hadamard in front; down_proj 13824->5120 and 28672->8192 with it)
 Decode workloads (M <= 64) rotate among several copies of the weights so that they are streamed from
 HBM rather than from the 256 MB last-level cache.
-Prints ONE JSON line on stdout (metric = TOPS of the whole step, 2.M.N.K / t).
+
+Timing follows benchmarks/qlinear_benchmark.py:20-40,88-113: warm-up, then a loop of K steps between two
+synchronisations, repeated R times; the step time is the median of the R loops and the spread is
+reported as mean +- 1.96 sigma.  Nothing but the step's own launches is inside a timed loop; the time
+of each kernel comes from a separate pass: back-to-back launches of that kernel alone, captured in a
+HIP graph so that the host's per-call cost does not show, timed with HIP events on the launch stream.
+
+Prints ONE JSON line on stdout.  The default run measures the headline workload (c2) and, in
+`per_config`, every other benchmark configuration with fewer repeats.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -38,93 +49,325 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 WORKLOADS = {
-    #        M      K      N     hadamard
-    "c1": (2048, 4096, 4096, False),
-    "c1n": (2048, 4096, 4096, False),       # input_layernorm -> Quantizer -> q_proj
-    "c1o": (2048, 4096, 4096, False),       # attention output -> Hadamard over heads -> Quantizer -> o_proj
-    "c2": (2048, 11008, 4096, True),
-    "c3d": (32768, 11008, 4096, True),
-    "c3a": (32768, 4096, 12288, False),     # fused qkv
-    "c3b": (32768, 4096, 4096, False),      # o_proj
-    "c3c": (32768, 4096, 22016, False),     # gate_up
-    "c3": (0, 0, 0, False),                 # the whole layer set (separate code path below)
-    "c4m32": (32, 28672, 8192, True),
-    "c4g32": (32, 8192, 57344, False),
-    "c4": (64, 28672, 8192, True),          # decode, 70B down_proj
-    "c4m1": (1, 28672, 8192, True),
-    "c4m8": (8, 28672, 8192, True),
-    "c4g1": (1, 8192, 57344, False),        # decode, 70B gate_up (input already quantised upstream: no Hadamard)
-    "c4g8": (8, 8192, 57344, False),
-    "c4g64": (64, 8192, 57344, False),
-    "c5": (0, 0, 0, False),                 # KV-cache quantisation (separate code path below)
+    #        M      K      N     front
+    "c1": (2048, 4096, 4096, "quant"),
+    "c1n": (2048, 4096, 4096, "rmsnorm"),     # input_layernorm -> Quantizer -> q_proj
+    "c1o": (2048, 4096, 4096, "heads"),       # attention output -> Hadamard over heads -> Quantizer -> o_proj
+    "c2": (2048, 11008, 4096, "had"),
+    "c3a": (32768, 4096, 12288, "quant"),     # fused qkv
+    "c3b": (32768, 4096, 4096, "quant"),      # o_proj
+    "c3c": (32768, 4096, 22016, "quant"),     # gate_up
+    "c3d": (32768, 11008, 4096, "had"),       # down_proj
+    "c3": None,                               # the whole layer set as one step
+    "c5": None,                               # KV-cache quantisation
+    "b13v": (2048, 5120, 5120, "had"),        # qlinear_benchmark.py model_sizes / mlp_sizes at 13B and 70B
+    "b70v": (2048, 8192, 8192, "had"),
+    "b13d": (2048, 13824, 5120, "had"),
+    "b70d": (2048, 28672, 8192, "had"),
 }
+for _t in (1, 8, 32, 64):
+    WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
+    WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
+PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 HBM_PEAK_GBS = 8000.0
 
-# HBM-side traffic of the GEMM kernel per launch, from two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch, averaged over the run's dispatches of that kernel).
-# The same counters read 131083.8 KiB / 262144.0 KiB for a plain 256 MiB device copy
-# (--copy-calibration: 262144 KiB read and written), so reads are scaled by 2.0 and writes by 1.0.
-FETCH_SCALE, WRITE_SCALE = 262144.0 / 131083.8, 262144.0 / 262144.0
-TRAFFIC_KIB = {
-    #        FETCH_SIZE   WRITE_SIZE
-    "c1": (16551.0, 16384.0),
-    "c1o": (16590.5, 16384.0),
-    "c2": (44210.0, 16384.0),
-    "c3d": (528791.7, 262144.0),
-    "c4": (62375.6, 1024.0),
-    "c4m1": (57494.0, 16.0),
-    "c4g64": (124423.7, 7168.0),
-    "c5": (131145.3, 69774.2),              # kv_had128_kernel (K cache), per launch
+# Profile summaries that hold the FETCH_SIZE / WRITE_SIZE readings of a workload's dominant kernel
+# ("traffic_kib: kernel=<substring> fetch=<KiB per dispatch> write=<KiB per dispatch>") and the copy
+# calibration ("traffic_scale: fetch=<factor> write=<factor>").
+PROFILE_OF = {
+    "c1": "gemm_spk_c1_q_proj_7b.txt", "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt",
+    "c2": "gemm_spk_and_hadamard_m64_c2_down_proj_7b.txt", "c3d": "gemm_sp256_c3d_prefill_16x2048.txt",
+    "c4m64": "decode_i4_c4_decode_64_tokens_70b_down_proj.txt", "c4m1": "gemv_i4_c4m1_decode_70b_down_proj.txt",
+    "c4g64": "gemm_ks_64x256_c4g64_decode_64_tokens_70b_gate_up.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
 }
 
 
-def synth_x(m, k, seed=0, outliers=True):
-    g = torch.Generator().manual_seed(seed)
-    x = torch.randn(m, k, generator=g)
+def traffic_from_profile(workload, kernel):
+    """(bytes per launch, source file) from the committed rocprofv3 summary of this workload, scaled by
+    the copy calibration; (None, None) when no summary carries the readings."""
+    pdir = os.path.join(ROOT, "profiles")
+    name = PROFILE_OF.get(workload)
+    try:
+        text = open(os.path.join(pdir, name)).read() if name else ""
+        cal = open(os.path.join(pdir, "copy_calibration_256MiB.txt")).read()
+    except OSError:
+        return None, None
+    sc = re.search(r"traffic_scale:\s*fetch=([\d.]+)\s+write=([\d.]+)", cal)
+    if not sc:
+        return None, None
+    for m in re.finditer(r"traffic_kib:\s*kernel=(\S+)\s+fetch=([\d.]+)\s+write=([\d.]+)", text):
+        if m.group(1) in kernel:
+            kib = float(m.group(2)) * float(sc.group(1)) + float(m.group(3)) * float(sc.group(2))
+            return round(kib * 1024), f"profiles/{name}"
+    return None, None
+
+
+def synth_x(m, k, seed=0, outliers=True, device="cpu"):
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn(m, k, generator=g, device=device)
     if outliers:
-        idx = torch.randperm(k, generator=g)[: -(-k // 100)]
+        idx = torch.randperm(k, generator=g, device=device)[: -(-k // 100)]
         x[:, idx] *= 20
     return x.half()
 
 
-def synth_w(n, k, seed=1):
+def synth_w(n, k, seed=1, device="cpu"):
     """N(0, 0.02) weights ("already rotated"), per-row fp16 scale amax/7, RTN codes, packed."""
     from quarot_amd.functional import pack_i4
-    g = torch.Generator().manual_seed(seed)
-    w = (torch.randn(n, k, generator=g) * 0.02).half()
+    g = torch.Generator(device=device).manual_seed(seed)
+    w = (torch.randn(n, k, generator=g, device=device) * 0.02).half()
     s = (w.abs().amax(dim=1, keepdim=True).float() / 7).half()
     codes = torch.clamp(torch.round((w.float() / s.float()).half().float()), -8, 7).to(torch.int8)
     return pack_i4(codes), s
 
 
-def cpu_baseline(x, w_packed, w_scales, hadamard, m, n, k, budget_rows, rmsnorm=False, heads=0):
-    """The reference's CPU path (torch Hadamard + quant + integer matmul + dequant) on a bounded
-    row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
-    from oracle import cpu_baseline as cb
-    rows = min(m, budget_rows)
-    xs = x[:rows].clone()
-    wc = cb.unpacked_codes(w_packed.numpy())
-    ws = w_scales.view(-1)
-    torch.set_num_threads(os.cpu_count() or 1)
-    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
-    times = []
-    for _ in range(3):
+def timed_loops(step, steps, warmup, repeats):
+    """warm-up, then `repeats` loops of `steps` steps, each between two synchronisations and holding
+    nothing but the step's own launches.  Returns per-step milliseconds of every loop."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
         t0 = time.perf_counter()
-        cb.linear4bit_path(xs, wc, ws, hadamard, rmsnorm, heads)
-        times.append(time.perf_counter() - t0)
-    t = float(np.median(times))
-    return {"value": round(2.0 * rows * n * k / t / 1e12, 5), "unit": "TOPS", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"first {rows} of {m} rows, full N and K, median of 3 ({t * 1e3:.0f} ms); torch "
-                      + ("fp32 RMSNorm + " if rmsnorm else "fp32 matmul_hadU + " if hadamard
-                         else "fp32 matmul_hadU over heads + " if heads else "")
-                      + "fp16 sym quant + int32 torch matmul + fp16 dequant"}
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        out.append((time.perf_counter() - t0) * 1e3 / steps)
+    return out
 
 
-def bench_kv(args, dev):
+def spread(ms_list):
+    a = np.asarray(ms_list, dtype=np.float64)
+    return {"median_ms": round(float(np.median(a)), 5), "mean_ms": round(float(a.mean()), 5),
+            "ci95_ms": round(float(1.96 * a.std()), 5), "min_ms": round(float(a.min()), 5), "repeats": int(a.size)}
+
+
+def kernel_ms(fn, reps, replays=3):
+    """Average time of one launch of fn() with the GPU kept busy: `reps` launches are captured in a HIP
+    graph (so the host's per-call cost, longer than the short kernels, is out of the picture) and the
+    replays are timed with HIP events on the launch stream."""
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(reps):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (reps * replays)
+
+
+def gemm_kernel_name(m, n):
+    t256 = ((m + 255) // 256) * ((n + 255) // 256)
+    t128 = ((m + 127) // 128) * ((n + 255) // 256)
+    if m <= 4:
+        return "gemv_i4_kernel"
+    if m <= 64:
+        return "gemm_ks_kernel<64,256>" if m > 16 and (n + 255) // 256 >= 128 else "decode_i4_kernel"
+    if t128 >= 128:         # the library's choice between its two pipelined kernels, by rounds of tiles
+        return "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
+    return "gemm_ks_kernel<64,256>"
+
+
+FRONT_KERNEL = {"had": "hadamard kernel + quantiser (fused)", "quant": "quant_rows_kernel",
+                "rmsnorm": "rmsnorm_quant_rows_kernel", "heads": "heads_hadamard_quant_rows_kernel"}
+
+
+class LinearWorkload:
+    """One quantised linear layer: front (quantiser, optionally behind a Hadamard / RMSNorm / heads
+    Hadamard) + Linear4bit, operands resident in HBM."""
+
+    def __init__(self, name, dev, on_gpu_data=False):
+        import quarot_amd
+        self.q = quarot_amd
+        self.name = name
+        self.m, self.k, self.n, self.front_kind = WORKLOADS[name]
+        m, k, n = self.m, self.k, self.n
+        self.decode = m <= 64
+        src = dev if on_gpu_data else "cpu"
+        self.x_cpu = None
+        x = synth_x(m, k, seed=0 if not self.decode else 3, outliers=not self.decode, device=src)
+        w, sw = synth_w(n, k, seed=1, device=src)
+        if not on_gpu_data:
+            self.x_cpu, self.w_cpu, self.sw_cpu = x, w, sw
+        self.x = x.to(dev)
+        self.lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
+        self.lin.weight.copy_(w.to(dev))
+        self.lin.weight_scales.copy_(sw.to(dev))
+        self.heads = 32 if self.front_kind == "heads" else 0
+        if self.heads:
+            self.x = self.x.view(m, self.heads, k // self.heads)   # as attention writes it: [tokens, heads, head_dim]
+        nn_ = quarot_amd.nn
+        self.front = {"had": lambda: nn_.OnlineHadamardQuantizer(k), "rmsnorm": lambda: nn_.RMSNormQuantizer(k),
+                      "heads": lambda: nn_.HeadsHadamardQuantizer(self.heads), "quant": lambda: nn_.Quantizer()}[self.front_kind]().to(dev)
+        # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
+        self.copies = [self.lin.weight]
+        if self.decode:
+            while sum(c.numel() for c in self.copies) < 640 * 1024 * 1024:
+                self.copies.append(self.lin.weight.clone())
+        self.i = 0
+        # front kernel and GEMM go out in ONE call into the library (decode steps, and the shorter prefill
+        # steps, are otherwise bound by the host's per-call cost)
+        self.one_call = self.front_kind in ("had", "quant")
+        self.had_args = (self.front.had_rem_dim, self.front.rem_dim) if self.front_kind == "had" else (None, 0)
+        self.ops = 2.0 * m * n * k
+
+    def weight(self):
+        w = self.copies[self.i % len(self.copies)]
+        self.i += 1
+        return w
+
+    def step(self):
+        if self.one_call:
+            return self.q.quantized_linear(self.x, self.weight(), self.lin.weight_scales, self.lin.bias, *self.had_args)
+        p = self.front(self.x)
+        return self.q.linear_i4(p.quantized_x, p.scales_x, self.weight(), self.lin.weight_scales, self.lin.bias)
+
+    def gemm(self, p):
+        return self.q.linear_i4(p.quantized_x, p.scales_x, self.weight(), self.lin.weight_scales, self.lin.bias)
+
+    def staged_step(self):
+        """The reference-shaped chain of separate modules (untimed in `value`)."""
+        nn_ = self.q.nn
+        if not hasattr(self, "_staged"):
+            dev = self.x.device
+            if self.front_kind == "had":
+                self._staged = torch.nn.Sequential(nn_.OnlineHadamard(self.k), nn_.Quantizer()).to(dev)
+            elif self.front_kind == "rmsnorm":
+                self._staged = torch.nn.Sequential(nn_.RMSNorm(self.k), nn_.Quantizer()).to(dev)
+            elif self.front_kind == "heads":
+                had_heads, quant = nn_.OnlineHadamard(self.heads).to(dev), nn_.Quantizer()
+                self._staged = lambda t: quant(had_heads(t.transpose(-1, -2)).transpose(-1, -2).reshape(self.m, self.k).contiguous())
+            else:
+                self._staged = nn_.Quantizer()
+        return self.lin(self._staged(self.x))
+
+    def kernel_times(self, reps):
+        """(front kernel ms, GEMM kernel ms), each from a pass of its own: back-to-back launches of that
+        kernel alone (decode: the weights still rotating among their copies)."""
+        p = self.front(self.x)
+        return kernel_ms(lambda: self.front(self.x), reps), kernel_ms(lambda: self.gemm(p), reps)
+
+    def front_bytes(self):
+        return 2.0 * self.m * self.k + self.m * self.k / 2 + 2 * self.m
+
+    def gemm_bytes(self):
+        m, k, n = self.m, self.k, self.n
+        return n * k / 2 + m * k / 2 + 2 * m + 2 * n + 2 * m * n
+
+    def rooflines(self, front_ms, gemm_ms):
+        kern = gemm_kernel_name(self.m, self.n)
+        if self.decode:
+            g = {"bound": "hbm", "achieved": round(self.gemm_bytes() / (gemm_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+        else:
+            g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s"}
+        g["frac"] = round(g["achieved"] / g["peak"], 4)
+        g["kernel"] = kern + " (int4 GEMM + dequant epilogue)"
+        g["kernel_ms"] = round(gemm_ms, 5)
+        f = {"bound": "hbm", "achieved": round(self.front_bytes() / (front_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "kernel": FRONT_KERNEL[self.front_kind], "kernel_ms": round(front_ms, 5)}
+        f["frac"] = round(f["achieved"] / f["peak"], 4)
+        return g, f
+
+    def describe(self):
+        tail = {"had": " with online Hadamard", "rmsnorm": " behind RMSNorm", "heads": f" behind the Hadamard across {self.heads} heads",
+                "quant": ""}[self.front_kind]
+        data = "1% outlier channels x20" if not self.decode else "N(0,1)"
+        return f"{self.name}: Linear4bit X[{self.m},{self.k}] fp16 ({data}) . W int4[{self.n},{self.k}]" + tail
+
+
+def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, graph=False):
+    wl = LinearWorkload(name, dev, on_gpu_data)
+    extra = {}
+    if graph:
+        # one graph per weight copy would defeat the rotation: capture a run of len(copies) steps
+        wl.i = 0
+        want = wl.step().clone()
+        wl.i = 0
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs = [wl.step() for _ in range(len(wl.copies))]
+        g.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(outs[0], want):
+            raise RuntimeError("graph replay differs from the eager step")
+        per = len(wl.copies)
+        loops = [t / per for t in timed_loops(g.replay, max(1, steps // per), max(1, warmup // per), repeats)]
+        extra["launch"] = "hip graph replay"
+    else:
+        loops = timed_loops(wl.step, steps, warmup, repeats)
+        extra["launch"] = "eager" + (" (one library call per step)" if wl.one_call else "")
+    sp = spread(loops)
+    ms = sp["median_ms"]
+    front_ms, gemm_ms = wl.kernel_times(kernel_reps)
+    groof, froof = wl.rooflines(front_ms, gemm_ms)
+    staged = timed_loops(wl.staged_step, max(5, steps // 4), 3, min(repeats, 3))
+    res = {"ms": ms, "value": round(wl.ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": groof,
+           "front": froof, "kernels_ms_sum": round(front_ms + gemm_ms, 5),
+           "staged_reference_api_ms": round(float(np.median(staged)), 5), "workload": wl.describe(), **extra}
+    return wl, res
+
+
+def run_layer(dev, steps, warmup, repeats, kernel_reps):
+    """Workload c3: the four W4A4 linears of a Llama-2-7B decoder layer at M = 32768 tokens (prefill,
+    16 x 2048) as one step; operands generated on the GPU, resident in HBM."""
+    import quarot_amd
+    m = 32768
+    parts = [("qkv", 4096, 12288, "quant", 10), ("o", 4096, 4096, "quant", 11), ("gate_up", 4096, 22016, "quant", 12),
+             ("down", 11008, 4096, "had", 13)]
+    xs = {4096: synth_x(m, 4096, seed=0, device=dev), 11008: synth_x(m, 11008, seed=0, device=dev)}
+    mods = []
+    for name, k, n, kind, seed in parts:
+        w, sw = synth_w(n, k, seed=seed, device=dev)
+        lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
+        lin.weight.copy_(w)
+        lin.weight_scales.copy_(sw)
+        front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if kind == "had" else quarot_amd.nn.Quantizer()).to(dev)
+        mods.append((xs[k], front, lin))
+    ops = sum(2.0 * m * k * n for _, k, n, _, _ in parts)
+
+    def step():
+        for x, front, lin in mods:
+            p = front(x)
+            y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None)
+            del y                                           # 0.3 - 1.4 GB each: returned to the pool before the next one
+
+    sp = spread(timed_loops(step, steps, warmup, repeats))
+    ms = sp["median_ms"]
+    per, gemm_total, front_total = {}, 0.0, 0.0
+    for (name, k, n, kind, _), (x, front, lin) in zip(parts, mods):
+        p = front(x)
+        f_ms = kernel_ms(lambda: front(x), kernel_reps)
+        g_ms = kernel_ms(lambda: quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None), kernel_reps)
+        del p
+        gemm_total += g_ms
+        front_total += f_ms
+        per[name] = {"gemm_ms": round(g_ms, 4), "gemm_TOPS": round(2.0 * m * k * n / (g_ms * 1e-3) / 1e12, 1),
+                     "gemm_frac": round(2.0 * m * k * n / (g_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS, 4),
+                     "front_ms": round(f_ms, 4), "front_GBs": round((2.5 * m * k + 2 * m) / (f_ms * 1e-3) / 1e9, 1)}
+    roof = {"bound": "mfma", "achieved": round(ops / (gemm_total * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s"}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["kernel"] = "gemm_sp256_kernel (int4 GEMM + dequant epilogue), four launches"
+    roof["kernel_ms"] = round(gemm_total, 4)
+    return {"ms": ms, "value": round(ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": roof,
+            "per_linear": per, "kernels_ms_sum": round(gemm_total + front_total, 4), "total_TOP": round(ops / 1e12, 2),
+            "workload": "c3: Llama-2-7B decoder-layer linear set at M=32768 (qkv 4096->12288, o 4096->4096, gate_up 4096->22016, "
+                        "down 11008->4096 with online Hadamard), W4A4, one step = 8 launches"}
+
+
+def run_kv(dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
     """Workload c5: quantise K (Hadamard over the head dimension, then asymmetric int4) and V
-    (asymmetric int4) of one layer, [32, 4096, 8, 128] fp16 each, resident in HBM."""
+    (asymmetric int4) of one layer, [32, 4096, 8, 128] fp16 each, and dequantise both again."""
     from quarot_amd.transformers import kv_cache as kv
     shape = (32, 4096, 8, 128)
 
@@ -139,48 +382,33 @@ def bench_kv(args, dev):
     k, v = k_cpu.to(dev), v_cpu.to(dev)
     vectors = k.numel() // 128
     bytes_one = 2 * k.numel() + vectors * (64 + 4)          # fp16 in; codes + scale + zero out
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
 
-    def step(ev=None):
-        if ev is not None:
-            ev[0].record()
+    def step():
         kq = kv.asym_quantize_and_pack_i4(k, hadamard=True)
-        if ev is not None:
-            ev[1].record()
         vq = kv.asym_quantize_and_pack_i4(v, hadamard=False)
         kd = kv.unpack_i4_and_asym_dequantize(*kq)          # the round trip of the config
         vd = kv.unpack_i4_and_asym_dequantize(*vq)
         return kd, vd
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(evs[i])
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    k_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
-    traffic = None
-    if TRAFFIC_KIB.get("c5"):
-        f, w = TRAFFIC_KIB["c5"]
-        traffic = round((f * FETCH_SCALE + w * WRITE_SCALE) * 1024)
-    roof = {"bound": "hbm", "achieved": round(bytes_one / (k_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "traffic": traffic}
+    sp = spread(timed_loops(step, steps, warmup, repeats))
+    ms = sp["median_ms"]
+    kq = kv.asym_quantize_and_pack_i4(k, hadamard=True)
+    times = {
+        "k_quant_hadamard": kernel_ms(lambda: kv.asym_quantize_and_pack_i4(k, hadamard=True), kernel_reps),
+        "v_quant": kernel_ms(lambda: kv.asym_quantize_and_pack_i4(v, hadamard=False), kernel_reps),
+        "dequant": kernel_ms(lambda: kv.unpack_i4_and_asym_dequantize(*kq), kernel_reps),
+    }
+    k_ms = times["k_quant_hadamard"]
+    roof = {"bound": "hbm", "achieved": round(bytes_one / (k_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
     roof["kernel"] = "kv_had128_kernel (K cache: Hadamard on the matrix cores + asymmetric int4)"
-    roof["kernel_ms"] = round(k_ms, 4)
-    out = {
-        "metric": "KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)", "value": round(4 * bytes_one / (ms * 1e-3) / 1e9, 1),
-        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 -> u4 (fp32 Hadamard, fp16 quantiser)",
-        "data": "synthetic",
-        "config": {"workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector "
-                               "-> fp16 again (four launches)",
-                   "vectors_per_tensor": vectors, "head_dim": 128},
-        "roofline": roof,
-    }
-    if not args.no_cpu_baseline:
+    roof["kernel_ms"] = round(k_ms, 5)
+    res = {"ms": ms, "value": round(4 * bytes_one / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "timing": sp, "roofline": roof,
+           "kernels": {n: {"ms": round(t, 5), "GBs": round(bytes_one / (t * 1e-3) / 1e9, 1), "frac": round(bytes_one / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                       for n, t in times.items()},
+           "workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector "
+                       "-> fp16 again (four launches)", "vectors_per_tensor": vectors, "head_dim": 128}
+    if cpu_baseline:
         from oracle import quarot_oracle as o
         n = vectors // 256                                   # 4096 vectors of each tensor
         ks, vs = k_cpu.reshape(-1, 128)[:n].numpy(), v_cpu.reshape(-1, 128)[:n].numpy()
@@ -189,78 +417,55 @@ def bench_kv(args, dev):
         o.kv_asym_quant(vs)
         t = time.perf_counter() - t0
         sample_bytes = 2 * (2 * ks.size + n * 68)
-        out["cpu_baseline"] = {"value": round(sample_bytes / t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+        res["cpu_baseline"] = {"value": round(sample_bytes / t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"first {n} of {vectors} vectors of each tensor ({t * 1e3:.0f} ms); numpy oracle "
                                          f"(fp32 FWHT + fp16 asymmetric quantiser)"}
-    print(json.dumps(out))
+    return res
 
 
-def bench_layer(args, dev):
-    """Workload c3: the four W4A4 linears of a Llama-2-7B decoder layer at M = 32768 tokens (prefill,
-    16 x 2048) as one step; inputs of each linear are separate seeded tensors resident in HBM."""
-    import quarot_amd
-    m = 32768
-    parts = [("qkv", 4096, 12288, False, 0), ("o", 4096, 4096, False, 10), ("gate_up", 4096, 22016, False, 20),
-             ("down", 11008, 4096, True, 30)]
-    mods = []
-    for name, k, n, had, seed in parts:
-        x = synth_x(m, k, seed=seed, outliers=True).to(dev)
-        w, sw = synth_w(n, k, seed=seed + 1)
-        lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
-        lin.weight.copy_(w.to(dev))
-        lin.weight_scales.copy_(sw.to(dev))
-        front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if had else quarot_amd.nn.Quantizer()).to(dev)
-        mods.append((x, front, lin))
-    ops = sum(2.0 * m * k * n for _, k, n, _, _ in parts)
-    evs = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in parts]
-           for _ in range(args.steps)]
+def cpu_baseline(wl, budget_rows):
+    """The reference's CPU path (torch Hadamard + quant + integer matmul + dequant) on a bounded
+    row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
+    from oracle import cpu_baseline as cb
+    rows = min(wl.m, budget_rows)
+    xs = wl.x_cpu[:rows].clone()
+    wc = cb.unpacked_codes(wl.w_cpu.numpy())
+    ws = wl.sw_cpu.view(-1)
+    hadamard, rmsnorm, heads = wl.front_kind == "had", wl.front_kind == "rmsnorm", wl.heads
+    torch.set_num_threads(os.cpu_count() or 1)
+    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        cb.linear4bit_path(xs, wc, ws, hadamard, rmsnorm, heads)
+        times.append(time.perf_counter() - t0)
+    t = float(np.median(times))
+    return {"value": round(2.0 * rows * wl.n * wl.k / t / 1e12, 5), "unit": "TOPS", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"first {rows} of {wl.m} rows, full N and K, median of 3 ({t * 1e3:.0f} ms); torch "
+                      + ("fp32 RMSNorm + " if rmsnorm else "fp32 matmul_hadU + " if hadamard
+                         else "fp32 matmul_hadU over heads + " if heads else "")
+                      + "fp16 sym quant + int32 torch matmul + fp16 dequant"}
 
-    def step(ev=None):
-        for j, (x, front, lin) in enumerate(mods):
-            p = front(x)
-            if ev is not None:
-                ev[j][0].record()
-            y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None)
-            if ev is not None:
-                ev[j][1].record()
-            del y                                           # 0.8 - 1.4 GB each: returned to the pool before the next one
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(evs[i])
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    gemm = [float(np.mean([evs[i][j][0].elapsed_time(evs[i][j][1]) for i in range(args.steps)])) for j in range(len(parts))]
-    gemm_ms = sum(gemm)
-    roof = {"bound": "mfma", "achieved": round(ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
-            "unit": "TFLOP/s", "traffic": None}
-    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = "gemm_sp256_kernel (int4 GEMM + dequant epilogue), four launches"
-    roof["kernel_ms"] = round(gemm_ms, 4)
-    roof["per_linear"] = {name: {"ms": round(t, 4), "TOPS": round(2.0 * m * k * n / (t * 1e-3) / 1e12, 1)}
-                          for (name, k, n, _, _), t in zip(parts, gemm)}
-    out = {
-        "metric": "Linear4bit TOPS (had+quant+GEMM)", "value": round(ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 scales", "data": "synthetic",
-        "config": {"workload": "c3: Llama-2-7B decoder-layer linear set at M=32768 (qkv 4096->12288, o 4096->4096, "
-                               "gate_up 4096->22016, down 11008->4096 with online Hadamard), W4A4",
-                   "M": m, "total_TOP": round(ops / 1e12, 2)},
-        "roofline": roof,
-    }
-    print(json.dumps(out))
+def brief(res):
+    """The per-config view of a result: step time, value and the dominant kernel's roofline."""
+    keep = ("ms", "value", "unit", "roofline", "front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms", "launch")
+    out = {k: res[k] for k in keep if k in res}
+    out["ci95_ms"] = res["timing"]["ci95_ms"]
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=500, help="steps per timed loop")
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=10, help="timed loops (median and mean +- 1.96 sigma are reported)")
+    ap.add_argument("--kernel-reps", type=int, default=50, help="launches in the separate per-kernel event pass")
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-config", action="store_true", help="measure the chosen workload only")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of the step captured in a HIP graph (decode steps are host-launch-bound when "
                          "launched eagerly from Python); the first replay is checked against the eager result")
@@ -274,7 +479,6 @@ def main():
               "run one process per GPU and add the values (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
 
-    import quarot_amd
     from quarot_amd import _lib
     if not _lib.LIB_PATH.exists():
         from quarot_amd import build
@@ -289,164 +493,67 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": {"launches": 20, "read_bytes": src.numel(), "written_bytes": src.numel()}}))
         return
-    if args.workload == "c5":
-        return bench_kv(args, dev)
-    if args.workload == "c3":
-        return bench_layer(args, dev)
-    m, k, n, hadamard = WORKLOADS[args.workload]
-    x_cpu = synth_x(m, k, seed=0, outliers=True)
-    w_cpu, sw_cpu = synth_w(n, k, seed=1)
-    x = x_cpu.to(dev)
-    lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
-    lin.weight.copy_(w_cpu.to(dev))
-    lin.weight_scales.copy_(sw_cpu.to(dev))
-    rmsnorm = args.workload == "c1n"
-    heads = 32 if args.workload == "c1o" else 0
-    if heads:
-        x = x.view(m, heads, k // heads)                    # as attention writes it: [tokens, heads, head_dim]
-    front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if hadamard else quarot_amd.nn.RMSNormQuantizer(k) if rmsnorm
-             else quarot_amd.nn.HeadsHadamardQuantizer(heads) if heads else quarot_amd.nn.Quantizer()).to(dev)
-    # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
-    copies = [lin.weight]
-    if m <= 64:
-        while sum(c.numel() for c in copies) < 640 * 1024 * 1024:
-            copies.append(lin.weight.clone())
-    state = {"i": 0}
 
-    # decode steps are bound by the host: front kernel and GEMM go out in ONE call into the library
-    # (same two launches; the per-kernel events of the prefill workloads need the two-call form)
-    one_call = m <= 64 and not rmsnorm and not heads
-    had_args = (front.had_rem_dim, front.rem_dim) if hadamard else (None, 0)
+    def measure(name, headline):
+        """headline: the protocol's full step / repeat counts; per-config: a fifth of the steps (at least 20 per
+        loop, at most ~60 ms of GPU time per loop) and 5 loops."""
+        spec = WORKLOADS[name]
+        big = name.startswith("c3") or name == "c5"
+        steps = args.steps if headline else max(20, args.steps // 5)
+        if big:
+            steps = max(5, steps // (25 if name == "c3" else 10))
+        repeats = args.repeats if headline else max(3, args.repeats // 2)
+        kreps = args.kernel_reps if not big else max(5, args.kernel_reps // 5)
+        warm = args.warmup if not big else max(2, args.warmup // 5)
+        if name == "c3":
+            return None, run_layer(dev, steps, warm, repeats, kreps), steps, repeats
+        if name == "c5":
+            return None, run_kv(dev, steps, warm, repeats, kreps, headline and not args.no_cpu_baseline), steps, repeats
+        assert spec is not None
+        wl, res = run_linear(name, dev, steps, warm, repeats, kreps, on_gpu_data=not headline, graph=args.graph and headline)
+        return wl, res, steps, repeats
 
-    def step(ev=None):
-        if one_call and ev is None:
-            w = copies[state["i"] % len(copies)]
-            state["i"] += 1
-            return quarot_amd.quantized_linear(x, w, lin.weight_scales, lin.bias, *had_args)
-        p = front(x)
-        if ev is not None:
-            ev[0].record()
-        w = copies[state["i"] % len(copies)]
-        state["i"] += 1
-        y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, w, lin.weight_scales, lin.bias)
-        if ev is not None:
-            ev[1].record()
-        return y
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    if args.graph:
-        # one graph per weight copy would defeat the rotation: capture a run of len(copies) steps
-        state["i"] = 0
-        want = step().clone()
-        state["i"] = 0
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            outs = [step() for _ in range(len(copies))]
-        graph.replay()
-        torch.cuda.synchronize()
-        if not torch.equal(outs[0], want):
-            raise RuntimeError("graph replay differs from the eager step")
-        reps = max(1, args.steps // len(copies))
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            graph.replay()
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / (reps * len(copies))
-        for i in range(min(args.steps, 20)):                # GEMM time from eager launches (events cannot go into the graph)
-            step(events[i])
-        torch.cuda.synchronize()
-        gemm_ms = float(np.mean([a.elapsed_time(b) for a, b in events[:min(args.steps, 20)]]))
-    else:
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(None if one_call else events[i])
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        ms = (t1 - t0) * 1e3 / args.steps
-        # (decode: the GEMM is timed further down from back-to-back launches)
-        gemm_ms = 0.0 if one_call else float(np.mean([a.elapsed_time(b) for a, b in events]))
-    ops = 2.0 * m * n * k
-    value = ops / (ms * 1e-3) / 1e12
-
-    # staged (reference-shaped) chain for comparison, untimed in `value`
-    staged_front = (torch.nn.Sequential(quarot_amd.nn.OnlineHadamard(k), quarot_amd.nn.Quantizer()) if hadamard
-                    else torch.nn.Sequential(quarot_amd.nn.RMSNorm(k), quarot_amd.nn.Quantizer()) if rmsnorm
-                    else quarot_amd.nn.Quantizer()).to(dev)
-    if heads:
-        # the reference's sequence: transform on the transposed view, transpose back, reshape, quantise
-        had_heads, quant = quarot_amd.nn.OnlineHadamard(heads).to(dev), quarot_amd.nn.Quantizer()
-        staged_front = lambda t: quant(had_heads(t.transpose(-1, -2)).transpose(-1, -2).reshape(m, k).contiguous())
-    for _ in range(3):
-        lin(staged_front(x))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(max(10, args.steps // 4)):
-        lin(staged_front(x))
-    torch.cuda.synchronize()
-    staged_ms = (time.perf_counter() - t0) * 1e3 / max(10, args.steps // 4)
-
-    decode = m <= 64
-    if decode:
-        # a decode step is launch-bound on the host, so events around one launch would time an idle
-        # GPU: time a back-to-back batch of the GEMM launch instead (weights still rotating)
-        p = front(x)
-        reps = 60
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for phase in range(2):
-            if phase == 1:
-                e0.record()
-            for i in range(reps):
-                quarot_amd.linear_i4(p.quantized_x, p.scales_x, copies[i % len(copies)], lin.weight_scales, lin.bias)
-        e1.record()
-        torch.cuda.synchronize()
-        gemm_ms = e0.elapsed_time(e1) / reps
-    traffic = None
-    if args.workload in TRAFFIC_KIB:
-        f, w = TRAFFIC_KIB[args.workload]
-        traffic = round((f * FETCH_SCALE + w * WRITE_SCALE) * 1024)
-    if decode:
-        algo_bytes = n * k / 2 + m * k / 2 + 2 * m + 2 * n + 2 * m * n
-        roof = {"bound": "hbm", "achieved": round(algo_bytes / (gemm_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "traffic": traffic}
-    else:
-        roof = {"bound": "mfma", "achieved": round(ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
-                "unit": "TFLOP/s", "traffic": traffic}
-    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    t256 = ((m + 255) // 256) * ((n + 255) // 256)
-    t128 = ((m + 127) // 128) * ((n + 255) // 256)
-    if m <= 4:
-        kern = "gemv_i4_kernel"
-    elif decode:
-        kern = "gemm_ks_kernel<64,256>" if m > 16 and (n + 255) // 256 >= 128 else "decode_i4_kernel"
-    elif t128 >= 128:       # the library's choice between its two pipelined kernels, by rounds of tiles
-        kern = "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
-    else:
-        kern = "gemm_ks_kernel<64,256>"
-    roof["kernel"] = kern
-    roof["kernel"] += " (int4 GEMM + dequant epilogue)"
-    roof["kernel_ms"] = round(gemm_ms, 4)
-
+    wl, res, steps, repeats = measure(args.workload, True)
+    roof = dict(res["roofline"])
+    traffic, source = traffic_from_profile(args.workload, roof["kernel"])
+    roof["traffic"] = traffic
+    roof["traffic_source"] = source
+    kv_line = args.workload == "c5"
     out = {
-        "metric": "Linear4bit TOPS (had+quant+GEMM)", "value": round(value, 2), "unit": "TOPS", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "int4 x int4 -> int32 (int8 MFMA), fp16 scales",
+        "metric": "KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)" if kv_line else "Linear4bit TOPS (had+quant+GEMM)",
+        "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": steps, "warmup": args.warmup, "repeats": repeats,
+        "ms_per_step": res["ms"], "ms_per_step_mean": res["timing"]["mean_ms"], "ms_per_step_ci95": res["timing"]["ci95_ms"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 -> u4 (fp32 Hadamard, fp16 quantiser)" if kv_line else "int4 x int4 -> int32 (int8 MFMA), fp16 scales",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: Linear4bit X[{m},{k}] fp16 (1% outlier channels x20) . W int4[{n},{k}]"
-                               + (" with online Hadamard" if hadamard else " behind RMSNorm" if rmsnorm
-                                  else f" behind the Hadamard across {heads} heads" if heads else ""),
-                   "M": m, "K": k, "N": n,
-                   "path": ("fused Hadamard+quantise kernel" if hadamard else "fused RMSNorm+quantise kernel" if rmsnorm
-                            else "fused heads-Hadamard+quantise kernel" if heads else "quantise kernel")
-                           + ", fused GEMM+dequant kernel" + (" (one library call per step)" if one_call else ""),
-                   "staged_reference_api_ms": round(staged_ms, 4), "launch": "hip graph replay" if args.graph else "eager"},
+        "config": {"workload": res["workload"], "launch": res.get("launch", "eager"),
+                   "timing": "median of `repeats` loops of `steps` steps, each loop between two synchronisations; kernel times from a "
+                             "separate pass: back-to-back launches of one kernel (a HIP graph), HIP events on the launch stream"},
         "roofline": roof,
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(x_cpu, w_cpu, sw_cpu, hadamard, m, n, k, args.cpu_rows, rmsnorm, heads)
+    for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms"):
+        if key in res:
+            out[key] = res[key]
+    if wl is not None:
+        out["config"].update({"M": wl.m, "K": wl.k, "N": wl.n})
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline(wl, args.cpu_rows)
+    elif "cpu_baseline" in res:
+        out["cpu_baseline"] = res["cpu_baseline"]
+    del wl
+    if not args.no_per_config and args.workload == "c2":
+        per = {}
+        for name in PER_CONFIG:
+            torch.cuda.empty_cache()
+            _, r, _, _ = measure(name, False)
+            per[name] = brief(r)
+            if name != "c3":
+                t, s = traffic_from_profile(name, r["roofline"]["kernel"])
+                if t is not None:
+                    per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = t, s
+        out["per_config"] = per
+        out["per_config_note"] = ("same step definition as the headline; operands generated on the GPU, a fifth of the steps per loop "
+                                  "(c3, c5: fewer still) and half the repeats")
     print(json.dumps(out))
 
 
