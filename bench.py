@@ -28,8 +28,9 @@ HBM rather than from the 256 MB last-level cache.
 Timing follows benchmarks/qlinear_benchmark.py:20-40,88-113: warm-up, then a loop of K steps between two
 synchronisations, repeated R times; the step time is the median of the R loops and the spread is
 reported as mean +- 1.96 sigma.  Nothing but the step's own launches is inside a timed loop; the time
-of each kernel comes from a separate pass: back-to-back launches of that kernel alone, captured in a
-HIP graph so that the host's per-call cost does not show, timed with HIP events on the launch stream.
+of each kernel comes from a separate pass: launches of that kernel alone, each between two HIP events
+on the launch stream, queued behind a few milliseconds of device copies so that the host's per-call
+cost (longer than the short kernels) does not show.
 
 Prints ONE JSON line on stdout.  The default run measures the headline workload (c2) and, in
 `per_config`, every other benchmark configuration with fewer repeats.
@@ -145,25 +146,28 @@ def spread(ms_list):
             "ci95_ms": round(float(1.96 * a.std()), 5), "min_ms": round(float(a.min()), 5), "repeats": int(a.size)}
 
 
-def kernel_ms(fn, reps, replays=3):
-    """Average time of one launch of fn() with the GPU kept busy: `reps` launches are captured in a HIP
-    graph (so the host's per-call cost, longer than the short kernels, is out of the picture) and the
-    replays are timed with HIP events on the launch stream."""
+_BLOCKER = {}
+
+
+def kernel_ms(fn, reps):
+    """Average duration of one launch of fn(), HIP events on the launch stream around every launch.  The
+    host needs longer to issue a launch than a short kernel runs, and an event recorded on an idle GPU
+    would time that host latency: a few milliseconds of device copies are queued first, so that every
+    event and launch of the pass is already waiting in the stream when the GPU reaches it."""
+    if "src" not in _BLOCKER:
+        _BLOCKER["src"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
+        _BLOCKER["dst"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
     fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
     torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        for _ in range(reps):
-            fn()
-    g.replay()
+    for _ in range(max(2, reps // 16)):                      # ~1.6 ms each
+        _BLOCKER["dst"].copy_(_BLOCKER["src"])
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(replays):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / (reps * replays)
+    return float(np.mean([a.elapsed_time(b) for a, b in pairs]))
 
 
 def gemm_kernel_name(m, n):
@@ -252,8 +256,8 @@ class LinearWorkload:
         return self.lin(self._staged(self.x))
 
     def kernel_times(self, reps):
-        """(front kernel ms, GEMM kernel ms), each from a pass of its own: back-to-back launches of that
-        kernel alone (decode: the weights still rotating among their copies)."""
+        """(front kernel ms, GEMM kernel ms), each from a pass of its own (decode: the weights still
+        rotating among their copies)."""
         p = self.front(self.x)
         return kernel_ms(lambda: self.front(self.x), reps), kernel_ms(lambda: self.gemm(p), reps)
 
@@ -528,7 +532,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": res["workload"], "launch": res.get("launch", "eager"),
                    "timing": "median of `repeats` loops of `steps` steps, each loop between two synchronisations; kernel times from a "
-                             "separate pass: back-to-back launches of one kernel (a HIP graph), HIP events on the launch stream"},
+                             "separate pass of that kernel alone, HIP events around every launch on the launch stream"},
         "roofline": roof,
     }
     for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms"):

@@ -231,6 +231,68 @@ int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int had_mode, vo
 int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void* zero, int64_t vectors,
                          int dim, void* y, void* stream);
 
+/*
+ * Paged int4 KV cache (quarot/kernels/include/flashinfer/page.cuh:19-113), head_dim 128:
+ *   kv_data   uint8 [num_pages, num_layers, 2 (K, V), num_heads, page_size, 64]   packed codes
+ *   kv_param  fp16  [num_pages, num_layers, 2 (K, V), num_heads, page_size, 2]    {scale, zero} per vector
+ *   kv_indptr int32 [batch_size + 1], kv_indices int32 [kv_indptr[batch_size]], last_page_offset int32 [batch_size]:
+ *   sequence b owns pages kv_indices[kv_indptr[b] .. kv_indptr[b + 1] - 1] and holds
+ *   (pages - 1) * page_size + last_page_offset[b] tokens.  All five are device pointers.
+ * The index arrays cannot be checked on the host: a token whose place lies outside the sequence's page
+ * list, or on a page number outside [0, num_pages), is skipped on the device instead of written / read.
+ */
+
+/*
+ * Copy already quantised K and V vectors of new tokens into their pages.
+ * Replaces quarot._CUDA.init_kv_i4 and append_kv_i4 (quarot/kernels/bindings.cpp:155-245 ->
+ * AppendPagedKVCachePrefillKernel / AppendPagedKVCacheDecodeKernel, page.cuh:120-219).
+ *   k, v uint8 [tokens, num_heads, 64]; k_param, v_param fp16 [tokens, num_heads, 2] = {scale, zero}.
+ *   append_indptr_or_null: int32 [batch_size + 1] (init_kv_i4's seqlen_indptr): the tokens of sequence b
+ *   are append_indptr[b] .. append_indptr[b + 1] - 1 and become the LAST positions of the sequence, whose
+ *   length (from kv_indptr / last_page_offset) already includes them.  NULL: one token per sequence
+ *   (append_kv_i4), tokens == batch_size, written at position length - 1.
+ *   k, v, kv_data 16-byte aligned.
+ */
+int qr_kv_append_i4(void* kv_data, void* kv_param, const void* kv_indptr, const void* kv_indices,
+                    const void* last_page_offset, int64_t num_pages, const void* k, const void* v,
+                    const void* k_param, const void* v_param, const void* append_indptr_or_null,
+                    int64_t tokens, int num_layers, int layer_idx, int num_heads, int page_size,
+                    int head_dim, int64_t batch_size, void* stream);
+
+/*
+ * The same from fp16 K and V, quantising on the way: what MultiLayerPagedKVCache4Bit.update runs as
+ * matmul_had_cuda(K), asym_quantize_and_pack_i4 (K and V), two torch.cat of {scale, zero} and
+ * init_kv_i4 / append_kv_i4 (quarot/transformers/kv_cache.py:174-251).  Codes, scales and zeros are those
+ * of qr_kv_quant_f16_i4 bit for bit; they go straight to their pages (two launches).
+ *   k, v fp16 [tokens, num_heads, 128]; k_had_mode as qr_kv_quant_f16_i4's had_mode (1: Hadamard over the
+ *   head dimension first); append_indptr_or_null as above.
+ */
+int qr_kv_quant_append_f16_i4(const void* k, const void* v, int64_t tokens, const void* append_indptr_or_null,
+                              int k_had_mode, void* kv_data, void* kv_param, const void* kv_indptr,
+                              const void* kv_indices, const void* last_page_offset, int64_t num_pages,
+                              int num_layers, int layer_idx, int num_heads, int page_size, int head_dim,
+                              int64_t batch_size, void* stream);
+
+/*
+ * Single-query attention over the paged int4 cache:
+ *   o[b, h, :] = sum_j softmax_j( q[b, h, :] . k_j / sqrt(head_dim) ) v_j,   j over the tokens of sequence b,
+ *   k_j[i] = float(code) * scale_j - zero_j in fp32 (quarot/kernels/include/flashinfer/quantization.cuh:59-84).
+ * Replaces quarot._CUDA.batch_decode_i4 (quarot/kernels/bindings.cpp:118-153 ->
+ * BatchDecodeWithPagedKVCacheKernel, decode.cuh:492-689; no rotary embedding, as the reference calls it).
+ *   q, o fp16 [batch_size, num_heads, 128] (q 16-byte aligned).  fp32 arithmetic, results within
+ *   rtol 1e-3 / atol 1e-3 of the exact softmax over the dequantised cache.
+ *   max_seq_len: an upper bound of the sequences' lengths if the caller knows one, else 0.  With it and a
+ *   workspace of qr_batch_decode_workspace_bytes(batch_size, num_heads, max_seq_len) bytes (16-byte
+ *   aligned) a small batch is split along the sequence over several workgroups per (sequence, head) and
+ *   a second launch merges them; without, one workgroup serves each (sequence, head).
+ */
+size_t qr_batch_decode_workspace_bytes(int64_t batch_size, int num_heads, int64_t max_seq_len);
+int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, const void* kv_param,
+                       const void* kv_indptr, const void* kv_indices, const void* last_page_offset,
+                       int64_t num_pages, int num_layers, int layer_idx, int num_heads, int page_size,
+                       int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

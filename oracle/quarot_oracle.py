@@ -26,6 +26,11 @@ How each function is pinned (see tests/test_oracle.py):
                        across heads (only head 0 survives, times sqrt(H)), one-hot heads (sign columns)
   rmsnorm              float64 closed form x / sqrt(sum(x^2) / mean_dim + eps) rounded once,
                        constant rows, mean_dim different from the row length, sign symmetry
+  paged_append/gather  an element-by-element walk over a flat buffer with the reference's offset formulas
+                       (page.cuh:75-103), append -> gather round trips, untouched bytes stay untouched
+  paged_dequant        exact rational arithmetic of float(nibble) * scale - zero rounded once to float32
+  paged_batch_decode   torch's scaled_dot_product_attention in float64 on the gathered, dequantised cache;
+                       a one-token sequence returns v_0, equal V vectors return that vector, q = 0 the mean
 """
 from __future__ import annotations
 
@@ -344,3 +349,89 @@ def kv_asym_dequant(packed, scale, zero):
     nib = np.stack([p & 0xF, p >> 4], axis=-1).reshape(*p.shape[:-1], 2 * p.shape[-1])
     prod = (nib.astype(F32) * np.asarray(scale, F16).astype(F32)).astype(F16)
     return (prod.astype(F32) - np.asarray(zero, F16).astype(F32)).astype(F16)
+
+
+# ----------------------------------------------------------------------------------------------
+# paged int4 KV cache: append and single-query attention
+
+def paged_seq_lens(kv_indptr, last_page_offset, page_size):
+    """Tokens held by every sequence: (pages - 1) * page_size + last_page_offset
+    (quarot/kernels/include/flashinfer/page.cuh:131-133, decode.cuh:516)."""
+    indptr = np.asarray(kv_indptr, dtype=np.int64)
+    pages = indptr[1:] - indptr[:-1]
+    return (pages - 1) * int(page_size) + np.asarray(last_page_offset, dtype=np.int64)
+
+
+def paged_append(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, layer_idx,
+                 append_indptr=None):
+    """AppendPagedKVCachePrefillKernel / AppendPagedKVCacheDecodeKernel (page.cuh:120-219) on numpy arrays,
+    in place.  kv_data uint8 [pages, L, 2, H, P, D/2], kv_param fp16 [pages, L, 2, H, P, 2];
+    k, v uint8 [tokens, H, D/2], k_param, v_param fp16 [tokens, H, 2].  append_indptr None: one token per
+    sequence at position seq_len - 1 (page.cuh:136-140); else the tokens append_indptr[b] ..
+    append_indptr[b + 1] - 1 of sequence b fill its last positions (page.cuh:183-193)."""
+    page_size = kv_data.shape[4]
+    seq = paged_seq_lens(kv_indptr, last_page_offset, page_size)
+    batch = len(seq)
+    for b in range(batch):
+        if append_indptr is None:
+            first, count = b, 1
+        else:
+            first, count = int(append_indptr[b]), int(append_indptr[b + 1] - append_indptr[b])
+        start = int(seq[b]) - count
+        for j in range(count):
+            pos = start + j
+            page = int(kv_indices[int(kv_indptr[b]) + pos // page_size])
+            entry = pos % page_size
+            kv_data[page, layer_idx, 0, :, entry, :] = k[first + j]
+            kv_data[page, layer_idx, 1, :, entry, :] = v[first + j]
+            kv_param[page, layer_idx, 0, :, entry, :] = k_param[first + j]
+            kv_param[page, layer_idx, 1, :, entry, :] = v_param[first + j]
+
+
+def paged_gather(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, b):
+    """The cached vectors of sequence b in position order: (k codes [seq, H, D/2], k param [seq, H, 2],
+    v codes, v param), walking its page list as decode.cuh:560-600 does."""
+    page_size = kv_data.shape[4]
+    n = int(paged_seq_lens(kv_indptr, last_page_offset, page_size)[b])
+    out = [[], [], [], []]
+    for pos in range(n):
+        page = int(kv_indices[int(kv_indptr[b]) + pos // page_size])
+        entry = pos % page_size
+        out[0].append(kv_data[page, layer_idx, 0, :, entry, :])
+        out[1].append(kv_param[page, layer_idx, 0, :, entry, :])
+        out[2].append(kv_data[page, layer_idx, 1, :, entry, :])
+        out[3].append(kv_param[page, layer_idx, 1, :, entry, :])
+    heads, half = kv_data.shape[3], kv_data.shape[5]
+    shapes = [(0, heads, half), (0, heads, 2), (0, heads, half), (0, heads, 2)]
+    return tuple(np.stack(o) if o else np.zeros(s, kv_data.dtype if i % 2 == 0 else kv_param.dtype)
+                 for i, (o, s) in enumerate(zip(out, shapes)))
+
+
+def paged_dequant(codes, param):
+    """dequantize_impl (quarot/kernels/include/flashinfer/quantization.cuh:59-84): float(nibble) * scale - zero
+    in float32, low nibble = even element; scale, zero = the half2 parameter widened to float
+    (decode.cuh:631-636).  codes uint8 [..., D/2], param fp16 [..., 2] -> float32 [..., D]."""
+    p = np.asarray(codes, dtype=np.uint8)
+    nib = np.stack([p & 0xF, p >> 4], axis=-1).reshape(*p.shape[:-1], 2 * p.shape[-1]).astype(F32)
+    prm = np.asarray(param, dtype=F16).astype(F32)
+    return (nib * prm[..., 0:1]).astype(F32) - prm[..., 1:2]
+
+
+def paged_batch_decode(q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx):
+    """BatchDecodeWithPagedKVCacheKernel (decode.cuh:492-689) without rotary embedding, as
+    quarot/kernels/flashinfer.cu:10-46 instantiates it: per sequence and head,
+    softmax(q . K^T / sqrt(D)) . V over the dequantised cache.  float64 here (the kernel works in
+    float32 with an online softmax); q fp16 [B, H, D] -> float64 [B, H, D]."""
+    q = np.asarray(q, dtype=F16).astype(np.float64)
+    batch, heads, dim = q.shape
+    out = np.zeros((batch, heads, dim), np.float64)
+    for b in range(batch):
+        kc, kp, vc, vp = paged_gather(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, b)
+        kf = paged_dequant(kc, kp).astype(np.float64)          # [seq, H, D]
+        vf = paged_dequant(vc, vp).astype(np.float64)
+        logits = np.einsum("hd,shd->hs", q[b], kf) / np.sqrt(np.float64(dim))
+        logits -= logits.max(axis=1, keepdims=True)
+        w = np.exp(logits)
+        w /= w.sum(axis=1, keepdims=True)
+        out[b] = np.einsum("hs,shd->hd", w, vf)
+    return out

@@ -32,6 +32,13 @@ SIGNATURES = {
     "qr_linear_i4_f16_static": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
     "qr_kv_quant_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _ptr, _ptr, _ptr)),
     "qr_kv_dequant_i4_f16": (_int, (_ptr, _ptr, _ptr, _i64, _int, _ptr, _ptr)),
+    "qr_kv_append_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int,
+                               _i64, _ptr)),
+    "qr_kv_quant_append_f16_i4": (_int, (_ptr, _ptr, _i64, _ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int,
+                                         _int, _i64, _ptr)),
+    "qr_batch_decode_workspace_bytes": (_c.c_size_t, (_i64, _int, _i64)),
+    "qr_batch_decode_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int, _i64, _i64, _ptr,
+                                  _c.c_size_t, _ptr)),
 }
 
 QR_DTYPE_F16, QR_DTYPE_F32 = 0, 1

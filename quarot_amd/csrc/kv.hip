@@ -1,7 +1,7 @@
 // KV-cache path: per-head Hadamard (optional) + per-vector asymmetric int4 quantise/pack, and the
 // inverse dequantiser.  A vector of `dim` halves is spread over dim/8 adjacent lanes, 16 bytes each;
 // a wave handles 512/dim vectors, so all global accesses are full-width and coalesced.
-#include "qr_common.h"
+#include "qr_paged.h"
 
 namespace {
 
@@ -71,10 +71,12 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
 }
 
 // LG = log2(lanes per vector) = log2(dim) - 3, 1..5
-template <int LG, bool HAD>
+// PAGED (head dimension 128 only): codes and {scale, zero} go straight to the vector's place in the paged
+// cache instead of dense arrays.
+template <int LG, bool HAD, bool PAGED = false>
 __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ x, int64_t nchunks, float hscale,
                                                       u32* __restrict__ q, f16* __restrict__ scale,
-                                                      f16* __restrict__ zero) {
+                                                      f16* __restrict__ zero, PagedDst pd) {
     const int lane = threadIdx.x & 63;
     constexpr int U = 4;                                 // chunks per thread and turn: their loads are all issued first
     const int64_t stride = (int64_t)gridDim.x * KT * U;  // multiple of 64 > lanes per vector
@@ -195,10 +197,21 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
       for (int u = 0; u < U; ++u) {
           const int64_t c = c0 + u * KT + threadIdx.x;   // nchunks is a multiple of lanes-per-vector: groups are all-live or all-dead
           if (c < nchunks) {
-              q[c] = outws[u];
-              if ((lane & ((1 << LG) - 1)) == 0) {
-                  scale[c >> LG] = scs[u];
-                  zero[c >> LG] = zps[u];
+              if (PAGED) {
+                  const int64_t vec = c >> LG, token = vec / pd.c.num_heads;
+                  int64_t page;
+                  int entry;
+                  if (paged_locate(pd.c, pd.append_indptr, token, page, entry)) {
+                      const int64_t s = paged_slot(pd.c, page, pd.kv, (int)(vec - token * pd.c.num_heads), entry);
+                      ((u32*)pd.c.data)[s * (1 << LG) + (c & ((1 << LG) - 1))] = outws[u];
+                      if ((lane & ((1 << LG) - 1)) == 0) pd.c.param[s] = pack_scale_zero(scs[u], zps[u]);
+                  }
+              } else {
+                  q[c] = outws[u];
+                  if ((lane & ((1 << LG) - 1)) == 0) {
+                      scale[c >> LG] = scs[u];
+                      zero[c >> LG] = zps[u];
+                  }
               }
           }
       }
@@ -262,11 +275,11 @@ constexpr int KM_WAVES = 4;
 
 __device__ __forceinline__ int km_slot(int row, int piece) { return row * 16 + (piece ^ (row & 15)); }
 
-template <bool QUANT>
+template <bool QUANT, bool PAGED = false>
 __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4* __restrict__ x, int64_t vectors,
                                                                      float hscale, u32x4* __restrict__ q,
                                                                      f16* __restrict__ scale, f16* __restrict__ zero,
-                                                                     u32x4* __restrict__ y) {
+                                                                     u32x4* __restrict__ y, PagedDst pd) {
     __shared__ u32x4 km_lds[KM_WAVES * 512];                       // 8 KB per wave
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int v = lane & 31, h = lane >> 5;
@@ -446,25 +459,39 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
             W[2 * m + 1] = __builtin_amdgcn_perm(sw[1], sw[0], 0x07060302u);
         }
         if (vec < vectors) {
-            q[vec * 4 + 2 * h] = u32x4{W[0], W[1], W[2], W[3]};
-            q[vec * 4 + 2 * h + 1] = u32x4{W[4], W[5], W[6], W[7]};
-            if (h == 0) {
-                scale[vec] = sc;
-                zero[vec] = zp;
+            if (PAGED) {
+                const int64_t token = vec / pd.c.num_heads;
+                int64_t page;
+                int entry;
+                if (paged_locate(pd.c, pd.append_indptr, token, page, entry)) {
+                    const int64_t s = paged_slot(pd.c, page, pd.kv, (int)(vec - token * pd.c.num_heads), entry);
+                    u32x4* dst = (u32x4*)pd.c.data + s * 4 + 2 * h;
+                    dst[0] = u32x4{W[0], W[1], W[2], W[3]};
+                    dst[1] = u32x4{W[4], W[5], W[6], W[7]};
+                    if (h == 0) pd.c.param[s] = pack_scale_zero(sc, zp);
+                }
+            } else {
+                q[vec * 4 + 2 * h] = u32x4{W[0], W[1], W[2], W[3]};
+                q[vec * 4 + 2 * h + 1] = u32x4{W[4], W[5], W[6], W[7]};
+                if (h == 0) {
+                    scale[vec] = sc;
+                    zero[vec] = zp;
+                }
             }
         }
     }
 }
 
-template <bool QUANT>
-int launch_had128(const void* x, int64_t vectors, float hscale, void* q, void* scale, void* zero, void* y, hipStream_t st) {
-    auto kern = kv_had128_kernel<QUANT>;
+template <bool QUANT, bool PAGED = false>
+int launch_had128(const void* x, int64_t vectors, float hscale, void* q, void* scale, void* zero, void* y, hipStream_t st,
+                  const PagedDst& pd = PagedDst{}) {
+    auto kern = kv_had128_kernel<QUANT, PAGED>;
     const int64_t blocks = (vectors + 31) >> 5;
     const int64_t want = (blocks + KM_WAVES - 1) / KM_WAVES;
     const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, 64 * KM_WAVES, 0);
     const unsigned grid = (unsigned)(want < cap ? want : cap);
     kern<<<dim3(grid), dim3(64 * KM_WAVES), 0, st>>>((const u32x4*)x, vectors, hscale, (u32x4*)q, (f16*)scale, (f16*)zero,
-                                                    (u32x4*)y);
+                                                    (u32x4*)y, pd);
     return qr_launch_status();
 }
 
@@ -501,10 +528,10 @@ extern "C" int qr_kv_quant_f16_i4(const void* x, int64_t vectors, int dim, int h
     case LG + 3:                                                                                                      \
         if (had_mode)                                                                                                 \
             kv_quant_kernel<LG, true><<<grid, block, 0, st>>>((const u32x4*)x, nchunks, hs, (u32*)q, (f16*)scale,     \
-                                                              (f16*)zero);                                            \
+                                                              (f16*)zero, PagedDst{});                                \
         else                                                                                                          \
             kv_quant_kernel<LG, false><<<grid, block, 0, st>>>((const u32x4*)x, nchunks, hs, (u32*)q, (f16*)scale,    \
-                                                               (f16*)zero);                                           \
+                                                               (f16*)zero, PagedDst{});                               \
         break;
     switch (l2) {
         QR_KV(1) QR_KV(2) QR_KV(3) QR_KV(4) QR_KV(5)
@@ -537,5 +564,44 @@ extern "C" int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void
         case 4: kv_dequant_kernel<4><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
         case 5: kv_dequant_kernel<5><<<grid, block, 0, st>>>((const u32*)q, (const f16*)scale, (const f16*)zero, nchunks, (u32x4*)y); break;
     }
+    return qr_launch_status();
+}
+
+// Quantise new K and V vectors and write them straight into their pages: what
+// MultiLayerPagedKVCache4Bit.update does with matmul_had_cuda, asym_quantize_and_pack_i4 (twice), two
+// torch.cat and init_kv_i4 / append_kv_i4 (quarot/transformers/kv_cache.py:174-251), as two launches.
+extern "C" int qr_kv_quant_append_f16_i4(const void* k, const void* v, int64_t tokens, const void* append_indptr_or_null,
+                                         int k_had_mode, void* kv_data, void* kv_param, const void* kv_indptr,
+                                         const void* kv_indices, const void* last_page_offset, int64_t num_pages,
+                                         int num_layers, int layer_idx, int num_heads, int page_size, int head_dim,
+                                         int64_t batch_size, void* stream) {
+    if (tokens < 0 || num_pages < 0 || num_layers <= 0 || layer_idx < 0 || layer_idx >= num_layers || num_heads <= 0 ||
+        page_size <= 0 || batch_size < 0 || batch_size > 0x7fffffff || head_dim <= 0)
+        return QR_E_SHAPE;
+    if (head_dim != 128) return QR_E_UNSUPPORTED;
+    if (k_had_mode != 0 && k_had_mode != 1) return QR_E_DTYPE;
+    if (batch_size == 0 || tokens == 0) return QR_OK;
+    if (!append_indptr_or_null && tokens != batch_size) return QR_E_SHAPE;
+    if (!k || !v || !kv_data || !kv_param || !kv_indptr || !kv_indices || !last_page_offset) return QR_E_NULL;
+    if (((uintptr_t)k & 15) || ((uintptr_t)v & 15) || ((uintptr_t)kv_data & 15) || ((uintptr_t)kv_param & 3)) return QR_E_ALIGN;
+    PagedDst pd;
+    pd.c = qr_internal_paged_kv(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
+                                num_heads, page_size, batch_size);
+    pd.append_indptr = (const int32_t*)append_indptr_or_null;
+    const int64_t vectors = tokens * num_heads, nchunks = vectors * 16;
+    const float hs = (float)(1.0 / __builtin_sqrt(128.0));
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(grid_for(nchunks, 4 * KT)), block(KT);
+    pd.kv = 0;
+    if (k_had_mode) {
+        const int rc = launch_had128<true, true>(k, vectors, hs, nullptr, nullptr, nullptr, nullptr, st, pd);
+        if (rc != QR_OK) return rc;
+    } else {
+        kv_quant_kernel<4, false, true><<<grid, block, 0, st>>>((const u32x4*)k, nchunks, hs, nullptr, nullptr, nullptr, pd);
+        const int rc = qr_launch_status();
+        if (rc != QR_OK) return rc;
+    }
+    pd.kv = 1;
+    kv_quant_kernel<4, false, true><<<grid, block, 0, st>>>((const u32x4*)v, nchunks, hs, nullptr, nullptr, nullptr, pd);
     return qr_launch_status();
 }

@@ -1,1 +1,3 @@
-from .kv_cache import asym_quantize_and_pack_i4, unpack_i4_and_asym_dequantize, matmul_had_cuda
+"""Mirror of quarot.transformers (quarot/transformers/__init__.py:1)."""
+from .kv_cache import MultiLayerPagedKVCache4Bit
+from . import kv_cache

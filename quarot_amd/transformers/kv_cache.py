@@ -1,8 +1,12 @@
-"""KV-cache quantisation helpers (mirror of quarot/transformers/kv_cache.py:10-33) on HIP kernels.
-The paged cache and decode attention of that file are outside this package."""
+"""KV-cache path (mirror of quarot/transformers/kv_cache.py) on HIP kernels: the asymmetric int4
+quantiser and its inverse, the paged int4 cache (append, quantise-and-append, single-query attention over
+the cache) and the cache class the model code drives.  Pages of fp16 (the reference's disable_quant
+debugging mode) are not built."""
+import functools
 import math
 
 import torch
+
 
 from .. import _lib
 from ..functional.hadamard import hadamard_transform
@@ -59,3 +63,273 @@ def matmul_had_cuda(X, dtype):
     n = X.shape[-1]
     out = hadamard_transform(X.to(dtype).contiguous(), scale=1 / math.sqrt(n))
     return out.to(X.dtype).view(X.shape)
+
+
+# ---------------------------------------------------------------------------------------------------
+# paged int4 cache: kv_data uint8 [pages, layers, 2, heads, page_size, head_dim / 2],
+# kv_param fp16 [pages, layers, 2, heads, page_size, 2] = {scale, zero}
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx):
+    """The checks of quarot/kernels/bindings.cpp:118-245 (CHECK_INPUT / CHECK_DIM / CHECK_EQ) as RuntimeError."""
+    for name, t in (("kv_data", kv_data), ("kv_param", kv_param), ("kv_indptr", kv_indptr), ("kv_indicies", kv_indices),
+                    ("last_page_offset", last_page_offset)):
+        _check(t.is_cuda, f"{fn}: {name} must be a CUDA tensor")
+        _check(t.is_contiguous(), f"{fn}: {name} must be contiguous")
+    _check(kv_data.dim() == 6, f"{fn}: kv_data must be a 6D tensor")
+    _check(kv_param.dim() == 6, f"{fn}: kv_param must be a 6D tensor")
+    _check(kv_indptr.dim() == 1 and kv_indices.dim() == 1 and last_page_offset.dim() == 1,
+           f"{fn}: kv_indptr, kv_indicies and last_page_offset must be 1D tensors")
+    _check(kv_data.dtype == torch.uint8, f"{fn}: kv_data must be uint8 (fp16 pages are not built)")
+    _check(kv_param.dtype == torch.float16, f"{fn}: kv_param must be fp16")
+    for name, t in (("kv_indptr", kv_indptr), ("kv_indicies", kv_indices), ("last_page_offset", last_page_offset)):
+        _check(t.dtype == torch.int32, f"{fn}: {name} must be int32")
+    pages, layers, two, heads, page_size, half_dim = kv_data.shape
+    _check(two == 2 and tuple(kv_param.shape) == (pages, layers, 2, heads, page_size, 2),
+           f"{fn}: kv_param must be [pages, layers, 2, heads, page_size, 2]")
+    _check(half_dim * 2 == 128, f"{fn}: CHECK_EQ(head_dim, 128) failed. {half_dim * 2} vs 128")
+    _check(0 <= int(layer_idx) < layers, f"{fn}: layer_idx out of range")
+    return pages, layers, heads, page_size, half_dim * 2
+
+
+def _append(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
+    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
+    batch = last_page_offset.shape[0]
+    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    for name, t in (("k", k), ("v", v), ("k_param", k_param), ("v_param", v_param)):
+        _check(t.is_cuda and t.is_contiguous() and t.dim() == 3, f"{fn}: {name} must be a contiguous 3D CUDA tensor")
+    _check(k.shape == v.shape and k.dtype == v.dtype == torch.uint8 and tuple(k.shape[1:]) == (heads, head_dim // 2),
+           f"{fn}: k and v must be uint8 [tokens, heads, head_dim / 2]")
+    tokens = k.shape[0]
+    for name, t in (("k_param", k_param), ("v_param", v_param)):
+        _check(t.dtype == torch.float16 and tuple(t.shape) == (tokens, heads, 2), f"{fn}: {name} must be fp16 [tokens, heads, 2]")
+    if seqlen_indptr is None:
+        _check(tokens == batch, f"{fn}: one token per sequence expected")
+    else:
+        _check(seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32
+               and tuple(seqlen_indptr.shape) == (batch + 1,), f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
+    dev = kv_data.device
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_kv_append_i4(
+            kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(), last_page_offset.data_ptr(),
+            pages, k.data_ptr(), v.data_ptr(), k_param.data_ptr(), v_param.data_ptr(),
+            None if seqlen_indptr is None else seqlen_indptr.data_ptr(), tokens, layers, int(layer_idx), heads, page_size,
+            head_dim, batch, _lib.stream_ptr(dev)))
+
+
+def init_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
+    """Write the quantised K / V vectors of a prompt into their pages (kv_cache.py:36-46 ->
+    bindings.cpp:155-198): the tokens seqlen_indptr[b] .. seqlen_indptr[b + 1] - 1 of sequence b become the
+    last positions of that sequence.  Returns None, like the reference's binding."""
+    _append("init_kv_i4", kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr,
+            layer_idx)
+
+
+def append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, layer_idx):
+    """Write one new quantised K / V vector per sequence at its last position (kv_cache.py:49-58 ->
+    bindings.cpp:200-245)."""
+    _append("append_kv_i4", kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, None, layer_idx)
+
+
+def quantize_append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, seqlen_indptr, layer_idx,
+                          hadamard=True):
+    """fp16 K and V [tokens, heads, 128] -> (Hadamard over the head dimension of K) -> asymmetric int4 ->
+    straight into the pages: matmul_had_cuda + asym_quantize_and_pack_i4 (twice) + the two torch.cat +
+    init_kv_i4 / append_kv_i4 of MultiLayerPagedKVCache4Bit.update (kv_cache.py:174-251) as two launches,
+    with the same codes, scales and zeros.  seqlen_indptr None: one token per sequence."""
+    fn = "quantize_append_kv_i4"
+    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
+    batch = last_page_offset.shape[0]
+    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    for name, t in (("k", k), ("v", v)):
+        _check(t.is_cuda and t.is_contiguous() and t.dtype == torch.float16 and t.dim() == 3
+               and tuple(t.shape[1:]) == (heads, head_dim), f"{fn}: {name} must be a contiguous fp16 [tokens, heads, 128] CUDA tensor")
+    _check(k.shape == v.shape, f"{fn}: k and v differ in shape")
+    tokens = k.shape[0]
+    if seqlen_indptr is None:
+        _check(tokens == batch, f"{fn}: one token per sequence expected")
+    else:
+        _check(seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32
+               and tuple(seqlen_indptr.shape) == (batch + 1,), f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
+    dev = kv_data.device
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_kv_quant_append_f16_i4(
+            k.data_ptr(), v.data_ptr(), tokens, None if seqlen_indptr is None else seqlen_indptr.data_ptr(), 1 if hadamard else 0,
+            kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(), last_page_offset.data_ptr(),
+            pages, layers, int(layer_idx), heads, page_size, head_dim, batch, _lib.stream_ptr(dev)))
+
+
+@functools.lru_cache(maxsize=1024)
+def _decode_workspace_bytes(batch, heads, max_seq_len):
+    return _lib.lib().qr_batch_decode_workspace_bytes(batch, heads, max_seq_len)
+
+
+def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, max_seq_len=0):
+    """o[b, h] = softmax(q[b, h] . K^T / sqrt(128)) . V over the int4 cache of sequence b, dequantised in
+    registers as float(code) * scale - zero (kv_cache.py:60-67 -> bindings.cpp:118-153).  Writes into `o`
+    and returns None, like the reference's binding.  max_seq_len (optional, an upper bound of the
+    sequence lengths) lets a small batch be split along the sequence."""
+    fn = "batch_decode_i4"
+    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
+    for name, t in (("o", o), ("q", q)):
+        _check(t.is_cuda and t.is_contiguous(), f"{fn}: {name} must be a contiguous CUDA tensor")
+        _check(t.dim() == 3, f"{fn}: {name} must be a 3D tensor")
+        _check(t.dtype == torch.float16, f"{fn}: {name} must be fp16")
+    _check(o.shape == q.shape, f"{fn}: o.size() != q.size()")
+    batch = o.shape[0]
+    _check(tuple(q.shape[1:]) == (heads, head_dim), f"{fn}: q must be [batch_size, {heads}, {head_dim}]")
+    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    _check(last_page_offset.shape[0] == batch, f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
+    dev = kv_data.device
+    ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len)) if max_seq_len else 0
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_batch_decode_i4(
+            o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
+            last_page_offset.data_ptr(), pages, layers, int(layer_idx), heads, page_size, head_dim, batch, int(max_seq_len),
+            None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+
+
+class _AttentionStub(object):
+    """What MultiLayerPagedKVCache4Bit.update hands back for a decode step (kv_cache.py:104-129): called
+    with the query states it runs attention over the cache."""
+
+    def __init__(self, cache_page_size, device, n_layers, disable_quant, hadamard_dtype):
+        self.cache_page_size = cache_page_size
+        self.n_layers = n_layers
+        self.disable_quant = disable_quant
+        self.hadamard_dtype = hadamard_dtype
+
+    def forward(self, q, num_kv_heads, attention_kwargs, layer_idx, max_seq_len=0):
+        batch_size, q_len, num_qo_heads, head_dim = q.shape
+        assert q_len == 1
+        q = q.view(batch_size, num_qo_heads, head_dim)
+        if self.hadamard_dtype is not None:
+            q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
+        attn_output = torch.empty_like(q)
+        batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len)
+        return attn_output.unsqueeze(1)
+
+
+class MultiLayerPagedKVCache4Bit:
+    """Paged int4 KV cache of all layers with the interface of kv_cache.py:132-289: `update` quantises
+    and stores the new keys and values (the first call per layer takes the whole prompt and returns the
+    fp16 states for the prefill's own attention; later calls take one token per sequence and return a
+    callable that runs decode attention over the cache).  Keys pass through the Hadamard transform over
+    the head dimension before quantisation, queries before attention (hadamard_dtype, None to skip).
+    The reference derives the class from transformers' Cache for the methods that base supplied in the
+    version it pins (get_usable_length); they are defined here instead, so the class does not depend on the
+    installed transformers version."""
+
+    def __init__(self, batch_size, page_size, max_seq_len, device, n_layers, num_heads, head_dim, disable_quant=False,
+                 hadamard_dtype=torch.float16):
+        if disable_quant:
+            raise NotImplementedError("fp16 pages (disable_quant=True) are not built: this cache is int4 only")
+        self.page_size = page_size
+        self.batch_size = batch_size
+        max_page_cnt = self.page_cnt_from_length(max_seq_len)
+        self.disable_quant = disable_quant
+        self.pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
+                                 dtype=torch.uint8, device=device)
+        self.scales = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=torch.float16,
+                                  device=device)
+        self.max_seq_len = max_seq_len
+        self._needs_init = [True] * n_layers
+        self.length = 0
+        self.device = device
+        self.hadamard_dtype = hadamard_dtype
+        self._stub = _AttentionStub(self.page_size, device, n_layers, disable_quant=self.disable_quant,
+                                    hadamard_dtype=self.hadamard_dtype)
+
+    def page_cnt_from_length(self, length):
+        return (length + self.page_size - 1) // self.page_size
+
+    def _ensure_page_cnt_per_batch(self, expected_page_cnt_per_batch):
+        if expected_page_cnt_per_batch * self.batch_size <= self.pages.shape[0]:
+            return
+        raise NotImplementedError
+
+    @property
+    def seen_tokens(self):
+        return self.length
+
+    def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
+        b_sz, added_length, num_heads, head_dim = key_states.shape
+        assert b_sz == self.batch_size
+        cache_kwargs = cache_kwargs or {}
+        if layer_idx == 0:
+            new_length = self.length + added_length
+            self._ensure_page_cnt_per_batch(self.page_cnt_from_length(new_length))
+            self.length = new_length
+        attention_mask = cache_kwargs.get("attention_mask")
+        first = self._needs_init[layer_idx]
+        specs = self.get_cache_specs_for_flash_infer(attention_mask)
+        k_in, fused_had = key_states, self.hadamard_dtype is not None
+        if self.hadamard_dtype is not None and self.hadamard_dtype != torch.float16:
+            k_in, fused_had = matmul_had_cuda(key_states, dtype=self.hadamard_dtype), False   # e.g. the fp32 transform
+        if first:
+            self._needs_init[layer_idx] = False
+            if attention_mask is not None:
+                # padded prompt: quantise every row, keep the rows the mask selects (kv_cache.py:206-220)
+                kq, ks, kz = asym_quantize_and_pack_i4(k_in, hadamard=fused_had)
+                vq, vs, vz = asym_quantize_and_pack_i4(value_states)
+                keep = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+                rows = self.batch_size * added_length
+                pick = lambda t, w: t.reshape(rows, num_heads, w).index_select(0, keep).contiguous()
+                seqlens = torch.nn.functional.pad(torch.cumsum(attention_mask.sum(dim=-1, dtype=torch.int32), dim=0,
+                                                               dtype=torch.int32), (1, 0))
+                init_kv_i4(**specs, k=pick(kq, head_dim // 2), v=pick(vq, head_dim // 2),
+                           k_param=pick(torch.cat([ks, kz], dim=-1), 2), v_param=pick(torch.cat([vs, vz], dim=-1), 2),
+                           seqlen_indptr=seqlens, layer_idx=layer_idx)
+            else:
+                seqlens = torch.arange(self.batch_size + 1, device=self.device, dtype=torch.int32) * added_length
+                quantize_append_kv_i4(**specs, k=k_in.reshape(-1, num_heads, head_dim).contiguous(),
+                                      v=value_states.reshape(-1, num_heads, head_dim).contiguous(), seqlen_indptr=seqlens,
+                                      layer_idx=layer_idx, hadamard=fused_had)
+            return key_states, value_states
+        assert added_length == 1
+        quantize_append_kv_i4(**specs, k=k_in.reshape(self.batch_size, num_heads, head_dim).contiguous(),
+                              v=value_states.reshape(self.batch_size, num_heads, head_dim).contiguous(), seqlen_indptr=None,
+                              layer_idx=layer_idx, hadamard=fused_had)
+        return functools.partial(self._stub.forward, num_kv_heads=num_heads, attention_kwargs=specs, layer_idx=layer_idx,
+                                 max_seq_len=self.length)
+
+    def get_cache_specs_for_flash_infer(self, attention_mask):
+        """Page tables of the current state (kv_cache.py:253-275): page i of sequence b is page number
+        i * batch_size + b; every sequence must span the same number of pages."""
+        if attention_mask is not None:
+            seqlens_in_batch = attention_mask.sum(dim=-1, dtype=torch.int32)
+        else:
+            seqlens_in_batch = torch.tensor([self.length], dtype=torch.int32, device=self.device).expand(self.batch_size)
+        page_cnt = self.page_cnt_from_length(seqlens_in_batch)
+        if (page_cnt[0] != page_cnt).any():
+            raise NotImplementedError("Current implementation does not support the case where batches have different number of pages")
+        page_cnt = page_cnt[0]
+        page_ptr = seqlens_in_batch % self.page_size
+        page_ptr = torch.where((seqlens_in_batch != 0) & (page_ptr == 0), self.page_size, page_ptr).to(torch.int32).contiguous()
+        arange = functools.partial(torch.arange, device=self.device, dtype=torch.int32)
+        return {
+            "kv_data": self.pages,
+            "kv_indptr": (arange(0, self.batch_size + 1) * page_cnt).to(torch.int32),
+            "kv_indices": ((arange(int(page_cnt)) * self.batch_size).unsqueeze(0) + arange(self.batch_size).unsqueeze(1)).reshape(-1).contiguous(),
+            "last_page_offset": page_ptr,
+            "kv_param": self.scales,
+        }
+
+    def get_seq_length(self, layer_idx=0):
+        return self.length
+
+    def get_max_length(self):
+        return None
+
+    def get_usable_length(self, new_seq_length, layer_idx=0):
+        """transformers' Cache.get_usable_length for a cache without a maximum length: everything seen so far
+        (called by e2e/quantized_llama/modeling_llama.py:54)."""
+        return self.get_seq_length(layer_idx)
+
+    def to_legacy_cache(self):
+        return self

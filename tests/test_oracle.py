@@ -8,6 +8,7 @@ from fractions import Fraction
 import numpy as np
 import pytest
 import scipy.linalg
+import torch
 
 from oracle import quarot_oracle as o
 
@@ -425,3 +426,126 @@ def test_heads_hadamard_is_the_transform_over_the_head_axis():
     H16 = scipy.linalg.hadamard(16)
     for g in range(16):
         assert np.array_equal(y[g], (e[0, 5].astype(F32) * F32(0.25 * H16[g, 5])).astype(F16))
+
+
+# ------------------------------------------------------------------------------ paged KV cache
+
+def bits(a):
+    return np.ascontiguousarray(a).view(np.uint16)
+
+
+def _paged_case(rng, batch, heads, page_size, lens, layers=2, spare_pages=3, shuffle=True):
+    """A cache with every sequence's pages scattered over the page pool."""
+    per = [max(1, -(-n // page_size)) for n in lens]
+    total = sum(per) + spare_pages
+    order = rng.permutation(total) if shuffle else np.arange(total)
+    indptr = np.concatenate([[0], np.cumsum(per)]).astype(np.int32)
+    indices = order[: sum(per)].astype(np.int32)
+    last = np.array([n - (p - 1) * page_size for n, p in zip(lens, per)], np.int32)
+    data = rng.integers(0, 256, (total, layers, 2, heads, page_size, 64), dtype=np.uint8)
+    param = rng.standard_normal((total, layers, 2, heads, page_size, 2)).astype(F16)
+    return data, param, indptr, indices, last
+
+
+def test_paged_append_follows_the_reference_offset_formulas():
+    """The numpy-indexed oracle against an element-by-element walk over FLAT buffers with the offset
+    formulas of page.cuh:75-103 spelled out, prefill (ragged lengths, pages partly filled before) and
+    one-token append; bytes of other layers, pages and entries must stay untouched."""
+    rng = np.random.default_rng(5)
+    heads, P, L, layer = 3, 4, 2, 1
+    lens = [6, 1, 9, 4]                                   # lengths AFTER the append
+    add = [3, 1, 9, 2]
+    data, param, indptr, indices, last = _paged_case(rng, 4, heads, P, lens, layers=L)
+    app = np.concatenate([[0], np.cumsum(add)]).astype(np.int32)
+    T = int(app[-1])
+    k, v = rng.integers(0, 256, (T, heads, 64), dtype=np.uint8), rng.integers(0, 256, (T, heads, 64), dtype=np.uint8)
+    kp, vp = rng.standard_normal((T, heads, 2)).astype(F16), rng.standard_normal((T, heads, 2)).astype(F16)
+    want_d, want_p = data.copy().reshape(-1), param.copy().reshape(-1, 2)
+    for b in range(4):
+        seq = (indptr[b + 1] - indptr[b] - 1) * P + last[b]
+        for j in range(add[b]):
+            pos = seq - add[b] + j
+            page, entry = indices[indptr[b] + pos // P], pos % P
+            for h in range(heads):
+                for kv, src, sp in ((0, k, kp), (1, v, vp)):
+                    # get_k_elem_offset / get_v_elem_offset in elements of 4 bits -> bytes / 2; parameters in half2
+                    slot = (((page * L + layer) * 2 + kv) * heads + h) * P + entry
+                    for f in range(64):
+                        want_d[slot * 64 + f] = src[app[b] + j, h, f]
+                    want_p[slot] = sp[app[b] + j, h]
+    before = data.copy()
+    o.paged_append(data, param, indptr, indices, last, k, v, kp, vp, layer, app)
+    assert np.array_equal(data.reshape(-1), want_d) and np.array_equal(bits(param.reshape(-1, 2)), bits(want_p))
+    assert np.array_equal(data[:, 0], before[:, 0])                           # the other layer
+    # one token per sequence
+    d2, p2 = data.copy(), param.copy()
+    k1, v1 = k[:4], v[:4]
+    o.paged_append(d2, p2, indptr, indices, last, k1, v1, kp[:4], vp[:4], layer, None)
+    for b in range(4):
+        kc, kpar, vc, vpar = o.paged_gather(d2, p2, indptr, indices, last, layer, b)
+        assert kc.shape == (lens[b], heads, 64)
+        assert np.array_equal(kc[-1], k1[b]) and np.array_equal(vc[-1], v1[b]) and np.array_equal(bits(vpar[-1]), bits(vp[b]))
+        if lens[b] > 1:                                                       # earlier positions: what the prefill wrote
+            kc0, _, _, _ = o.paged_gather(data, param, indptr, indices, last, layer, b)
+            assert np.array_equal(kc[:-1], kc0[:-1])
+
+
+def test_paged_append_then_gather_round_trip():
+    rng = np.random.default_rng(6)
+    heads, P = 2, 16
+    lens = [16, 33, 5]
+    data, param, indptr, indices, last = _paged_case(rng, 3, heads, P, lens, layers=1)
+    app = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(app[-1])
+    k, v = rng.integers(0, 256, (T, heads, 64), dtype=np.uint8), rng.integers(0, 256, (T, heads, 64), dtype=np.uint8)
+    kp, vp = rng.standard_normal((T, heads, 2)).astype(F16), rng.standard_normal((T, heads, 2)).astype(F16)
+    o.paged_append(data, param, indptr, indices, last, k, v, kp, vp, 0, app)
+    for b in range(3):
+        kc, kpar, vc, vpar = o.paged_gather(data, param, indptr, indices, last, 0, b)
+        sl = slice(app[b], app[b + 1])
+        assert np.array_equal(kc, k[sl]) and np.array_equal(vc, v[sl])
+        assert np.array_equal(bits(kpar), bits(kp[sl])) and np.array_equal(bits(vpar), bits(vp[sl]))
+    assert np.array_equal(o.paged_seq_lens(indptr, last, P), lens)
+
+
+def test_paged_dequant_is_one_float32_rounding_of_the_exact_value():
+    """float(nibble) * scale is exact in float32 (4 + 11 significant bits); subtracting zero rounds once."""
+    rng = np.random.default_rng(7)
+    codes = rng.integers(0, 256, (40, 64), dtype=np.uint8)
+    param = (rng.standard_normal((40, 2)) * np.array([0.3, 2.0])).astype(F16)
+    got = o.paged_dequant(codes, param)
+    assert got.dtype == F32 and got.shape == (40, 128)
+    for r in range(0, 40, 7):
+        s, z = Fraction(float(param[r, 0])), Fraction(float(param[r, 1]))
+        for i in (0, 1, 2, 63, 126, 127):
+            nib = int(codes[r, i // 2]) >> (4 * (i % 2)) & 0xF                # even element in the low nibble
+            exact = nib * s - z
+            assert got[r, i] == F32(float(exact)) or abs(Fraction(float(got[r, i])) - exact) <= abs(exact) * Fraction(1, 1 << 24)
+            assert Fraction(float(F32(nib) * F32(float(param[r, 0])))) == nib * s
+
+
+def test_paged_batch_decode_against_textbook_attention():
+    """torch's scaled_dot_product_attention in float64 on the gathered, dequantised vectors; and special
+    cases a wrong softmax axis, a missing 1/sqrt(D) or K/V swapped would fail."""
+    rng = np.random.default_rng(8)
+    heads, P = 4, 8
+    lens = [1, 8, 19, 40]
+    data, param, indptr, indices, last = _paged_case(rng, 4, heads, P, lens, layers=2)
+    param[..., 0] = (np.abs(param[..., 0].astype(F32)) * 0.05 + 0.01).astype(F16)      # positive scales
+    q = rng.standard_normal((4, heads, 128)).astype(F16)
+    got = o.paged_batch_decode(q, data, param, indptr, indices, last, 1)
+    for b in range(4):
+        kc, kp, vc, vp = o.paged_gather(data, param, indptr, indices, last, 1, b)
+        kf = torch.from_numpy(o.paged_dequant(kc, kp)).double().permute(1, 0, 2)      # [H, seq, D]
+        vf = torch.from_numpy(o.paged_dequant(vc, vp)).double().permute(1, 0, 2)
+        want = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q[b]).double().unsqueeze(1), kf, vf)
+        np.testing.assert_allclose(got[b], want.squeeze(1).numpy(), rtol=1e-10, atol=1e-10)
+    # a sequence of one token returns v_0 whatever q is
+    _, _, vc, vp = o.paged_gather(data, param, indptr, indices, last, 1, 0)
+    np.testing.assert_allclose(got[0], o.paged_dequant(vc, vp)[0].astype(np.float64), rtol=1e-12)
+    # q = 0: uniform weights, the mean of V
+    g0 = o.paged_batch_decode(np.zeros_like(q), data, param, indptr, indices, last, 1)
+    _, _, vc, vp = o.paged_gather(data, param, indptr, indices, last, 1, 3)
+    np.testing.assert_allclose(g0[3], o.paged_dequant(vc, vp).astype(np.float64).mean(axis=0), rtol=1e-10, atol=1e-12)
+    # the other layer holds different data: a wrong layer offset changes the result
+    assert not np.allclose(o.paged_batch_decode(q, data, param, indptr, indices, last, 0), got)
