@@ -20,6 +20,10 @@ outlier channels that motivate the Hadamard):
     c4gT  gate_up 70B decode    X [T, 8192]   W int4 [57344, 8192]
     c5  KV-cache write path of one layer: K and V [32, 4096, 8, 128] fp16 -> asymmetric int4 per head
         vector (K through the head-dimension Hadamard first) -> fp16 again; metric GB/s of algorithmic bytes
+    c6  one decode step on the paged int4 cache that c5's tensors fill (32 sequences x 4096 tokens x 8 heads x 128,
+        pages of 16): quantise-and-append of the new token's K / V, Hadamard of the query, attention over the
+        cache; metric GB/s of the cache bytes read (c6b: 1 sequence x 2048 tokens x 32 heads, the default of
+        benchmarks/qattention_benchmark.py:9-13,129-139)
     b13v, b70v, b13d, b70d  the other sizes of the reference's benchmarks/qlinear_benchmark.py:8-18 at 2048 tokens
         (5120->5120, 8192->8192 with the Hadamard in front; down_proj 13824->5120 and 28672->8192 with it)
 Decode workloads (M <= 64) rotate among several copies of the weights so that they are streamed from
@@ -61,6 +65,8 @@ WORKLOADS = {
     "c3d": (32768, 11008, 4096, "had"),       # down_proj
     "c3": None,                               # the whole layer set as one step
     "c5": None,                               # KV-cache quantisation
+    "c6": None,                               # decode attention over the paged int4 cache of config 5's size
+    "c6b": None,                              # the same at the reference benchmark's default: 1 sequence x 2048 tokens x 32 heads
     "b13v": (2048, 5120, 5120, "had"),        # qlinear_benchmark.py model_sizes / mlp_sizes at 13B and 70B
     "b70v": (2048, 8192, 8192, "had"),
     "b13d": (2048, 13824, 5120, "had"),
@@ -69,7 +75,7 @@ WORKLOADS = {
 for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
-PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5"]
+PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 HBM_PEAK_GBS = 8000.0
 
@@ -427,6 +433,58 @@ def run_kv(dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
     return res
 
 
+def run_attention(name, dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
+    """Workloads c6 / c6b: one decode step on the paged int4 KV cache, driven as
+    benchmarks/qattention_benchmark.py:53-57 drives it (length set by hand, update() with one new token per
+    sequence, the returned callable on the query)."""
+    from quarot_amd.transformers import kv_cache as kv
+    B, S, H, P = (32, 4096, 8, 16) if name == "c6" else (1, 2048, 32, 2048)
+    g = torch.Generator(device=dev).manual_seed(4)
+    k = torch.randn(B, S, H, 128, generator=g, device=dev)
+    mask = torch.rand(k.shape, generator=g, device=dev) < 0.005
+    k[mask] *= 15
+    v = torch.randn(B, S, H, 128, generator=g, device=dev)
+    v[mask] *= 15
+    cache = kv.MultiLayerPagedKVCache4Bit(B, P, S, dev, 1, H, 128)
+    cache.update(k.half(), v.half(), 0, {})                  # the prompt: S tokens per sequence
+    del k, v, mask
+    k1 = torch.randn(B, 1, H, 128, generator=g, device=dev).half()
+    v1 = torch.randn(B, 1, H, 128, generator=g, device=dev).half()
+    q1 = torch.randn(B, 1, H, 128, generator=g, device=dev).half()
+
+    def step():
+        cache.length = S - 1                                 # the new token overwrites the last position every step
+        return cache.update(k1, v1, 0, {})(q1)
+
+    sp = spread(timed_loops(step, steps, warmup, repeats))
+    ms = sp["median_ms"]
+    specs = cache.get_cache_specs_for_flash_infer(None)
+    qh = kv.matmul_had_cuda(q1.view(B, H, 128), torch.float16)
+    out = torch.empty_like(qh)
+    a_ms = kernel_ms(lambda: kv.batch_decode_i4(out, qh, **specs, layer_idx=0, max_seq_len=S), kernel_reps)
+    cache_bytes = B * H * S * (2 * 64 + 2 * 4)               # codes and {scale, zero} of K and V
+    roof = {"bound": "hbm", "achieved": round(cache_bytes / (a_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
+    roof["kernel"] = "paged_decode_i4_kernel (single-query attention, in-register dequantisation)"
+    roof["kernel_ms"] = round(a_ms, 5)
+    res = {"ms": ms, "value": round(cache_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "timing": sp, "roofline": roof,
+           "workload": f"{name}: decode step on the paged int4 KV cache, {B} sequences x {S} tokens x {H} heads x 128, pages of {P}: "
+                       "quantise-and-append of one token per sequence, query Hadamard, attention over the cache"}
+    if cpu_baseline:
+        from oracle import quarot_oracle as o
+        nb = 1                                               # one sequence, all heads
+        tabs = [specs[n].cpu().numpy() for n in ("kv_indptr", "kv_indices", "last_page_offset")]
+        one = (tabs[0][:2], tabs[1][:tabs[0][1]], tabs[2][:1])
+        pages, scales = cache.pages.cpu().numpy(), cache.scales.cpu().numpy()
+        t0 = time.perf_counter()
+        o.paged_batch_decode(qh[:nb].cpu().numpy(), pages, scales, *one, 0)
+        t = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": round(nb * H * S * 136 / t / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"sequence 0 of {B}, all heads ({t * 1e3:.0f} ms); numpy oracle (gather, fp32 dequantisation, "
+                                         "float64 softmax attention)"}
+    return res
+
+
 def cpu_baseline(wl, budget_rows):
     """The reference's CPU path (torch Hadamard + quant + integer matmul + dequant) on a bounded
     row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
@@ -502,7 +560,7 @@ def main():
         """headline: the protocol's full step / repeat counts; per-config: a fifth of the steps (at least 20 per
         loop, at most ~60 ms of GPU time per loop) and 5 loops."""
         spec = WORKLOADS[name]
-        big = name.startswith("c3") or name == "c5"
+        big = name.startswith("c3") or name in ("c5", "c6")
         steps = args.steps if headline else max(20, args.steps // 5)
         if big:
             steps = max(5, steps // (25 if name == "c3" else 10))
@@ -513,6 +571,8 @@ def main():
             return None, run_layer(dev, steps, warm, repeats, kreps), steps, repeats
         if name == "c5":
             return None, run_kv(dev, steps, warm, repeats, kreps, headline and not args.no_cpu_baseline), steps, repeats
+        if name in ("c6", "c6b"):
+            return None, run_attention(name, dev, steps, warm, repeats, kreps, headline and not args.no_cpu_baseline), steps, repeats
         assert spec is not None
         wl, res = run_linear(name, dev, steps, warm, repeats, kreps, on_gpu_data=not headline, graph=args.graph and headline)
         return wl, res, steps, repeats
@@ -522,9 +582,11 @@ def main():
     traffic, source = traffic_from_profile(args.workload, roof["kernel"])
     roof["traffic"] = traffic
     roof["traffic_source"] = source
-    kv_line = args.workload == "c5"
+    kv_line = args.workload in ("c5", "c6", "c6b")
     out = {
-        "metric": "KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)" if kv_line else "Linear4bit TOPS (had+quant+GEMM)",
+        "metric": ("KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)" if args.workload == "c5"
+                   else "decode attention over the paged int4 KV cache, GB/s of cache bytes" if kv_line
+                   else "Linear4bit TOPS (had+quant+GEMM)"),
         "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": steps, "warmup": args.warmup, "repeats": repeats,
         "ms_per_step": res["ms"], "ms_per_step_mean": res["timing"]["mean_ms"], "ms_per_step_ci95": res["timing"]["ci95_ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

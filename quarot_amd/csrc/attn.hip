@@ -43,8 +43,7 @@ __global__ __launch_bounds__(256) void paged_append_i4_kernel(PagedKV c, const u
 // keeps its own running maximum, denominator and 32-dimension accumulator for the positions it visits
 // (U of them per step, so the accumulator is rescaled once per U positions); the 64 partial states of
 // the workgroup are merged through LDS at the end.
-constexpr int AT = 256;
-constexpr int AU = 4;                 // positions per lane group and step
+constexpr int AU = 2;                 // positions per lane group and step (two steps are in flight)
 
 __device__ __forceinline__ float quad_sum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // lanes ^ 1
@@ -52,138 +51,286 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
+// float(byte k of w): one instruction each (v_cvt_f32_ubyte0..3).  Spelled as asm because the compiler,
+// seeing the nibble mask applied before, prefers a 4-bit field extract per element plus ubyte0, which
+// doubles the instruction count of the inner loops.
 __device__ __forceinline__ float byte_f32(u32 w, int k) {
+    float f;
     switch (k) {
-        case 0: return (float)(w & 0xffu);
-        case 1: return (float)((w >> 8) & 0xffu);
-        case 2: return (float)((w >> 16) & 0xffu);
-        default: return (float)(w >> 24);
+        case 0: asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(w)); break;
+        case 1: asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(w)); break;
+        case 2: asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(w)); break;
+        default: asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(w)); break;
     }
+    return f;
 }
 
-// ALIGNED: page_size is a multiple of 16, so the 16 positions of a wave step lie in one page
-template <bool ALIGNED>
-__global__ __launch_bounds__(AT, 4) void paged_decode_i4_kernel(const f16* __restrict__ q, PagedKV c, f16* __restrict__ o,
-                                                            float sm_scale_log2, int splits, float* __restrict__ part) {
-    __shared__ float st[64 * 4 * 36];                      // [wave * 16 + slot][quarter][m, d, -, -, acc[32]]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Codes of one 32-bit word (eight nibbles) as four fp16 pairs, exponent bits or-ed in so that no integer
+// to float conversion is needed: pair i holds codes i and i + 4 as BIAS + code, BIAS = 1024 for i = 0, 2
+// (code in mantissa bits 0..3 under exponent 25) and 64 for i = 1, 3 (code in mantissa bits 4..7 under
+// exponent 21).  One shift and four and-or instructions per word.
+struct CodePairs {
+    u32 p[4];
+};
+__device__ __forceinline__ CodePairs code_pairs(u32 w, u32 mask_lo, u32 bias_lo, u32 mask_hi, u32 bias_hi) {
+    CodePairs r;
+    const u32 w8 = w >> 8;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r.p[0]) : "v"(w), "v"(mask_lo), "v"(bias_lo));
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r.p[1]) : "v"(w), "v"(mask_hi), "v"(bias_hi));
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r.p[2]) : "v"(w8), "v"(mask_lo), "v"(bias_lo));
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r.p[3]) : "v"(w8), "v"(mask_hi), "v"(bias_hi));
+    return r;
+}
+constexpr float kBiasEven = 1024.0f, kBiasOdd = 64.0f;
+
+template <int CTRL>
+__device__ __forceinline__ float row_rotate(float v) {   // DPP row_ror within each row of 16 lanes
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+// ALIGNED: page_size is a multiple of 16, so the 16 positions of a wave step lie in one page.
+// NW: waves per workgroup (4 or 16): a (sequence, head) gets NW * splits waves in all.
+template <bool ALIGNED, int NW>
+__global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void paged_decode_i4_kernel(
+    const f16* __restrict__ q, PagedKV c, f16* __restrict__ o, float sm_scale_log2, int splits, float* __restrict__ part) {
+    __shared__ float st[NW * 4 * 4 * 36];                  // [wave * 4 + row][quarter][m, d, -, -, acc[32]]
+    __shared__ float st2[(NW / 2) * 128 * 3];              // second merge level: [part][dimension][m, d, o]
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int slot = lane >> 2, c4 = lane & 3;
     const int bh = blockIdx.x / splits, sp = blockIdx.x - bh * splits;
     const int b = bh / c.num_heads, h = bh - b * c.num_heads;
     const int p0 = c.indptr[b], npages = c.indptr[b + 1] - p0;
     const int seq_len = npages > 0 ? (npages - 1) * c.page_size + c.last_page_offset[b] : 0;
 
-    // this lane's 32 query values, in the order the code bytes are consumed: word j, byte k holds
-    // dimensions 8 j + 2 k (low nibble) and 8 j + 2 k + 1 (high nibble, converted times 16)
-    float qlo[4][4], qhi[4][4], qs = 0.f;
+    // this lane's 32 query values as fp16 pairs in the order the codes are consumed: word j of a 16-byte
+    // piece holds dimensions 8 j .. 8 j + 7, and (word >> 4 i) & 0x000F000F isolates codes i and i + 4
+    f16x2 qp[4][4];
+    float ql = 0.f;                                        // sum of this lane's 32 values
     {
-        const u32x4* qp = (const u32x4*)(q + (int64_t)bh * 128 + c4 * 32);
+        const u32x4* qsrc = (const u32x4*)(q + (int64_t)bh * 128 + c4 * 32);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const u32x4 w = qp[j];
+            const u32x4 w = qsrc[j];
+            f16 e[8];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const f16x2 pr = as_f16x2(w[k]);
-                qlo[j][k] = (float)pr[0];
-                qhi[j][k] = (float)pr[1] * 0.0625f;
-                qs += (float)pr[0] + (float)pr[1];
+                e[2 * k] = pr[0];
+                e[2 * k + 1] = pr[1];
+                ql += (float)pr[0] + (float)pr[1];
             }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) qp[j][i] = f16x2{e[i], e[i + 4]};
         }
     }
-    qs = quad_sum(qs);                                     // sum of all 128 query values
+    const float qs = quad_sum(ql);                         // sum of all 128 query values
+    float qbias = 0.f;                                     // sum over this lane's values of q * (bias of its code)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            qbias = __builtin_fmaf((float)qp[j][i][0] + (float)qp[j][i][1], (i & 1) ? kBiasOdd : kBiasEven, qbias);
+    u32 mask_lo = 0x000F000Fu, bias_lo = 0x64006400u, mask_hi = 0x00F000F0u, bias_hi = 0x54005400u;
+    asm volatile("" : "+v"(mask_lo), "+v"(bias_lo), "+v"(mask_hi), "+v"(bias_hi));     // kept in registers for v_and_or_b32
 
-    float m = -5e4f, d = 0.f, pz = 0.f, acc[32];
+    float m = -5e4f, d = 0.f, pz = 0.f, psum = 0.f, acc[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i) acc[i] = 0.f;
 
     const int chunks = (seq_len + 15) >> 4;
-    const int cpp = ALIGNED ? c.page_size >> 4 : 1;        // chunks per page
-    for (int g0 = sp * 4 + wave; g0 < chunks; g0 += 4 * splits * AU) {
+    // a vector's place: slot = page * page_slots + head_slots + entry (K), + kv_slots (V); 64 code bytes and
+    // one parameter word per slot
+    const int64_t page_slots = (int64_t)c.num_layers * 2 * c.num_heads * c.page_size;
+    const int64_t head_slots = ((int64_t)c.layer_idx * 2 * c.num_heads + h) * c.page_size;
+    const int64_t kv_slots = (int64_t)c.num_heads * c.page_size;
+    const int stride = NW * splits;                         // chunks between the steps of one wave
+    // ALIGNED: chunk g lies in page g / cpp at entry 16 (g % cpp); both advance without divisions
+    const int cpp = ALIGNED ? c.page_size >> 4 : 1;
+    const int it_step = stride / cpp, r_step = stride - it_step * cpp;
+    int g = sp * NW + wave;
+    int it_u = g / cpp, r_u = g - it_u * cpp;
+    // Two sets of AU positions per lane group: the loads of the next set are issued before the current
+    // one is consumed, so their latency hides under the arithmetic.  Loads are unconditional (a position
+    // beyond the sequence reads entry 0 of a valid page and is masked), which keeps the loop free of
+    // branches around memory operations.
+    struct Step {
         u32x4 kw[AU], vw[AU];
         u32 kp[AU], vp[AU];
         bool ok[AU];
+    };
+    auto issue = [&](Step& t, int g0) {
+        int64_t page[AU];
+        int entry[AU];
+        // page numbers first (scalar loads when ALIGNED), then every vector load of the step
 #pragma unroll
         for (int u = 0; u < AU; ++u) {
-            const int g = g0 + u * 4 * splits, pos = g * 16 + slot;
-            int it, entry;
+            const int pos = (g0 + u * stride) * 16 + slot;
+            int it;
             if (ALIGNED) {
-                it = g / cpp;                              // wave-uniform
-                entry = (g - it * cpp) * 16 + slot;
+                it = __builtin_amdgcn_readfirstlane(it_u);  // wave-uniform: the page number comes by a scalar load
+                entry[u] = r_u * 16 + slot;
+                it_u += it_step;
+                r_u += r_step;
+                if (r_u >= cpp) {
+                    r_u -= cpp;
+                    ++it_u;
+                }
             } else {
                 it = pos / c.page_size;
-                entry = pos - it * c.page_size;
+                entry[u] = pos - it * c.page_size;
             }
-            ok[u] = pos < seq_len && it < npages;
-            int64_t page = ok[u] ? c.indices[p0 + it] : 0;
-            ok[u] = ok[u] && page >= 0 && page < c.num_pages;
-            page = ok[u] ? page : 0;
-            entry = ok[u] ? entry : 0;
-            const int64_t ks = paged_slot(c, page, 0, h, entry), vs = paged_slot(c, page, 1, h, entry);
-            kw[u] = __builtin_nontemporal_load((const u32x4*)c.data + ks * 4 + c4);
-            vw[u] = __builtin_nontemporal_load((const u32x4*)c.data + vs * 4 + c4);
-            kp[u] = c.param[ks];
-            vp[u] = c.param[vs];
+            t.ok[u] = pos < seq_len && it < npages;
+            const int32_t* pp = c.indices + p0 + (it < npages ? it : 0);
+            if (ALIGNED) {
+                // a scalar load, spelled out: behind the scheduling barriers of the loop the compiler falls back
+                // to a vector load plus a wait for EVERY outstanding vector load, which would drain the pipeline
+                int pg;
+                asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(pg) : "s"(pp) : "memory");
+                page[u] = pg;
+            } else {
+                page[u] = *pp;
+            }
         }
+#pragma unroll
+        for (int u = 0; u < AU; ++u) {
+            const bool page_ok = page[u] >= 0 && page[u] < c.num_pages;
+            t.ok[u] = t.ok[u] && page_ok;
+            // the page part of the address is wave-uniform when ALIGNED (scalar base, 32-bit lane offsets)
+            const int64_t kbase = (page_ok ? page[u] : 0) * page_slots + head_slots;
+            const u32 e = t.ok[u] ? (u32)entry[u] : 0u;
+            const uint8_t* kd = c.data + kbase * 64;
+            const uint8_t* vd = c.data + (kbase + kv_slots) * 64;
+            t.kw[u] = __builtin_nontemporal_load((const u32x4*)(kd + (e * 64u + (u32)c4 * 16u)));
+            t.vw[u] = __builtin_nontemporal_load((const u32x4*)(vd + (e * 64u + (u32)c4 * 16u)));
+            t.kp[u] = *(const u32*)((const uint8_t*)(c.param + kbase) + e * 4u);
+            t.vp[u] = *(const u32*)((const uint8_t*)(c.param + kbase + kv_slots) + e * 4u);
+        }
+    };
+    auto consume = [&](const Step& t) {
         float lg[AU], mx = m;
 #pragma unroll
         for (int u = 0; u < AU; ++u) {
+            // q . (bias + codes) with fp32 accumulation of exact products, minus sum(q * bias)
             float a0 = 0.f, a1 = 0.f;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32 lo = kw[u][j] & 0x0F0F0F0Fu, hi = kw[u][j] & 0xF0F0F0F0u;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    a0 = __builtin_fmaf(qlo[j][k], byte_f32(lo, k), a0);
-                    a1 = __builtin_fmaf(qhi[j][k], byte_f32(hi, k), a1);
-                }
+                const CodePairs cp = code_pairs(t.kw[u][j], mask_lo, bias_lo, mask_hi, bias_hi);
+                a0 = __builtin_amdgcn_fdot2(qp[j][0], as_f16x2(cp.p[0]), a0, false);
+                a1 = __builtin_amdgcn_fdot2(qp[j][1], as_f16x2(cp.p[1]), a1, false);
+                a0 = __builtin_amdgcn_fdot2(qp[j][2], as_f16x2(cp.p[2]), a0, false);
+                a1 = __builtin_amdgcn_fdot2(qp[j][3], as_f16x2(cp.p[3]), a1, false);
             }
-            const float dot = quad_sum(a0 + a1);
-            const f16x2 prm = as_f16x2(kp[u]);
+            const float dot = quad_sum((a0 + a1) - qbias);
+            const f16x2 prm = as_f16x2(t.kp[u]);
             const float x = (dot * (float)prm[0] - (float)prm[1] * qs) * sm_scale_log2;
-            lg[u] = ok[u] ? x : -__builtin_inff();
+            lg[u] = t.ok[u] ? x : -__builtin_inff();
             mx = __builtin_fmaxf(mx, lg[u]);
         }
         const float alpha = __builtin_amdgcn_exp2f(m - mx);
         m = mx;
         d *= alpha;
         pz *= alpha;
+        psum *= alpha;
 #pragma unroll
         for (int i = 0; i < 32; ++i) acc[i] *= alpha;
 #pragma unroll
         for (int u = 0; u < AU; ++u) {
             const float p = __builtin_amdgcn_exp2f(lg[u] - m);
-            const f16x2 prm = as_f16x2(vp[u]);
-            const float ps = p * (float)prm[0], ps16 = ps * 0.0625f;
+            const f16x2 prm = as_f16x2(t.vp[u]);
+            const float ps = p * (float)prm[0];
             d += p;
             pz = __builtin_fmaf(p, (float)prm[1], pz);
+            psum += ps;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32 lo = vw[u][j] & 0x0F0F0F0Fu, hi = vw[u][j] & 0xF0F0F0F0u;
+                const CodePairs cp = code_pairs(t.vw[u][j], mask_lo, bias_lo, mask_hi, bias_hi);
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    acc[8 * j + 2 * k] = __builtin_fmaf(ps, byte_f32(lo, k), acc[8 * j + 2 * k]);
-                    acc[8 * j + 2 * k + 1] = __builtin_fmaf(ps16, byte_f32(hi, k), acc[8 * j + 2 * k + 1]);
+                for (int i = 0; i < 4; ++i) {
+                    const f16x2 pr = as_f16x2(cp.p[i]);
+                    acc[8 * j + i] = __builtin_fmaf(ps, (float)pr[0], acc[8 * j + i]);
+                    acc[8 * j + i + 4] = __builtin_fmaf(ps, (float)pr[1], acc[8 * j + i + 4]);
                 }
             }
         }
+    };
+    Step sa, sb;
+    const int gs = stride * AU;
+    issue(sa, g);
+    for (; g < chunks; g += 2 * gs) {
+        issue(sb, g + gs);
+        __builtin_amdgcn_sched_barrier(0);                 // the compiler would otherwise sink the loads below the arithmetic
+        consume(sa);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(sa, g + 2 * gs);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g + gs < chunks) consume(sb);                  // (no loads inside: the branch does not disturb the wait counts)
+        __builtin_amdgcn_sched_barrier(0);
     }
-    // ---- merge the 64 lane-group states of the workgroup
-    float* mine = st + ((wave * 16 + slot) * 4 + c4) * 36;
-    mine[0] = m;
-    mine[1] = d;
+    // ---- merge: first the four lane groups of each row of 16 lanes (two DPP rotations: every lane ends
+    // with its row's state), then the NW * 4 row states of the workgroup through LDS
 #pragma unroll
-    for (int i = 0; i < 32; ++i) mine[4 + i] = acc[i] - pz;          // sum p (code scale - zero)
+    for (int i = 0; i < 32; ++i) acc[i] -= __builtin_fmaf(psum, (i & 1) ? kBiasOdd : kBiasEven, pz);     // sum p (code scale - zero)
+#pragma unroll
+    for (int step = 0; step < 2; ++step) {
+        const float om = step == 0 ? row_rotate<0x124>(m) : row_rotate<0x128>(m);
+        const float od = step == 0 ? row_rotate<0x124>(d) : row_rotate<0x128>(d);
+        const float M = __builtin_fmaxf(m, om);
+        const float ws = __builtin_amdgcn_exp2f(m - M), wo = __builtin_amdgcn_exp2f(om - M);
+        d = __builtin_fmaf(d, ws, od * wo);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const float oa = step == 0 ? row_rotate<0x124>(acc[i]) : row_rotate<0x128>(acc[i]);
+            acc[i] = __builtin_fmaf(acc[i], ws, oa * wo);
+        }
+        m = M;
+    }
+    if ((lane & 12) == 0) {                                           // the first lane group of every row writes
+        float* mine = st + ((wave * 4 + (lane >> 4)) * 4 + c4) * 36;
+        mine[0] = m;
+        mine[1] = d;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) mine[4 + i] = acc[i];
+    }
+    __syncthreads();
+    // two levels, so that no thread walks more than eight states: thread (part, dimension) merges the row
+    // states part, part + PARTS, ...; then 128 threads merge the PARTS partial results
+    constexpr int PARTS = NW / 2, PER = NW * 4 / PARTS;              // 8 states per thread
+    {
+        const int dim = threadIdx.x & 127, prt = threadIdx.x >> 7, qd = dim >> 5, r = dim & 31;
+        float sm_[PER], sd_[PER], so_[PER], M = -5e4f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const float* src = st + ((prt + k * PARTS) * 4 + qd) * 36;
+            sm_[k] = src[0];
+            sd_[k] = src[1];
+            so_[k] = src[4 + r];
+            M = __builtin_fmaxf(M, sm_[k]);
+        }
+        float D = 0.f, O = 0.f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const float w = __builtin_amdgcn_exp2f(sm_[k] - M);
+            D = __builtin_fmaf(sd_[k], w, D);
+            O = __builtin_fmaf(so_[k], w, O);
+        }
+        float* dst = st2 + (prt * 128 + dim) * 3;
+        dst[0] = M;
+        dst[1] = D;
+        dst[2] = O;
+    }
     __syncthreads();
     if (threadIdx.x < 128) {
-        const int dim = threadIdx.x, qd = dim >> 5, r = dim & 31;
+        const int dim = threadIdx.x;
         float M = -5e4f;
-        for (int s = 0; s < 64; ++s) M = __builtin_fmaxf(M, st[(s * 4 + qd) * 36]);
+#pragma unroll
+        for (int k = 0; k < PARTS; ++k) M = __builtin_fmaxf(M, st2[(k * 128 + dim) * 3]);
         float D = 0.f, O = 0.f;
-        for (int s = 0; s < 64; ++s) {
-            const float* src = st + (s * 4 + qd) * 36;
+#pragma unroll
+        for (int k = 0; k < PARTS; ++k) {
+            const float* src = st2 + (k * 128 + dim) * 3;
             const float w = __builtin_amdgcn_exp2f(src[0] - M);
             D = __builtin_fmaf(src[1], w, D);
-            O = __builtin_fmaf(src[4 + r], w, O);
+            O = __builtin_fmaf(src[2], w, O);
         }
         if (splits == 1) {
             o[(int64_t)bh * 128 + dim] = (f16)(O / D);     // an empty sequence gives 0 / 0, as the reference's kernel does
@@ -274,21 +421,28 @@ extern "C" int qr_kv_append_i4(void* kv_data, void* kv_param, const void* kv_ind
 }
 
 namespace {
-// Parts per (sequence, head): enough workgroups to fill the GPU four deep, each with at least 256
-// positions, when the caller says how long the sequences can be and provides room for the partial states.
-int decode_splits(int64_t batch_size, int num_heads, int64_t max_seq_len) {
-    if (max_seq_len <= 0) return 1;
+// Waves per (sequence, head): enough to fill the GPU's 4096 wave slots, each with at least four steps of 16
+// positions when the caller says how long the sequences can be.  Up to 16 of them form one workgroup;
+// beyond that the sequence is split over several workgroups, which needs room for their partial states.
+struct DecodePlan {
+    int nw, splits;
+};
+DecodePlan decode_plan(int64_t batch_size, int num_heads, int64_t max_seq_len) {
     const int64_t bh = batch_size * num_heads;
-    int64_t s = (1024 + bh - 1) / bh, cap = max_seq_len / 256;
-    s = s > cap ? cap : s;
-    s = s > 64 ? 64 : s;
-    return s < 1 ? 1 : (int)s;
+    if (max_seq_len <= 0) return DecodePlan{bh >= 1024 ? 4 : bh >= 256 ? 8 : 16, 1};
+    const int64_t chunks = (max_seq_len + 15) / 16;
+    int64_t wp = (4096 + bh - 1) / bh, cap = chunks / 4;
+    wp = wp > cap ? cap : wp;
+    if (wp <= 4) return DecodePlan{4, 1};
+    if (wp <= 16) return DecodePlan{8, 1};                  // (measured a few percent ahead of 16 waves at 256 (sequence, head) pairs)
+    int64_t s = (wp + 15) / 16;
+    return DecodePlan{16, (int)(s > 16 ? 16 : s)};
 }
 }  // namespace
 
 extern "C" size_t qr_batch_decode_workspace_bytes(int64_t batch_size, int num_heads, int64_t max_seq_len) {
     if (batch_size <= 0 || num_heads <= 0) return 0;
-    const int s = decode_splits(batch_size, num_heads, max_seq_len);
+    const int s = decode_plan(batch_size, num_heads, max_seq_len).splits;
     return s > 1 ? (size_t)batch_size * num_heads * s * 132 * sizeof(float) : 0;
 }
 
@@ -305,17 +459,27 @@ extern "C" int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, c
     if (batch_size * num_heads > 0x3fffffff / 64) return QR_E_SHAPE;
     const PagedKV c = qr_internal_paged_kv((void*)kv_data, (void*)kv_param, kv_indptr, kv_indices, last_page_offset, num_pages,
                                            num_layers, layer_idx, num_heads, page_size, batch_size);
-    int splits = decode_splits(batch_size, num_heads, max_seq_len);
+    DecodePlan plan = decode_plan(batch_size, num_heads, max_seq_len);
+    int splits = plan.splits;
     if (splits > 1 && (!workspace || ((uintptr_t)workspace & 15) ||
                        workspace_bytes < (size_t)batch_size * num_heads * splits * 132 * sizeof(float)))
         splits = 1;                                        // no room for partial states: one workgroup per (sequence, head)
     const float sm = (float)(1.4426950408889634 / __builtin_sqrt((double)head_dim));
     const unsigned grid = (unsigned)(batch_size * num_heads * splits);
     hipStream_t st = (hipStream_t)stream;
-    if (page_size % 16 == 0)
-        paged_decode_i4_kernel<true><<<dim3(grid), dim3(AT), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits, (float*)workspace);
-    else
-        paged_decode_i4_kernel<false><<<dim3(grid), dim3(AT), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits, (float*)workspace);
+#define QR_DECODE(AL, NWV)                                                                                              \
+    paged_decode_i4_kernel<AL, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits,      \
+                                                                          (float*)workspace)
+    if (page_size % 16 == 0) {
+        if (plan.nw == 16) QR_DECODE(true, 16);
+        else if (plan.nw == 8) QR_DECODE(true, 8);
+        else QR_DECODE(true, 4);
+    } else {
+        if (plan.nw == 16) QR_DECODE(false, 16);
+        else if (plan.nw == 8) QR_DECODE(false, 8);
+        else QR_DECODE(false, 4);
+    }
+#undef QR_DECODE
     int lrc = qr_launch_status();
     if (lrc != QR_OK || splits == 1) return lrc;
     paged_decode_merge_kernel<<<dim3((unsigned)(batch_size * num_heads)), dim3(128), 0, st>>>((const float*)workspace, splits,

@@ -301,10 +301,26 @@ class MultiLayerPagedKVCache4Bit:
     def get_cache_specs_for_flash_infer(self, attention_mask):
         """Page tables of the current state (kv_cache.py:253-275): page i of sequence b is page number
         i * batch_size + b; every sequence must span the same number of pages."""
-        if attention_mask is not None:
-            seqlens_in_batch = attention_mask.sum(dim=-1, dtype=torch.int32)
-        else:
-            seqlens_in_batch = torch.tensor([self.length], dtype=torch.int32, device=self.device).expand(self.batch_size)
+        if attention_mask is None:
+            # every sequence holds self.length tokens: the tables depend on that number alone and are built
+            # once per length (every layer of a decode step asks for them), with host arithmetic
+            cached = getattr(self, "_specs", None)
+            if cached is not None and cached[0] == self.length:
+                return cached[1]
+            page_cnt = self.page_cnt_from_length(self.length)
+            ptr = self.length % self.page_size
+            ptr = self.page_size if (self.length != 0 and ptr == 0) else ptr
+            arange = functools.partial(torch.arange, device=self.device, dtype=torch.int32)
+            specs = {
+                "kv_data": self.pages,
+                "kv_indptr": arange(0, self.batch_size + 1) * page_cnt,
+                "kv_indices": (arange(page_cnt).unsqueeze(0) * self.batch_size + arange(self.batch_size).unsqueeze(1)).reshape(-1),
+                "last_page_offset": torch.full((self.batch_size,), ptr, dtype=torch.int32, device=self.device),
+                "kv_param": self.scales,
+            }
+            self._specs = (self.length, specs)
+            return specs
+        seqlens_in_batch = attention_mask.sum(dim=-1, dtype=torch.int32)
         page_cnt = self.page_cnt_from_length(seqlens_in_batch)
         if (page_cnt[0] != page_cnt).any():
             raise NotImplementedError("Current implementation does not support the case where batches have different number of pages")
