@@ -32,9 +32,9 @@ HBM rather than from the 256 MB last-level cache.
 Timing follows benchmarks/qlinear_benchmark.py:20-40,88-113: warm-up, then a loop of K steps between two
 synchronisations, repeated R times; the step time is the median of the R loops and the spread is
 reported as mean +- 1.96 sigma.  Nothing but the step's own launches is inside a timed loop; the time
-of each kernel comes from a separate pass: launches of that kernel alone, each between two HIP events
-on the launch stream, queued behind a few milliseconds of device copies so that the host's per-call
-cost (longer than the short kernels) does not show.
+of each kernel comes from a separate pass: back-to-back launches of that kernel alone between one pair
+of HIP events on the launch stream, queued behind a few milliseconds of device copies so that the
+host's per-call cost (longer than the short kernels) does not show.
 
 Prints ONE JSON line on stdout.  The default run measures the headline workload (c2) and, in
 `per_config`, every other benchmark configuration with fewer repeats.
@@ -156,24 +156,24 @@ _BLOCKER = {}
 
 
 def kernel_ms(fn, reps):
-    """Average duration of one launch of fn(), HIP events on the launch stream around every launch.  The
-    host needs longer to issue a launch than a short kernel runs, and an event recorded on an idle GPU
-    would time that host latency: a few milliseconds of device copies are queued first, so that every
-    event and launch of the pass is already waiting in the stream when the GPU reaches it."""
+    """Average duration of one launch of fn(): `reps` back-to-back launches between one pair of HIP events
+    on the launch stream.  The host needs longer to issue a launch than a short kernel runs, and an idle
+    GPU would then time the host: a few milliseconds of device copies are queued first, so that the events
+    and every launch are already waiting in the stream when the GPU reaches them."""
     if "src" not in _BLOCKER:
         _BLOCKER["src"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
         _BLOCKER["dst"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
     fn()
-    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    for _ in range(max(2, reps // 16)):                      # ~1.6 ms each
+    for _ in range(max(2, reps // 12)):                      # ~1.6 ms each
         _BLOCKER["dst"].copy_(_BLOCKER["src"])
-    for a, b in pairs:
-        a.record()
+    e0.record()
+    for _ in range(reps):
         fn()
-        b.record()
+    e1.record()
     torch.cuda.synchronize()
-    return float(np.mean([a.elapsed_time(b) for a, b in pairs]))
+    return e0.elapsed_time(e1) / reps
 
 
 def gemm_kernel_name(m, n):
@@ -594,7 +594,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": res["workload"], "launch": res.get("launch", "eager"),
                    "timing": "median of `repeats` loops of `steps` steps, each loop between two synchronisations; kernel times from a "
-                             "separate pass of that kernel alone, HIP events around every launch on the launch stream"},
+                             "separate pass of back-to-back launches of that kernel alone between two HIP events on the launch stream"},
         "roofline": roof,
     }
     for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms"):
