@@ -867,6 +867,9 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 #pragma unroll
             for (int c = 0; c < 2; ++c) xr[i][c] = *((const u32x4*)src + goff[i][c]);
     };
+    u32 amask[TPW];                                          // magnitude bits of this lane's output row in tile i, 0 beyond K
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) amask[i] = (wave + 4 * i) * 16 + l16 < K ? 0x7fff7fffu : 0u;
 
     int64_t row = blockIdx.x;
     if (row < rows) load_row(x + row * (int64_t)n);
@@ -957,8 +960,9 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
                 o[1] = narrow_f16x2(acc[i][2], acc[i][3]);
                 *(u32x2*)(ybase + i * 64 * YS + ct * 16) = o;
                 if (QUANT) {
-                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & 0x7fff7fffu));
-                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[1] & 0x7fff7fffu));
+                    // rows beyond K do not exist: they are zero except when the row holds an infinity (0 . inf)
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & amask[i]));
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[1] & amask[i]));
                 }
             }
         }
@@ -1031,6 +1035,278 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
     }
 }
 
+// ---- K > 1, m = 64, fp16 staging, quantiser fused, no copy of the transformed row: the lean form ---
+// The same two matrix-core stages and the same arithmetic as hadamard_m64_kernel (identical fragments
+// and accumulation order, so codes and scales are identical bit for bit), with two of its three trips
+// through LDS removed:
+//   * stage 1 takes its A fragments straight from global memory: lane (row l16 of a 16-row tile, g) loads
+//     the 16 bytes k = 8 g .. 8 g + 7 of its row for each of the two k steps: 64 consecutive bytes per
+//     row and instruction, both halves of every 128-byte row within one pair of loads;
+//   * the fp16 results of stage 2 stay in registers (a lane holds, for ONE output row k', the four
+//     columns 16 ct + 4 g .. + 3 of every column tile ct) until the row maximum is known; the codes are
+//     then formed in registers and four-lane groups exchange their 16-bit pieces (v_permlane32_swap,
+//     v_permlane16_swap, byte permutes: a 4 x 4 transpose of pieces across the lanes l16 + 16 g) so
+//     that every lane stores 8 contiguous bytes and a wave 32 contiguous bytes per output row.
+// Only T (stage 1's output, read by every wave in stage 2) lives in LDS: 4 KB per 32 hadK columns.
+template <int KS2>
+__global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
+                                                             const f16* __restrict__ hadK, float scale, float clip,
+                                                             u32* __restrict__ q, f16* __restrict__ scales) {
+    constexpr int CT = 4;
+    constexpr int NT = 2 * KS2;
+    constexpr int TPW = (NT + 3) / 4;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[HT / QR_WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int nchunks = n >> 3;
+    u32x2* Tl = (u32x2*)smem_raw;                                      // [CT][NT][64 lanes]
+    for (int i = tid; i < CT * NT * 32; i += HT) ((u32x4*)Tl)[i] = u32x4{0, 0, 0, 0};
+
+    f16x8 hf[TPW][KS2];
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+        const int hr = (wave + 4 * t) * 16 + l16;
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int hc = ks * 32 + hh * 16 + g * 4;
+                // unconditional loads (a clamped address, then a select): all of them are in flight
+                // together; a branch around each would serialise 12 KS2 round trips through the cache
+                const bool ok = hr < K && hc < K;
+                f16x4 v = *(const f16x4*)(hadK + (ok ? hr * K + hc : 0));
+                if (!ok) v = f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hf[t][ks][hh * 4 + e] = v[e];
+            }
+    }
+    f16x8 sb[2][2];                                          // Sylvester fragments, as in hadamard_m64_kernel
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool neg = ((__builtin_popcount(((g & 1) * 8 + j) & l16) + ((g >> 1) & o)) & 1) != 0;
+            sb[o][0][j] = neg ? (f16)-1.0f : (f16)1.0f;
+            sb[o][1][j] = neg ? (f16)1.0f : (f16)-1.0f;
+        }
+    // fragment (tile i, k step c) of a row: 16-byte piece 4 c + g of row (wave + 4 i) 16 + l16 of X[K][64]
+    int goff[TPW][2];
+    bool dval[TPW];
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+        const int r = (wave + 4 * i) * 16 + l16;
+        dval[i] = r < K;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) goff[i][c] = dval[i] ? r * 8 + 4 * c + g : 0;
+    }
+    u32x4 xr[TPW][2];
+    auto load_row = [&](const f16* src) {
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) xr[i][c] = *((const u32x4*)src + goff[i][c]);
+    };
+    u32 amask[TPW];                                          // magnitude bits of this lane's output row in tile i, 0 beyond K:
+#pragma unroll                                               // those rows are zero except when the row holds an infinity (0 . inf)
+    for (int i = 0; i < TPW; ++i) amask[i] = dval[i] ? 0x7fff7fffu : 0u;
+    int64_t row = blockIdx.x;
+    if (row < rows) load_row(x + row * (int64_t)n);
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks) asm volatile("" : "+v"(hf[t][ks]));
+    __syncthreads();
+    // The quantiser of row r is ~250 vector instructions per lane, the hadK stage of row r + 1 is 12 KS2
+    // matrix instructions of 16 cycles each whose issue slots are otherwise empty: the two are interleaved
+    // in program order (three matrix instructions, then one pair of the previous row's values), pinned by
+    // scheduling barriers, so that the vector and matrix pipes overlap by construction rather than by
+    // the chance phase of the two workgroups that share a SIMD.
+    u32x2 yp[TPW][CT];                                       // previous row's fp16 results (the same lane layout)
+    u32 pb[TPW][CT][2];                                      // ... its codes as fp16 1536 + code pairs
+    // Before the first row there is no previous one: the turn then "finishes" zeros with scale 1 into the
+    // first row's own place, which the real codes overwrite a turn later (same lanes, same addresses, in
+    // order).  Every turn thus issues the same memory operations, branch-free.
+    FastRecip fqp = make_fast_recip(1.0f);
+    float sp = 1.0f;
+    u32 mxp = 0x3c00u;
+    int64_t prow = blockIdx.x;
+#pragma unroll
+    for (int i = 0; i < TPW; ++i)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) yp[i][ct] = u32x2{0, 0};
+    // One register pair of the previous row in three parts of two or three vector instructions (the
+    // arithmetic of sym_codes8_fast): each part goes behind one matrix instruction, whose 16 cycles leave
+    // room for about three vector instructions of the same wave.
+    float qa0 = 0.f, qa1 = 0.f;
+    auto quant_part = [&](int p, int part) {
+        const int i = p / (2 * CT), ct = (p / 2) % CT, w = p & 1;
+        if (part == 0) {
+            const f16x2 h2 = as_f16x2(yp[i][ct][w]);
+            qa0 = __builtin_fmaf((float)h2[0], fqp.rh, 0.0f);
+            qa1 = __builtin_fmaf((float)h2[1], fqp.rh, 0.0f);
+        } else if (part == 1) {
+            const f16x2 h2 = as_f16x2(yp[i][ct][w]);
+            qa0 = __builtin_fmaf((float)h2[0], fqp.rl, qa0);
+            qa1 = __builtin_fmaf((float)h2[1], fqp.rl, qa1);
+            qa0 = __builtin_amdgcn_fmed3f(qa0, -8.0f, 7.0f);
+        } else {
+            qa1 = __builtin_amdgcn_fmed3f(qa1, -8.0f, 7.0f);
+            f16x2 h = {(f16)qa0, (f16)qa1};
+            h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
+            pb[i][ct][w] = __builtin_bit_cast(u32, h);
+        }
+    };
+    auto quant_pair = [&](int p) {
+        quant_part(p, 0);
+        quant_part(p, 1);
+        quant_part(p, 2);
+    };
+    auto finish_prev = [&](bool fast) {                      // pack, exchange pieces between lanes, store
+        u32 c01[TPW], c23[TPW];
+        if (fast) {
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                const u32 b0[4] = {pb[i][0][0], pb[i][0][1], pb[i][1][0], pb[i][1][1]};
+                const u32 b1[4] = {pb[i][2][0], pb[i][2][1], pb[i][3][0], pb[i][3][1]};
+                c01[i] = pack_nibbles8(b0);
+                c23[i] = pack_nibbles8(b1);
+            }
+        } else {
+            const bool fs = scale_fast_ok(sp);
+            const float rs = fs ? 1.0f / sp : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                c01[i] = sym_codes8(u32x4{yp[i][0][0], yp[i][0][1], yp[i][1][0], yp[i][1][1]}, sp, rs, fs);
+                c23[i] = sym_codes8(u32x4{yp[i][2][0], yp[i][2][1], yp[i][3][0], yp[i][3][1]}, sp, rs, fs);
+            }
+        }
+        u32x2* qrow = (u32x2*)(q + prow * (int64_t)nchunks);
+        u32x2 outv[TPW];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            // lanes l16 + 16 g: piece (g, ct) -> lane ct.  First the halves of the wave (g and g ^ 2) ...
+            const auto s1 = __builtin_amdgcn_permlane32_swap(c01[i], c23[i], false, false);
+            const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);     // the even column tile of this lane's pair
+            const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);     // the odd one
+            // ... then neighbouring rows of 16 lanes (g and g ^ 1)
+            const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
+            const u32 lo = __builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u);     // pieces of g = 0, 1
+            const u32 hi = __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u);     // pieces of g = 2, 3
+            outv[i] = u32x2{lo, hi};
+        }
+        // lanes on rows beyond K store their first tile's piece once more (K >= 64: that row exists)
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int kp = (wave + 4 * i) * 16 + l16;
+            const bool ok = kp < K;
+            qrow[(ok ? kp : wave * 16 + l16) * 4 + g] = ok ? outv[i] : outv[0];
+        }
+    };
+    for (; row < rows; row += gridDim.x) {
+        const int64_t nrow = row + gridDim.x;
+        // ---- stage 1: T = X . H_64 for this wave's tiles (rows beyond K are zero fragments)
+        u32x4 af[TPW][2];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) af[i][c] = dval[i] ? xr[i][c] : u32x4{0, 0, 0, 0};
+        // (unconditional, like every store below: with a fixed number of memory operations per turn the wait
+        // for these loads, a turn later, need not include the stores issued after them; the last turn re-reads
+        // its own row)
+        load_row(x + (nrow < rows ? nrow : row) * (int64_t)n);
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int t = wave + 4 * i;
+            if (4 * i + 3 < NT || t < NT) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][0]), sb[ct & 1][0], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][1]), sb[ct & 1][ct >> 1], acc, 0, 0, 0);
+                    u32x2 hi;
+                    hi[0] = narrow_f16x2(acc[0] * scale, acc[1] * scale);
+                    hi[1] = narrow_f16x2(acc[2] * scale, acc[3] * scale);
+                    Tl[(ct * NT + t) * 64 + lane] = hi;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- stage 2: Y^T = T^T . hadK^T; results stay in registers.  Between the matrix instructions: the
+        // previous row's quantiser (when that row takes the lean path; else it is finished afterwards)
+        const bool pfast = fast_quant_ok(mxp, sp);
+        u16x2 mx2 = {0, 0};
+        u32x2 yv[TPW][CT];
+        u32x4 th[2][KS2];
+        auto fetch = [&](int ct, int b) {
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                const u32x2 p0 = Tl[(ct * NT + 2 * ks) * 64 + lane], p1 = Tl[(ct * NT + 2 * ks + 1) * 64 + lane];
+                th[b][ks] = u32x4{p0[0], p0[1], p1[0], p1[1]};
+            }
+        };
+        fetch(0, 0);
+        constexpr int PAIRS = TPW * CT * 2, GROUPS = CT * KS2;      // 24 pairs over 24 groups when KS2 = 6
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ct + 1 < CT) fetch(ct + 1, (ct + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x4 acc[TPW];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                const int grp = ct * KS2 + ks;
+                // pairs grp * PAIRS / GROUPS .. (grp + 1) * PAIRS / GROUPS - 1 of the previous row, their parts
+                // spread over the group's matrix instructions
+                const int p0 = grp * PAIRS / GROUPS, p1 = (grp + 1) * PAIRS / GROUPS, parts = (p1 - p0) * 3;
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, th[ct & 1][ks]), hf[i][ks], acc[i], 0, 0, 0);
+#pragma unroll
+                    for (int e = i * parts / TPW; e < (i + 1) * parts / TPW; ++e) quant_part(p0 + e / 3, e % 3);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                yv[i][ct][0] = narrow_f16x2(acc[i][0], acc[i][1]);
+                yv[i][ct][1] = narrow_f16x2(acc[i][2], acc[i][3]);
+                mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, yv[i][ct][0] & amask[i]));
+                mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, yv[i][ct][1] & amask[i]));
+            }
+        }
+        finish_prev(pfast);
+        // ---- this row's maximum and scale; its codes are formed during the next row's stage 2
+        u32 mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+        mx = wave_max_u32_dpp(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+        const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+        scales[row] = sh;                                     // every lane, the same value: no branch around the store
+        sp = (float)sh;
+        mxp = mx;
+        prow = row;
+        fqp = fast_quant_ok(mx, sp) ? make_fast_recip(sp) : FastRecip{0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) yp[i][ct] = yv[i][ct];
+        // Tl is next written after this row's second barrier, which every wave reaches only after its
+        // stage-2 reads; red[] is next written after the next row's first barrier
+    }
+    if ((int64_t)blockIdx.x < rows) {                        // the last row's codes
+        const bool pfast = fast_quant_ok(mxp, sp);
+        if (pfast) {
+#pragma unroll
+            for (int pq = 0; pq < TPW * CT * 2; ++pq) quant_pair(pq);
+        }
+        finish_prev(pfast);
+    }
+}
+
 // A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
 // kernel applies with a generated outer factor, in its fp32-precision mode so that the result is
 // rounded to fp16 once, like a plain fp32 transform.  Returns the outer order (0: not applicable).
@@ -1055,6 +1331,28 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
         const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
+        if (!MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
+            // fused, fp16 staging, no copy of the transformed rows wanted: the lean kernel (T alone in LDS)
+            const size_t ldsq = (size_t)4096 * KS2;
+#define QR_M64Q(KS)                                                                                                    \
+    do {                                                                                                               \
+        auto kern = hadamard_m64q_kernel<KS>;                                                                          \
+        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, ldsq);                                     \
+        const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
+        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \
+                                                 (f16*)scales);                                                        \
+    } while (0)
+            // (orders of 64 and more among the reference's tables: 108, 140, 156, 172)
+            if (KS2 >= 4) {
+                switch (KS2) {
+                    case 4: QR_M64Q(4); break;
+                    case 5: QR_M64Q(5); break;
+                    default: QR_M64Q(6); break;
+                }
+                return qr_launch_status();
+            }
+#undef QR_M64Q
+        }
         if (lds64 <= 80 * 1024) {
 #define QR_M64(KS)                                                                                                     \
     do {                                                                                                               \

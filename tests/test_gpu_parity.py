@@ -395,6 +395,39 @@ def test_fused_hadamard_quantize_equals_staged(n, fp32):
     assert close(y2.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
 
 
+@pytest.mark.parametrize("n", [11008, 8960, 6912])
+def test_fused_hadamard_quantize_lean_kernel_rows_of_every_kind(n):
+    """Without the copy of the transformed rows the m = 64 widths take a kernel of their own (results of
+    the hadK stage kept in registers, the previous row quantised between the next row's matrix
+    instructions, every workgroup walking several rows): more rows than workgroups, and rows holding an
+    infinity, a NaN, only zeros, huge and tiny values (the quantiser's slow path) next to ordinary ones.
+    Codes and scales must equal those of the kernel that also returns the rows, whose codes are checked
+    against the oracle on exactly those rows."""
+    rows = 1500
+    x = synth_x(rows, n, seed=n + 7)
+    x[3, 17] = np.inf
+    x[700, 5] = np.nan
+    x[701] = 0
+    x[1499] = 0
+    x[1200, 9] = 60000.0
+    x[44] *= F16(1e-4)
+    x[0, :] = 0
+    xg = gpu(x)
+    mod = quarot_amd.nn.OnlineHadamardQuantizer(n, input_clip_ratio=0.9).cuda()
+    p = mod(xg)
+    p2, y = quarot_amd.hadamard_quantize(xg, mod.had_rem_dim, mod.rem_dim, 0.9, return_transformed=True)
+    assert torch.equal(p.quantized_x, p2.quantized_x)
+    assert np.array_equal(bits(p.scales_x.cpu().numpy()), bits(p2.scales_x.cpu().numpy()))
+    with np.errstate(all="ignore"):
+        wq, ws = o.quantizer(y.cpu().numpy(), 0.9)
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    got_s = p.scales_x.cpu().numpy().reshape(-1)
+    nan = np.isnan(ws)                                             # (a NaN scale may carry any payload bits)
+    assert np.array_equal(np.isnan(got_s), nan) and np.array_equal(bits(got_s[~nan]), bits(ws[~nan]))
+    one = mod(xg[5:6])                                             # a single row: the first turn is also the last
+    assert torch.equal(one.quantized_x, p.quantized_x[5:6])
+
+
 @pytest.mark.parametrize("shape", [(5, 64), (9, 4096), (7, 5120), (3, 8192), (4, 11008), (2, 32768), (6, 24), (3, 100)])
 @pytest.mark.parametrize("clip", [1.0, 0.9])
 def test_fused_rmsnorm_quantize(shape, clip):
