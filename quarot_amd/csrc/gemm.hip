@@ -22,6 +22,7 @@
 // two K-groups take alternate 64-k sub-steps of every stage and exchange half of their accumulators
 // through LDS at the end.
 #include "qr_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -352,7 +353,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
 // 0), global loads run one more stage ahead through registers, one barrier per stage.
 // (A variant in which half the waves only unpacked into int8 planes in LDS for the other half was
 // measured LDS-bound: twice the LDS bytes at ~128 B/clk/CU exceed the MFMA time.)
-template <int BM, int BN, int WAVES_M, int WAVES_N, int RD, bool DEQ>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
 __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
@@ -424,7 +425,6 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             if (i * 64 < BM) r[i] = *(const u32x4*)(A + (size_t)(goff[i] + off));
-            else if (RD > 1) r[i] = __builtin_nontemporal_load((const u32x4*)(B + (size_t)(goff[i] + off)));
             else r[i] = *(const u32x4*)(B + (size_t)(goff[i] + off));
         }
     };
@@ -439,16 +439,6 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
             for (int i = 0; i < NL; ++i) base[i * 64 * 8] = r[i];
         }
     };
-    // the register ring's form writes stages past the end too (they repeat the last stage into a
-    // buffer nobody reads again): without a branch every wait counts exactly the loads issued after
-    // the ones it needs, with one the compiler waits for all outstanding loads
-    auto deposit_always = [&](int st, int buf, u32x4(&r)[NL]) {
-        const bool zero = ragged && (s_first + st) * 128 + scoff >= Kb;
-        u32x4* base = ks_lds + buf * CH + dst0;
-#pragma unroll
-        for (int i = 0; i < NL; ++i) base[i * 64 * 8] = zero ? u32x4{0, 0, 0, 0} : r[i];
-    };
-
     i32x16 acc[IM][JN];
 #pragma unroll
     for (int i = 0; i < IM; ++i)
@@ -500,82 +490,39 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 
     Ops ops;
     int bcur = 0;
-    if constexpr (RD == 1) {
-        // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during
-        // iteration ks from registers requested at the end of iteration ks-1.  The first three stages
-        // are requested together: the accumulators are not live yet, so two more register sets are
-        // free, and the prologue costs one memory round trip instead of three.
-        u32x4 regs[NL];
-        {
-            u32x4 first[NL], second[NL];
-            fetch(0, first);
-            fetch(1, second);
-            fetch(2, regs);
-            deposit(0, 0, first);
-            deposit(1, 1, second);
+    // Global loads run one stage ahead of the LDS fill: stage ks+2 is written to LDS during
+    // iteration ks from registers requested at the end of iteration ks-1.  The first three stages
+    // are requested together: the accumulators are not live yet, so two more register sets are
+    // free, and the prologue costs one memory round trip instead of three.
+    u32x4 regs[NL];
+    {
+        u32x4 first[NL], second[NL];
+        fetch(0, first);
+        fetch(1, second);
+        fetch(2, regs);
+        deposit(0, 0, first);
+        deposit(1, 1, second);
+    }
+    __syncthreads();                                    // stages 0 and 1 visible
+    if (kg == 1) load_ops(0, 0, ops);                   // group 1 starts one unpack ahead
+    for (int ks = 0; ks < stages; ++ks) {
+        const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+        const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
+        if (kg == 0) {
+            load_ops(bcur, 0, ops);
+            multiply(ops);
+            load_ops(bcur, 1, ops);
+            multiply(ops);
+        } else {
+            multiply(ops);                              // sub-step 2 of this stage (unpacked earlier)
+            load_ops(bcur, 1, ops);
+            multiply(ops);                              // sub-step 3
+            if (ks + 1 < stages) load_ops(bnext, 0, ops);   // next stage's sub-step 2
         }
-        __syncthreads();                                    // stages 0 and 1 visible
-        if (kg == 1) load_ops(0, 0, ops);                   // group 1 starts one unpack ahead
-        for (int ks = 0; ks < stages; ++ks) {
-            const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
-            const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
-            if (kg == 0) {
-                load_ops(bcur, 0, ops);
-                multiply(ops);
-                load_ops(bcur, 1, ops);
-                multiply(ops);
-            } else {
-                multiply(ops);                              // sub-step 2 of this stage (unpacked earlier)
-                load_ops(bcur, 1, ops);
-                multiply(ops);                              // sub-step 3
-                if (ks + 1 < stages) load_ops(bnext, 0, ops);   // next stage's sub-step 2
-            }
-            deposit(ks + 2, bfill, regs);
-            fetch(ks + 3, regs);
-            __syncthreads();
-            bcur = bnext;
-        }
-    } else {
-        // Weight streaming (few tokens): an iteration is far shorter than the memory latency, so RD
-        // register sets rotate, set (st % RD) carrying stage st, requested RD iterations before it
-        // is written to LDS.  The first two stages pass through the ring like all others.  Whole
-        // turns of the ring run without a branch around the loads.
-        u32x4 regs[RD][NL];
-#pragma unroll
-        for (int r = 0; r < RD; ++r) fetch(r, regs[r]);
-        deposit_always(0, 0, regs[0]);
-        fetch(RD, regs[0]);
-        deposit_always(1, 1, regs[1 % RD]);
-        fetch(RD + 1, regs[1 % RD]);
-        __syncthreads();                                    // stages 0 and 1 visible
-        if (kg == 1) load_ops(0, 0, ops);                   // group 1 starts one unpack ahead
-        auto iteration = [&](int ks, u32x4(&r)[NL]) {
-            const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
-            const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
-            if (kg == 0) {
-                load_ops(bcur, 0, ops);
-                multiply(ops);
-                load_ops(bcur, 1, ops);
-                multiply(ops);
-            } else {
-                multiply(ops);
-                load_ops(bcur, 1, ops);
-                multiply(ops);
-                if (ks + 1 < stages) load_ops(bnext, 0, ops);
-            }
-            deposit_always(ks + 2, bfill, r);
-            fetch(ks + 2 + RD, r);
-            __syncthreads();
-            bcur = bnext;
-        };
-        int ks0 = 0;
-        for (; ks0 + RD <= stages; ks0 += RD) {
-#pragma unroll
-            for (int r = 0; r < RD; ++r) iteration(ks0 + r, regs[(r + 2) % RD]);
-        }
-#pragma unroll
-        for (int r = 0; r < RD - 1; ++r)
-            if (ks0 + r < stages) iteration(ks0 + r, regs[(r + 2) % RD]);
+        deposit(ks + 2, bfill, regs);
+        fetch(ks + 3, regs);
+        __syncthreads();
+        bcur = bnext;
     }
 
     // K-split: group 0 finalises the lower half of the j tiles and group 1 the upper half; each sends
@@ -716,7 +663,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, int RD = 1>
+template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
               const void* bias, hipStream_t st, int ksplit = 1) {
     constexpr int NT = 128 * WAVES_M * WAVES_N;
@@ -730,13 +677,13 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
     const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
     hipError_t e;
     if (Y) {
-        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, RD, true>;
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, true>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, 1);
     } else {
-        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, RD, false>;
+        auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
@@ -1602,6 +1549,255 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
 }
 
 // ------------------------------------------------------------------------------------------------
+// Decode (M <= 64) with many weight rows: a workgroup of eight waves owns R groups of 32 weight rows
+// (R = 4 .. 8, chosen by the host so that the workgroups spread evenly over the CUs: 57344 rows are
+// 256 workgroups of 7 groups) and walks K in stages of 128 packed bytes per row.
+// * The tokens' codes are fetched ONCE per workgroup and stage and shared through LDS -- with
+//   wave-private staging every wave would pull its own copy through the vector cache, twice the weight
+//   bytes at 64 tokens -- and the thread that fetched a chunk of them stores it already unpacked into
+//   its two int8 planes, so that no wave unpacks tokens.
+// * All 512 threads fetch (eight consecutive threads one 128-byte line) into RD register sets that
+//   rotate RD stages ahead of the LDS fill; three LDS stage buffers rotate; one barrier per stage.
+//   Threads whose chunk index lies beyond the stage repeat their first load into a spare slot.
+// * Wave w < R multiplies row group w against all tokens; waves beyond R only fetch.
+// * Workgroup b starts its walk over K at stage b % stages and wraps around (integer sums do not depend
+//   on the order): with a row pitch that is a power of two, workgroups marching through K in step
+//   would all be reading the same few memory channels at any one time (measured 49 -> 41 us at
+//   57344 x 8192).
+template <int MT, int R, int RD, bool DEQ>
+__global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+                                                        int M, int N, int Kb, int32_t* __restrict__ C,
+                                                        f16* __restrict__ Y, const f16* __restrict__ sA,
+                                                        const f16* __restrict__ sB, const f16* __restrict__ bias) {
+    constexpr int XR = MT * 32;                             // staged rows of X
+    constexpr int ROWS = XR + R * 32;
+    constexpr int NL = (ROWS + 63) / 64;                    // 16-byte chunks per thread and stage: 64 rows each
+    constexpr int XPLANES = XR * 16;                        // slots of the tokens' planes (32 bytes per packed chunk)
+    constexpr int CH = XPLANES + (NL * 64 - XR) * 8;        // slots per stage buffer, spare ones included
+    constexpr int NBUF = 3;
+    extern __shared__ u32x4 xs_lds[];                       // [NBUF][CH]; later the exchange, then the output slabs
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * (R * 32);
+    const int stages = (Kb + 127) / 128;
+    const bool ragged = (Kb & 127) != 0;
+    // weights: chunk position XOR-keyed by the row pair, so that the 16 rows a quarter-wave reads at one
+    // logical chunk cover all sixteen 16-byte bank groups (row parity picks the half)
+    auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
+    // token planes: 16 slots per row; chunk keyed by row & 7, plane by bit 3 of the row
+    auto slot16 = [](int row, int chunk, int plane) {
+        return row * 16 + ((chunk ^ (row & 7)) << 1) + (plane ^ ((row >> 3) & 1));
+    };
+
+    const int srow = tid >> 3, piece = tid & 7;             // chunk i of this thread: row srow + 64 i, same piece
+    const bool xthread = XR == 64 || srow < XR;             // chunk 0 is a row of X (whole waves)
+    const uint8_t* src[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        int row = srow + i * 64;
+        if (row >= ROWS) row = srow;                        // spare slot: repeat the first chunk
+        if (row < XR) {
+            src[i] = A + (int64_t)(row < M ? row : M - 1) * Kb;
+        } else {
+            const int nr = n0 + row - XR;
+            src[i] = B + (int64_t)(nr < N ? nr : N - 1) * Kb;
+        }
+    }
+    const int wdst0 = XPLANES - XR * 8 + slot8(srow, piece);   // rows differ by multiples of 32: same swizzle
+    const int xdst0 = slot16(srow & (XR - 1), piece, 0);
+    const int s0 = blockIdx.x % stages;
+    auto stage_of = [&](int st) {
+        int a = (st < stages ? st : stages - 1) + s0;
+        return a >= stages ? a - stages : a;
+    };
+    auto fetch = [&](int st, u32x4(&v)[NL]) {
+        const int kb = stage_of(st) * 128;
+        const int off = (kb + piece * 16 < Kb) ? kb + piece * 16 : kb;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            // weights are used once: streaming loads keep the tokens' codes, which every workgroup
+            // re-reads, in the caches
+            if (i * 64 >= XR && (i + 1) * 64 <= ROWS) v[i] = __builtin_nontemporal_load((const u32x4*)(src[i] + off));
+            else v[i] = *(const u32x4*)(src[i] + off);
+        }
+    };
+    // stages past the end are written too (into a buffer nobody reads again): without a branch every
+    // wait counts exactly the loads issued after the ones it needs
+    auto deposit = [&](int st, int buf, const u32x4(&v)[NL]) {
+        const bool zero = ragged && stage_of(st) * 128 + piece * 16 >= Kb;
+        u32x4* base = xs_lds + buf * CH;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const u32x4 q = zero ? u32x4{0, 0, 0, 0} : v[i];
+            if (i == 0 && xthread) {
+                base[xdst0] = (q << 4) & 0xF0F0F0F0u;
+                base[xdst0 ^ 1] = q & 0xF0F0F0F0u;
+            } else {
+                base[wdst0 + i * 64 * 8] = q;
+            }
+        }
+    };
+    i32x16 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0;
+    // logical chunk 2u + h of weight row q sits at slot8(q, h) ^ (2u); plane p of a token row's chunk
+    // 2u + h at slot16(q, h, 0) ^ (4u + p): the swizzles only touch the low bits
+    const bool computes = wave < R;
+    const int wslot = XPLANES + slot8((computes ? wave : 0) * 32 + r, h), xslot = slot16(r, h, 0);
+    // The multiplications are software-pipelined over the 64-k sub-steps: while the 2 MT MFMAs of one
+    // sub-step run, the operands of the next one (the first of the next stage after the last: that
+    // buffer became visible with the previous barrier) are read from LDS and the weights unpacked.
+    // Written as slots of one MFMA plus its share of the reads and unpacking, with a scheduling barrier
+    // after every slot: left to itself the compiler reads, unpacks and multiplies in three phases, and
+    // with the two waves of a SIMD in step after every barrier the three pipes then take turns
+    // (measured: LDS, vector and matrix time added up to the whole launch).
+    struct Ops {
+        u32x4 w;
+        i32x4 wlo, whi, xlo[MT], xhi[MT];
+    };
+    Ops ops[2];
+    auto read_w = [&](const u32x4* base, int uu, Ops& o) { o.w = base[wslot ^ (2 * uu)]; };
+    auto read_x = [&](const u32x4* base, int uu, int t, int plane, Ops& o) {
+        const i32x4 q = (i32x4)base[(xslot ^ (4 * uu + plane)) + t * 32 * 16];
+        if (plane) o.xhi[t] = q;
+        else o.xlo[t] = q;
+    };
+    auto unpack_lo = [&](Ops& o) { o.wlo = (i32x4)((o.w << 4) & 0xF0F0F0F0u); };
+    auto unpack_hi = [&](Ops& o) { o.whi = (i32x4)(o.w & 0xF0F0F0F0u); };
+    auto substep = [&](const Ops& cur, Ops& nxt, const u32x4* nbase, int nu) {
+        // slot 0
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.wlo, cur.xlo[0], acc[0], 0, 0, 0);
+        read_w(nbase, nu, nxt);
+        read_x(nbase, nu, 0, 0, nxt);
+        if (MT == 1) read_x(nbase, nu, 0, 1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        if (MT == 2) {
+            acc[MT - 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.wlo, cur.xlo[MT - 1], acc[MT - 1], 0, 0, 0);
+            read_x(nbase, nu, 0, 1, nxt);
+            read_x(nbase, nu, MT - 1, 0, nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.whi, cur.xhi[0], acc[0], 0, 0, 0);
+        if (MT == 2) read_x(nbase, nu, MT - 1, 1, nxt);
+        unpack_lo(nxt);
+        if (MT == 1) unpack_hi(nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        if (MT == 2) {
+            acc[MT - 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.whi, cur.xhi[MT - 1], acc[MT - 1], 0, 0, 0);
+            unpack_hi(nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    u32x4 regs[RD][NL];
+#pragma unroll
+    for (int q = 0; q < RD; ++q) fetch(q, regs[q]);
+    deposit(0, 0, regs[0]);
+    fetch(RD, regs[0]);
+    deposit(1, 1, regs[1 % RD]);
+    fetch(RD + 1, regs[1 % RD]);
+    __syncthreads();                                        // stages 0 and 1 visible
+    if (computes) {
+        read_w(xs_lds, 0, ops[0]);
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            read_x(xs_lds, 0, t, 0, ops[0]);
+            read_x(xs_lds, 0, t, 1, ops[0]);
+        }
+        unpack_lo(ops[0]);
+        unpack_hi(ops[0]);
+    }
+    int bcur = 0;
+    auto iteration = [&](int ks, u32x4(&v)[NL]) {
+        const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+        const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
+        deposit(ks + 2, bfill, v);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(ks + 2 + RD, v);
+        __builtin_amdgcn_sched_barrier(0);
+        if (computes) {
+            const u32x4* cb = xs_lds + bcur * CH;
+            substep(ops[0], ops[1], cb, 1);
+            substep(ops[1], ops[0], cb, 2);
+            substep(ops[0], ops[1], cb, 3);
+            substep(ops[1], ops[0], xs_lds + bnext * CH, 0);   // after the last stage: read, never used
+        }
+        __syncthreads();
+        bcur = bnext;
+    };
+    int ks0 = 0;
+    for (; ks0 + RD <= stages; ks0 += RD) {
+#pragma unroll
+        for (int q = 0; q < RD; ++q) iteration(ks0 + q, regs[(q + 2) % RD]);
+    }
+#pragma unroll
+    for (int q = 0; q < RD - 1; ++q)
+        if (ks0 + q < stages) iteration(ks0 + q, regs[(q + 2) % RD]);
+
+    // ---- epilogue: lane l, register v -> weight row (v/4)*8 + (l/32)*4 + v%4 of the group, token l%32
+    auto finish = [&](const i32x16& a, int g, int t) {
+        const int c0 = n0 + g * 32;
+        const int row = t * 32 + r;
+        const bool by_rows = DEQ && c0 + 32 <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0 && t * 32 + 32 <= M;
+        f16x4 sb4[4], bi4[4];
+        if (DEQ) {
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const int col = c0 + gq * 8 + h * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int cc = col + e < N ? col + e : N - 1;
+                    sb4[gq][e] = sB[cc];
+                    bi4[gq][e] = bias ? bias[cc] : (f16)0;
+                }
+            }
+        }
+        if (DEQ && by_rows) {
+            const f16 sa = sA[row];
+            f16x4 o[1][4];
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq)
+                o[0][gq] = dequant4(a[gq * 4], a[gq * 4 + 1], a[gq * 4 + 2], a[gq * 4 + 3], sa, sb4[gq], bi4[gq], bias != nullptr);
+            store_slab_rows<1>((u32x2*)(xs_lds + wave * 128), o, lane, Y + (int64_t)(t * 32) * N + c0, N);
+            return;
+        }
+        if (row >= M) return;
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            const int col = c0 + gq * 8 + h * 4;
+            if (col >= N) continue;
+            const bool whole = (col + 4 <= N) && ((N & 3) == 0);
+            if (DEQ) {
+                const f16x4 o = dequant4(a[gq * 4], a[gq * 4 + 1], a[gq * 4 + 2], a[gq * 4 + 3], sA[row], sb4[gq], bi4[gq],
+                                         bias != nullptr);
+                f16* yp = Y + (int64_t)row * N + col;
+                if (whole) {
+                    *(f16x4*)yp = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) yp[e] = o[e];
+                }
+            } else {
+                int32_t* cp = C + (int64_t)row * N + col;
+                if (whole) {
+                    *(i32x4*)cp = i32x4{a[gq * 4] >> 8, a[gq * 4 + 1] >> 8, a[gq * 4 + 2] >> 8, a[gq * 4 + 3] >> 8};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) cp[e] = a[gq * 4 + e] >> 8;
+                }
+            }
+        }
+    };
+    if (!computes) return;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) finish(acc[t], wave, t);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Decode with very few tokens (M <= 8): a matrix-vector style kernel on the native int4 dot product
 // (v_dot8_i32_i4: eight signed 4-bit products per lane and instruction, no unpacking).  A wave owns
 // groups of four weight rows and walks K in 1 KB segments: lane l loads bytes [l*16, l*16+16) of
@@ -1851,6 +2047,61 @@ int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, v
     return qr_launch_status();
 }
 
+// Row groups per workgroup for the shared-token decode kernel: the count among 4 .. 8 with the least
+// work on the busiest CU (rounds of 256 workgroups times groups per workgroup), larger counts first
+// (fewer copies of the tokens' codes).  0: too few row groups to fill the CUs this way.
+int decode_xs_groups(int N) {
+    const int groups = (N + 31) / 32;
+    int best = 0, best_cost = 0;
+    for (int rg = 8; rg >= 4; --rg) {
+        const int wgs = (groups + rg - 1) / rg;
+        if (wgs < 192) continue;
+        const int cost = ((wgs + 255) / 256) * rg;
+        if (best == 0 || cost < best_cost) {
+            best = rg;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+int launch_decode_xs(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA,
+                     const void* sB, const void* bias, hipStream_t st, int rg) {
+    const unsigned grid = (unsigned)(((N + 31) / 32 + rg - 1) / rg);
+#define QR_XS(MT, R)                                                                                                  \
+    do {                                                                                                              \
+        constexpr int RD = 3;   /* deeper rings were measured slower (4: +3 %, 5: +6 %) */                            \
+        constexpr size_t LDS = (size_t)3 * (MT * 32 * 16 + ((MT * 32 + R * 32 + 63) / 64 * 64 - MT * 32) * 8) * 16;       \
+        hipError_t e;                                                                                                 \
+        if (Y) {                                                                                                      \
+            auto kern = decode_xs_kernel<MT, R, RD, true>;                                                            \
+            e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
+            if (e != hipSuccess) return (int)e;                                                                       \
+            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, \
+                                                     (const f16*)sA, (const f16*)sB, (const f16*)bias);               \
+        } else {                                                                                                      \
+            auto kern = decode_xs_kernel<MT, R, RD, false>;                                                           \
+            e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
+            if (e != hipSuccess) return (int)e;                                                                       \
+            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
+                                                     nullptr, nullptr, nullptr, nullptr);                             \
+        }                                                                                                             \
+    } while (0)
+#define QR_XS_R(MT)                                                                                                   \
+    do {                                                                                                              \
+        if (rg == 8) QR_XS(MT, 8);                                                                                    \
+        else if (rg == 7) QR_XS(MT, 7);                                                                               \
+        else if (rg == 6) QR_XS(MT, 6);                                                                               \
+        else if (rg == 5) QR_XS(MT, 5);                                                                               \
+        else QR_XS(MT, 4);                                                                                            \
+    } while (0)
+    if (M <= 32) QR_XS_R(1);
+    else QR_XS_R(2);
+#undef QR_XS_R
+#undef QR_XS
+    return qr_launch_status();
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st) {
@@ -1961,10 +2212,10 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         return qr_launch_status();
     }
     if (M <= 64) {
-        // weight streaming: above 16 tokens and with enough 256-row tiles to fill the CUs the tiled
-        // kernel wins (X is read once per tile); otherwise the barrier-free kernel in which the waves
-        // of a workgroup split K over groups of 32 rows
-        if (M > 16 && (N + 255) / 256 >= 128) return launch_ks<64, 256, 1, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        // weight streaming: with enough groups of 32 rows to fill the CUs the kernel that shares the
+        // tokens' codes through LDS (they are read once per workgroup); otherwise the barrier-free
+        // kernel in which the waves of a workgroup split K over groups of 32 rows
+        if (const int rg = decode_xs_groups(n)) return launch_decode_xs(A, B, m, n, kb, C, Y, sA, sB, bias, st, rg);
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);

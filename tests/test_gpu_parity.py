@@ -181,6 +181,30 @@ def test_matmul_and_linear_random_shapes_across_every_kernel_boundary():
         assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw, bias))), (m, n, k)
 
 
+@pytest.mark.parametrize("n", [25600, 35200, 44800, 57344, 65536, 57339, 65500])
+def test_decode_with_many_weight_rows_shares_the_tokens_through_lds(n):
+    """Decode batches (5..64 tokens) against enough weight rows to give every CU a workgroup of 4..8 groups
+    of 32 rows (the five listed multiples pick 4, 5, 6, 7 and 8 groups; the last two end in a ragged
+    group): one and two token tiles, a token count that is not a multiple of 32, a single K stage, a
+    ragged last stage, and workgroups that start their walk over K at different stages."""
+    rng = np.random.default_rng(n)
+    for k in (64, 1088):
+        w = o.pack_i4(rng.integers(-8, 8, (n, k)))
+        sw = (np.abs(rng.standard_normal(n)) * 0.01 + 0.001).astype(F16)
+        bias = rng.standard_normal(n).astype(F16)
+        wg = gpu(w)
+        for m in ((5, 33, 64) if n != 57344 else (5, 17, 32, 33, 48, 64)):
+            a = o.pack_i4(rng.integers(-8, 8, (m, k)))
+            sa = (np.abs(rng.standard_normal(m)) * 0.2 + 0.01).astype(F16)
+            want = o.int4_matmul(a, w)
+            c = quarot_amd.matmul(gpu(a), wg)
+            assert np.array_equal(c.cpu().numpy(), want), (m, n, k)
+            y = quarot_amd.linear_i4(gpu(a), gpu(sa), wg, gpu(sw), gpu(bias))
+            assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw, bias))), (m, n, k)
+            y = quarot_amd.linear_i4(gpu(a), gpu(sa), wg, gpu(sw))
+            assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw))), (m, n, k)
+
+
 def test_matmul_known_answers_and_leading_dims():
     k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
     a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
