@@ -1549,62 +1549,61 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
 }
 
 // ------------------------------------------------------------------------------------------------
-// Decode (M <= 64) with many weight rows: a workgroup of eight waves owns R groups of 32 weight rows
-// (R = 4 .. 8, chosen by the host so that the workgroups spread evenly over the CUs: 57344 rows are
-// 256 workgroups of 7 groups) and walks K in stages of 128 packed bytes per row.
+// Decode (M <= 64) with many weight rows: a workgroup owns R groups of 32 weight rows (R = 4 .. 8,
+// chosen by the host so that the workgroups spread evenly over the CUs: 57344 rows are 256 workgroups
+// of 7 groups) and walks K in stages of 128 packed bytes per row.
+// * Twelve waves in two roles.  Waves 8..11 only FETCH: eight consecutive threads one 128-byte line,
+//   MT + R chunks per thread and stage, into RD register sets that rotate RD stages ahead of the LDS
+//   fill; three LDS stage buffers rotate; one barrier per stage.  Waves 0..R-1 only MULTIPLY: wave w
+//   takes row group w against all tokens.  With every wave doing both, a wave waits for its loads and
+//   then multiplies, the whole CU in step: the multiplications were not hidden behind the memory time
+//   (64 tokens: 47 us; with the roles split 42 us, the same as 8 tokens).
 // * The tokens' codes are fetched ONCE per workgroup and stage and shared through LDS -- with
 //   wave-private staging every wave would pull its own copy through the vector cache, twice the weight
 //   bytes at 64 tokens -- and the thread that fetched a chunk of them stores it already unpacked into
-//   its two int8 planes, so that no wave unpacks tokens.
-// * All 512 threads fetch (eight consecutive threads one 128-byte line) into RD register sets that
-//   rotate RD stages ahead of the LDS fill; three LDS stage buffers rotate; one barrier per stage.
-//   Threads whose chunk index lies beyond the stage repeat their first load into a spare slot.
-// * Wave w < R multiplies row group w against all tokens; waves beyond R only fetch.
+//   its two int8 planes, so that no multiplying wave unpacks tokens.
+// * The multiplications are software-pipelined over the 64-k sub-steps (see `substep`).
 // * Workgroup b starts its walk over K at stage b % stages and wraps around (integer sums do not depend
 //   on the order): with a row pitch that is a power of two, workgroups marching through K in step
 //   would all be reading the same few memory channels at any one time (measured 49 -> 41 us at
 //   57344 x 8192).
 template <int MT, int R, int RD, bool DEQ>
-__global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
+__global__ __launch_bounds__(768) void decode_xs_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
                                                         const f16* __restrict__ sB, const f16* __restrict__ bias) {
     constexpr int XR = MT * 32;                             // staged rows of X
-    constexpr int ROWS = XR + R * 32;
-    constexpr int NL = (ROWS + 63) / 64;                    // 16-byte chunks per thread and stage: 64 rows each
+    constexpr int NL = MT + R;                              // 16-byte chunks per loader thread and stage: 32 rows each
     constexpr int XPLANES = XR * 16;                        // slots of the tokens' planes (32 bytes per packed chunk)
-    constexpr int CH = XPLANES + (NL * 64 - XR) * 8;        // slots per stage buffer, spare ones included
+    constexpr int CH = XPLANES + R * 32 * 8;                // slots per stage buffer
     constexpr int NBUF = 3;
-    extern __shared__ u32x4 xs_lds[];                       // [NBUF][CH]; later the exchange, then the output slabs
+    extern __shared__ u32x4 xs_lds[];                       // [NBUF][CH]; later the output slabs
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
+    const bool loader = wave >= 8;                          // waves 8..11 fetch, waves 0..R-1 multiply
     const int n0 = blockIdx.x * (R * 32);
     const int stages = (Kb + 127) / 128;
     const bool ragged = (Kb & 127) != 0;
-    // weights: chunk position XOR-keyed by the row pair, so that the 16 rows a quarter-wave reads at one
-    // logical chunk cover all sixteen 16-byte bank groups (row parity picks the half)
     auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
-    // token planes: 16 slots per row; chunk keyed by row & 7, plane by bit 3 of the row
     auto slot16 = [](int row, int chunk, int plane) {
         return row * 16 + ((chunk ^ (row & 7)) << 1) + (plane ^ ((row >> 3) & 1));
     };
 
-    const int srow = tid >> 3, piece = tid & 7;             // chunk i of this thread: row srow + 64 i, same piece
-    const bool xthread = XR == 64 || srow < XR;             // chunk 0 is a row of X (whole waves)
+    const int ltid = tid & 255;
+    const int srow = ltid >> 3, piece = ltid & 7;           // chunk i of a loader thread: row srow + 32 i, same piece
     const uint8_t* src[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        int row = srow + i * 64;
-        if (row >= ROWS) row = srow;                        // spare slot: repeat the first chunk
-        if (row < XR) {
-            src[i] = A + (int64_t)(row < M ? row : M - 1) * Kb;
+        if (i < MT) {
+            const int mr = srow + 32 * i;
+            src[i] = A + (int64_t)(mr < M ? mr : M - 1) * Kb;
         } else {
-            const int nr = n0 + row - XR;
+            const int nr = n0 + srow + 32 * (i - MT);
             src[i] = B + (int64_t)(nr < N ? nr : N - 1) * Kb;
         }
     }
-    const int wdst0 = XPLANES - XR * 8 + slot8(srow, piece);   // rows differ by multiples of 32: same swizzle
-    const int xdst0 = slot16(srow & (XR - 1), piece, 0);
+    const int wdst0 = XPLANES + slot8(srow, piece);         // rows differ by multiples of 32: same swizzle
+    const int xdst0 = slot16(srow, piece, 0);
     const int s0 = blockIdx.x % stages;
     auto stage_of = [&](int st) {
         int a = (st < stages ? st : stages - 1) + s0;
@@ -1617,7 +1616,7 @@ __global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restric
         for (int i = 0; i < NL; ++i) {
             // weights are used once: streaming loads keep the tokens' codes, which every workgroup
             // re-reads, in the caches
-            if (i * 64 >= XR && (i + 1) * 64 <= ROWS) v[i] = __builtin_nontemporal_load((const u32x4*)(src[i] + off));
+            if (i >= MT) v[i] = __builtin_nontemporal_load((const u32x4*)(src[i] + off));
             else v[i] = *(const u32x4*)(src[i] + off);
         }
     };
@@ -1629,11 +1628,11 @@ __global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restric
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const u32x4 q = zero ? u32x4{0, 0, 0, 0} : v[i];
-            if (i == 0 && xthread) {
-                base[xdst0] = (q << 4) & 0xF0F0F0F0u;
-                base[xdst0 ^ 1] = q & 0xF0F0F0F0u;
+            if (i < MT) {
+                base[xdst0 + i * 32 * 16] = (q << 4) & 0xF0F0F0F0u;
+                base[(xdst0 ^ 1) + i * 32 * 16] = q & 0xF0F0F0F0u;
             } else {
-                base[wdst0 + i * 64 * 8] = q;
+                base[wdst0 + (i - MT) * 32 * 8] = q;
             }
         }
     };
@@ -1644,7 +1643,7 @@ __global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restric
         for (int v = 0; v < 16; ++v) acc[t][v] = 0;
     // logical chunk 2u + h of weight row q sits at slot8(q, h) ^ (2u); plane p of a token row's chunk
     // 2u + h at slot16(q, h, 0) ^ (4u + p): the swizzles only touch the low bits
-    const bool computes = wave < R;
+    const bool computes = wave < R;                         // (waves R..7 only keep the barriers' count)
     const int wslot = XPLANES + slot8((computes ? wave : 0) * 32 + r, h), xslot = slot16(r, h, 0);
     // The multiplications are software-pipelined over the 64-k sub-steps: while the 2 MT MFMAs of one
     // sub-step run, the operands of the next one (the first of the next stage after the last: that
@@ -1691,13 +1690,34 @@ __global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restric
         }
     };
 
-    u32x4 regs[RD][NL];
+    if (loader) {
+        u32x4 regs[RD][NL];
 #pragma unroll
-    for (int q = 0; q < RD; ++q) fetch(q, regs[q]);
-    deposit(0, 0, regs[0]);
-    fetch(RD, regs[0]);
-    deposit(1, 1, regs[1 % RD]);
-    fetch(RD + 1, regs[1 % RD]);
+        for (int q = 0; q < RD; ++q) fetch(q, regs[q]);
+        deposit(0, 0, regs[0]);
+        fetch(RD, regs[0]);
+        deposit(1, 1, regs[1 % RD]);
+        fetch(RD + 1, regs[1 % RD]);
+        __syncthreads();                                    // stages 0 and 1 visible
+        int bfill = 2;
+        auto iteration = [&](int ks, u32x4(&v)[NL]) {
+            deposit(ks + 2, bfill, v);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(ks + 2 + RD, v);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            bfill = bfill == NBUF - 1 ? 0 : bfill + 1;
+        };
+        int ks0 = 0;
+        for (; ks0 + RD <= stages; ks0 += RD) {
+#pragma unroll
+            for (int q = 0; q < RD; ++q) iteration(ks0 + q, regs[(q + 2) % RD]);
+        }
+#pragma unroll
+        for (int q = 0; q < RD - 1; ++q)
+            if (ks0 + q < stages) iteration(ks0 + q, regs[(q + 2) % RD]);
+        return;
+    }
     __syncthreads();                                        // stages 0 and 1 visible
     if (computes) {
         read_w(xs_lds, 0, ops[0]);
@@ -1709,32 +1729,21 @@ __global__ __launch_bounds__(512) void decode_xs_kernel(const uint8_t* __restric
         unpack_lo(ops[0]);
         unpack_hi(ops[0]);
     }
-    int bcur = 0;
-    auto iteration = [&](int ks, u32x4(&v)[NL]) {
-        const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
-        const int bfill = bnext == NBUF - 1 ? 0 : bnext + 1;
-        deposit(ks + 2, bfill, v);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(ks + 2 + RD, v);
-        __builtin_amdgcn_sched_barrier(0);
-        if (computes) {
-            const u32x4* cb = xs_lds + bcur * CH;
-            substep(ops[0], ops[1], cb, 1);
-            substep(ops[1], ops[0], cb, 2);
-            substep(ops[0], ops[1], cb, 3);
-            substep(ops[1], ops[0], xs_lds + bnext * CH, 0);   // after the last stage: read, never used
+    {
+        int bcur = 0;
+        for (int ks = 0; ks < stages; ++ks) {
+            const int bnext = bcur == NBUF - 1 ? 0 : bcur + 1;
+            if (computes) {
+                const u32x4* cb = xs_lds + bcur * CH;
+                substep(ops[0], ops[1], cb, 1);
+                substep(ops[1], ops[0], cb, 2);
+                substep(ops[0], ops[1], cb, 3);
+                substep(ops[1], ops[0], xs_lds + bnext * CH, 0);   // after the last stage: read, never used
+            }
+            __syncthreads();
+            bcur = bnext;
         }
-        __syncthreads();
-        bcur = bnext;
-    };
-    int ks0 = 0;
-    for (; ks0 + RD <= stages; ks0 += RD) {
-#pragma unroll
-        for (int q = 0; q < RD; ++q) iteration(ks0 + q, regs[(q + 2) % RD]);
     }
-#pragma unroll
-    for (int q = 0; q < RD - 1; ++q)
-        if (ks0 + q < stages) iteration(ks0 + q, regs[(q + 2) % RD]);
 
     // ---- epilogue: lane l, register v -> weight row (v/4)*8 + (l/32)*4 + v%4 of the group, token l%32
     auto finish = [&](const i32x16& a, int g, int t) {
@@ -2077,13 +2086,13 @@ int launch_decode_xs(const void* A, const void* B, int M, int N, int Kb, void* C
             auto kern = decode_xs_kernel<MT, R, RD, true>;                                                            \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
-            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, \
+            kern<<<dim3(grid), dim3(768), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, \
                                                      (const f16*)sA, (const f16*)sB, (const f16*)bias);               \
         } else {                                                                                                      \
             auto kern = decode_xs_kernel<MT, R, RD, false>;                                                           \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
-            kern<<<dim3(grid), dim3(512), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
+            kern<<<dim3(grid), dim3(768), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
                                                      nullptr, nullptr, nullptr, nullptr);                             \
         }                                                                                                             \
     } while (0)
