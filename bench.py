@@ -83,10 +83,14 @@ HBM_PEAK_GBS = 8000.0
 # ("traffic_kib: kernel=<substring> fetch=<KiB per dispatch> write=<KiB per dispatch>") and the copy
 # calibration ("traffic_scale: fetch=<factor> write=<factor>").
 PROFILE_OF = {
-    "c1": "gemm_spk_c1_q_proj_7b.txt", "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt",
-    "c2": "gemm_spk_and_hadamard_m64_c2_down_proj_7b.txt", "c3d": "gemm_sp256_c3d_prefill_16x2048.txt",
-    "c4m64": "decode_i4_c4_decode_64_tokens_70b_down_proj.txt", "c4m1": "gemv_i4_c4m1_decode_70b_down_proj.txt",
-    "c4g64": "gemm_ks_64x256_c4g64_decode_64_tokens_70b_gate_up.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
+    "c1": "gemm_spk_c1_q_proj_7b.txt", "c1n": "rmsnorm_quant_rows_c1n_q_proj_7b.txt",
+    "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt", "c2": "gemm_spk_and_hadamard_m64q_c2_down_proj_7b.txt",
+    "c3": "gemm_sp256_c3_prefill_layer_set_32768_tokens.txt",
+    "c4g8": "decode_xs_c4g8_decode_8_tokens_70b_gate_up.txt", "c4g32": "decode_xs_c4g32_decode_32_tokens_70b_gate_up.txt",
+    "c4g64": "decode_xs_c4g64_decode_64_tokens_70b_gate_up.txt", "c4m1": "gemv_i4_c4m1_decode_70b_down_proj.txt",
+    "c4m8": "decode_i4_c4m8_decode_8_tokens_70b_down_proj.txt", "c4m32": "decode_i4_c4m32_decode_32_tokens_70b_down_proj.txt",
+    "c4m64": "decode_i4_c4m64_decode_64_tokens_70b_down_proj.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
+    "c6": "paged_decode_i4_c6_decode_attention_32x4096x8x128.txt",
 }
 
 
@@ -581,6 +585,8 @@ def main():
     wl, res, steps, repeats = measure(args.workload, True)
     roof = dict(res["roofline"])
     traffic, source = traffic_from_profile(args.workload, roof["kernel"])
+    if traffic is not None and args.workload == "c3":
+        traffic *= 4                                       # the step is four launches; the summary holds their average
     roof["traffic"] = traffic
     roof["traffic_source"] = source
     kv_line = args.workload in ("c5", "c6", "c6b")
@@ -614,10 +620,9 @@ def main():
             torch.cuda.empty_cache()
             _, r, _, _ = measure(name, False)
             per[name] = brief(r)
-            if name != "c3":
-                t, s = traffic_from_profile(name, r["roofline"]["kernel"])
-                if t is not None:
-                    per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = t, s
+            t, s = traffic_from_profile(name, r["roofline"]["kernel"])
+            if t is not None:
+                per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = (4 * t if name == "c3" else t), s
         out["per_config"] = per
         out["per_config_note"] = ("same step definition as the headline; operands generated on the GPU, a fifth of the steps per loop "
                                   "(c3, c5: fewer still) and half the repeats")
