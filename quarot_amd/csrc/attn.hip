@@ -421,17 +421,17 @@ extern "C" int qr_kv_append_i4(void* kv_data, void* kv_param, const void* kv_ind
 }
 
 namespace {
-// Waves per (sequence, head): enough to fill the GPU's 4096 wave slots, each with at least four steps of 16
+// Waves per (sequence, head): enough to fill the GPU's wave slots (16 per CU), each with at least four steps of 16
 // positions when the caller says how long the sequences can be.  Up to 16 of them form one workgroup;
 // beyond that the sequence is split over several workgroups, which needs room for their partial states.
 struct DecodePlan {
     int nw, splits;
 };
 DecodePlan decode_plan(int64_t batch_size, int num_heads, int64_t max_seq_len) {
-    const int64_t bh = batch_size * num_heads;
-    if (max_seq_len <= 0) return DecodePlan{bh >= 1024 ? 4 : bh >= 256 ? 8 : 16, 1};
+    const int64_t bh = batch_size * num_heads, cus = qr_device().cus;
+    if (max_seq_len <= 0) return DecodePlan{bh >= 4 * cus ? 4 : bh >= cus ? 8 : 16, 1};
     const int64_t chunks = (max_seq_len + 15) / 16;
-    int64_t wp = (4096 + bh - 1) / bh, cap = chunks / 4;
+    int64_t wp = (16 * cus + bh - 1) / bh, cap = chunks / 4;
     wp = wp > cap ? cap : wp;
     if (wp <= 4) return DecodePlan{4, 1};
     if (wp <= 16) return DecodePlan{8, 1};                  // (measured a few percent ahead of 16 waves at 256 (sequence, head) pairs)

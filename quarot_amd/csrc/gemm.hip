@@ -85,7 +85,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int nxcd) {
     constexpr int NT = 64 * WAVES_M * WAVES_N;              // threads per workgroup
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;     // per-wave output tile
     constexpr int IM = TM / 32, JN = TN / 32;               // 32x32 MFMA tiles per wave
@@ -98,10 +98,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
     __shared__ u32x4 lds_raw[2 * CH];
     u32x4(*lds)[CH] = (u32x4(*)[CH])lds_raw;
 
-    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  Give every XCD a
+    // Workgroups are dealt round-robin to the nxcd XCDs (each with its own L2).  Give every XCD a
     // contiguous range of tile ids, and walk tiles in groups of GROUP_M rows so that the tiles in
     // flight on one XCD share A rows and B rows.
-    const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
     int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
     if (tile >= tiles_m * tiles_n) return;
@@ -357,7 +356,7 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool DEQ>
 __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n, int ksplit) {
+    int tiles_m, int tiles_n, int ksplit, int nxcd) {
     constexpr int NT = 128 * WAVES_M * WAVES_N;
     constexpr int TM = BM / WAVES_M, TN = BN / WAVES_N;
     constexpr int IM = TM / 32, JN = TN / 32;
@@ -373,7 +372,6 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
     static_assert(CH % NT == 0 && JN % 2 == 0, "tile shape");
     extern __shared__ u32x4 ks_lds[];                       // [NBUF][CH]; later the accumulator exchange
 
-    const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
     const int unit = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
     if (unit >= tiles_m * tiles_n * ksplit) return;
@@ -674,20 +672,21 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
     const int64_t tiles = (int64_t)tiles_m * tiles_n * ksplit;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     if (ksplit > 1 && Y) return QR_E_UNSUPPORTED;           // partial sums exist only as int32
-    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
+    const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
     hipError_t e;
     if (Y) {
         auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, true>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
-                                                (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, 1);
+                                                (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, 1, nxcd);
     } else {
         auto kern = gemm_ks_kernel<BM, BN, WAVES_M, WAVES_N, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(NT), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
-                                                nullptr, nullptr, nullptr, tiles_m, tiles_n, ksplit);
+                                                nullptr, nullptr, nullptr, tiles_m, tiles_n, ksplit, nxcd);
     }
     return qr_launch_status();
 }
@@ -711,7 +710,7 @@ template <bool DEQ, bool RAGGED>
 __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int nxcd) {
     constexpr int BM = 256, BN = 256, NT = 256;
     constexpr int TM = 128, TN = 128, IM = 4, JN = 4;
     constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
@@ -723,7 +722,6 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     constexpr bool DIRECT = !RAGGED;                        // whole stages go straight into LDS (see gemm_spk_kernel)
     extern __shared__ u32x4 sp2_lds[];                       // [2][CH]; later the output slabs
 
-    const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
     int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
     if (tile >= tiles_m * tiles_n) return;
@@ -977,7 +975,7 @@ template <bool DEQ, bool RAGGED>
 __global__ __launch_bounds__(256) void gemm_spk_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int nxcd) {
     constexpr int BM = 128, BN = 256, NT = 256;
     constexpr int TM = 128, TN = 128, IM = 4, JN = 4;
     constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
@@ -993,7 +991,6 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     constexpr bool DIRECT = !RAGGED;
     extern __shared__ u32x4 spk_lds[];                       // [DIRECT ? 3 : 2][CH]; later the output slabs
 
-    const int nxcd = 8;
     const int per_xcd = gridDim.x / nxcd;
     int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
     if (tile >= tiles_m * tiles_n) return;
@@ -1318,7 +1315,8 @@ int launch_spk(const void* A, const void* B, int M, int N, int Kb, void* C, void
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
-    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
+    const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
     const bool ragged = (Kb & 127) != 0;
     // stage buffers of 48 KB: two behind staging registers, three when loaded straight into LDS
     const size_t LDS = (size_t)(ragged ? 2 : 3) * (128 + 256) * 8 * 16;
@@ -1330,13 +1328,13 @@ int launch_spk(const void* A, const void* B, int M, int N, int Kb, void* C, void
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
-                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, nxcd);
     } else {
         auto kern = ragged ? gemm_spk_kernel<false, true> : gemm_spk_kernel<false, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
-                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
+                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n, nxcd);
     }
     return qr_launch_status();
 }
@@ -1351,7 +1349,8 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
-    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
+    const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
     const bool ragged = (Kb & 127) != 0;
     // operands are addressed through 32-bit buffer offsets
     if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
@@ -1362,13 +1361,13 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
-                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n);
+                                                 (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, nxcd);
     } else {
         auto kern = ragged ? gemm_sp256_kernel<false, true> : gemm_sp256_kernel<false, false>;
         e = qr_allow_dynamic_lds((const void*)kern, LDS);
         if (e != hipSuccess) return (int)e;
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
-                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n);
+                                                 nullptr, nullptr, nullptr, tiles_m, tiles_n, nxcd);
     }
     return qr_launch_status();
 }
@@ -1947,17 +1946,18 @@ __global__ __launch_bounds__(256) void gemv_i4_kernel(const uint8_t* __restrict_
 int launch_gemv(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                 const void* bias, hipStream_t st) {
     const int groups = (N + 3) / 4;
-    // row groups per wave: about 64 KB of weights per wave, but keep >= 2048 waves when N allows ...
+    // row groups per wave: about 64 KB of weights per wave, but keep >= 8 waves per CU when N allows ...
     int ng = (65536 + 4 * Kb - 1) / (4 * Kb);
-    while (ng > 1 && groups / ng < 2048) --ng;
+    const int cus = qr_device().cus;
+    while (ng > 1 && groups / ng < 8 * cus) --ng;
     // ... and, when all workgroups are resident at once (up to five per CU), a count that spreads
-    // evenly over the 256 CUs: 3.5 workgroups per CU run as long as 4.  Among ng / 2 ... 2 ng the
-    // value nearest to ng whose last round of 256 is at least 97 % full, else the fullest.
+    // evenly over the CUs: 3.5 workgroups per CU run as long as 4.  Among ng / 2 ... 2 ng the
+    // value nearest to ng whose last round over the CUs is at least 97 % full, else the fullest.
     {
         auto fill = [&](int g) {
             const int wgs = ((groups + g - 1) / g + 3) / 4;
-            if (wgs > 1280) return 1.0;
-            return (double)wgs / (double)(((wgs + 255) / 256) * 256);
+            if (wgs > 5 * cus) return 1.0;
+            return (double)wgs / (double)(((wgs + cus - 1) / cus) * cus);
         };
         int best = ng;
         double best_fill = fill(ng);
@@ -2025,12 +2025,13 @@ int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, v
     // is a fixed part (start, first loads, final sum: about six steps' worth) plus its steps per wave.
     if (kw == 0) {
         kw = 8;
+        const int cus = qr_device().cus;
         if (M <= 32) {
             const int steps = (Kb + 127) / 128;
             double best = 0;
             for (int c = 8; c >= 2; c >>= 1) {
                 const int wgs = (N + 32 * (8 / c) - 1) / (32 * (8 / c));
-                const double cost = (double)((wgs + 255) / 256) * (6.0 + (double)steps / c);
+                const double cost = (double)((wgs + cus - 1) / cus) * (6.0 + (double)steps / c);
                 if (c == 8 || cost < best) {
                     best = cost;
                     kw = c;
@@ -2057,15 +2058,15 @@ int launch_decode(const void* A, const void* B, int M, int N, int Kb, void* C, v
 }
 
 // Row groups per workgroup for the shared-token decode kernel: the count among 4 .. 8 with the least
-// work on the busiest CU (rounds of 256 workgroups times groups per workgroup), larger counts first
+// work on the busiest CU (rounds of workgroups over the CUs times groups per workgroup), larger counts first
 // (fewer copies of the tokens' codes).  0: too few row groups to fill the CUs this way.
 int decode_xs_groups(int N) {
-    const int groups = (N + 31) / 32;
+    const int groups = (N + 31) / 32, cus = qr_device().cus;
     int best = 0, best_cost = 0;
     for (int rg = 8; rg >= 4; --rg) {
         const int wgs = (groups + rg - 1) / rg;
-        if (wgs < 192) continue;
-        const int cost = ((wgs + 255) / 256) * rg;
+        if (wgs < cus * 3 / 4) continue;
+        const int cost = ((wgs + cus - 1) / cus) * rg;
         if (best == 0 || cost < best_cost) {
             best = rg;
             best_cost = cost;
@@ -2118,15 +2119,16 @@ int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
-    const unsigned grid = (unsigned)((tiles + 7) / 8 * 8);
+    const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
+    const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
     if (Y)
         gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, true><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, (const f16*)sA, (const f16*)sB,
-            (const f16*)bias, tiles_m, tiles_n);
+            (const f16*)bias, tiles_m, tiles_n, nxcd);
     else
         gemm_i4_kernel<BM, BN, WAVES_M, WAVES_N, false><<<dim3(grid), dim3(NT), 0, st>>>(
             (const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr, nullptr, nullptr, nullptr, tiles_m,
-            tiles_n);
+            tiles_n, nxcd);
     return qr_launch_status();
 }
 
@@ -2180,15 +2182,16 @@ __global__ __launch_bounds__(256) void dequant_slabs_kernel(const int32_t* __res
 int ks_split(int64_t M, int64_t N, int64_t Kb) {
     if (M <= 64 || N <= 128) return 1;
     const int64_t tn = (N + 255) / 256;
-    if (((M + 127) / 128) * tn >= 128) return 1;
+    const int64_t cus = qr_device().cus;
+    if (((M + 127) / 128) * tn >= cus / 2) return 1;
     const int64_t tiles = ((M + 63) / 64) * tn;
     const int64_t all_stages = (Kb + 127) / 128;
-    const double t_unsplit = 6.0 + 1.0 * (double)all_stages * (double)((tiles + 255) / 256);
+    const double t_unsplit = 6.0 + 1.0 * (double)all_stages * (double)((tiles + cus - 1) / cus);
     int best = 1;
     double t_best = 0.8 * t_unsplit;
     for (int64_t ks = 2; ks <= 16 && ks <= all_stages / 4; ++ks) {
         const double slabs_us = 2.0 * (double)ks * (double)M * (double)N * 4.0 / 4.0e6;
-        const double t = 8.0 + 1.0 * (double)((all_stages + ks - 1) / ks) * (double)((tiles * ks + 255) / 256) + slabs_us;
+        const double t = 8.0 + 1.0 * (double)((all_stages + ks - 1) / ks) * (double)((tiles * ks + cus - 1) / cus) + slabs_us;
         if (t < t_best) {
             t_best = t;
             best = (int)ks;
@@ -2228,12 +2231,13 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
         return launch_decode(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
-    if (t128x256 >= 128) {
+    const int64_t cus = qr_device().cus;
+    if (t128x256 >= cus / 2) {
         // 256x256 tiles run ~1.2x faster per unit of work (3 instead of 4.5 unpacking instructions per
         // MFMA) but quantise worse over the 256 CUs: compare rounds of tiles, a 128x256 tile costing
         // 0.61 of a 256x256 one
-        const double rounds256 = (double)((t256 + 255) / 256);
-        const double rounds128 = (double)((t128x256 + 255) / 256) * 0.61;
+        const double rounds256 = (double)((t256 + cus - 1) / cus);
+        const double rounds128 = (double)((t128x256 + cus - 1) / cus) * 0.61;
         if (rounds256 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_spk(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }

@@ -453,7 +453,7 @@ int launch_hadamard_km(const void* x, void* y, int64_t rows, int n, int K, int l
             hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds); \
             if (e != hipSuccess) return (int)e;                                                                       \
         }                                                                                                             \
-        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);                                     \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, lds);                                     \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                    \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, log2m, hadK, scale, clip, (u32*)q, \
                                                 (f16*)scales);                                                        \
@@ -1117,11 +1117,14 @@ __global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restr
 #pragma unroll
         for (int ks = 0; ks < KS2; ++ks) asm volatile("" : "+v"(hf[t][ks]));
     __syncthreads();
-    // The quantiser of row r is ~250 vector instructions per lane, the hadK stage of row r + 1 is 12 KS2
-    // matrix instructions of 16 cycles each whose issue slots are otherwise empty: the two are interleaved
-    // in program order (three matrix instructions, then one pair of the previous row's values), pinned by
-    // scheduling barriers, so that the vector and matrix pipes overlap by construction rather than by
-    // the chance phase of the two workgroups that share a SIMD.
+    // The quantiser of row r (~350 vector instructions per lane) is written between the matrix
+    // instructions of row r + 1's hadK stage.  What the compiler makes of it: the codes are only used on the
+    // lean path of finish_prev, so the optimiser sinks the arithmetic into that branch, behind the stage,
+    // and schedules it there as one block.  That is the fastest of the three forms measured at 11008
+    // columns (32768 rows): this one 270-283 us; the same arithmetic written after the stage 305-310 us;
+    // the interleaving forced (each part pinned with an empty asm statement, 2-5 vector instructions
+    // after every matrix instruction in the generated code) 340-350 us -- two workgroups share a SIMD, and
+    // a pure matrix phase of one overlaps a pure vector phase of the other better than two mixed streams.
     u32x2 yp[TPW][CT];                                       // previous row's fp16 results (the same lane layout)
     u32 pb[TPW][CT][2];                                      // ... its codes as fp16 1536 + code pairs
     // Before the first row there is no previous one: the turn then "finishes" zeros with scale 1 into the
@@ -1337,7 +1340,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
 #define QR_M64Q(KS)                                                                                                    \
     do {                                                                                                               \
         auto kern = hadamard_m64q_kernel<KS>;                                                                          \
-        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, ldsq);                                     \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                                     \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \
                                                  (f16*)scales);                                                        \
@@ -1361,7 +1364,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
             hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds64);                                             \
             if (e != hipSuccess) return (int)e;                                                                        \
         }                                                                                                              \
-        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds64);                                    \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, lds64);                                    \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), lds64, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,      \
                                                   (f16*)scales);                                                       \
@@ -1390,7 +1393,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
             hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);                                               \
             if (e != hipSuccess) return (int)e;                                                                        \
         }                                                                                                              \
-        const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);                                      \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, lds);                                      \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
                                                 (f16*)scales);                                                         \
@@ -1619,7 +1622,7 @@ int launch_hadamard(const void* x, void* y, int64_t rows, int n, int K, const vo
     }
     // persistent workgroups: as many as fit the CUs' LDS at once (256 CUs, 160 KB each), so that the
     // hadK staging is paid once per resident workgroup
-    const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, HT, lds);
+    const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, lds);
     const int64_t grid = rows < cap ? rows : cap;
     kern<<<dim3((unsigned)grid), dim3(HT), lds, st>>>((const IO*)x, (IO*)y, rows, n, K, log2m, hadK, scale, clip,
                                                       (u32*)q, (f16*)scales, hs_stride);

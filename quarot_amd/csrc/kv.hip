@@ -488,7 +488,7 @@ int launch_had128(const void* x, int64_t vectors, float hscale, void* q, void* s
     auto kern = kv_had128_kernel<QUANT, PAGED>;
     const int64_t blocks = (vectors + 31) >> 5;
     const int64_t want = (blocks + KM_WAVES - 1) / KM_WAVES;
-    const int64_t cap = 256LL * qr_blocks_per_cu((const void*)kern, 64 * KM_WAVES, 0);
+    const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, 64 * KM_WAVES, 0);
     const unsigned grid = (unsigned)(want < cap ? want : cap);
     kern<<<dim3(grid), dim3(64 * KM_WAVES), 0, st>>>((const u32x4*)x, vectors, hscale, (u32x4*)q, (f16*)scale, (f16*)zero,
                                                     (u32x4*)y, pd);

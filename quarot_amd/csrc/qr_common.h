@@ -47,6 +47,27 @@ static inline hipError_t qr_allow_dynamic_lds(const void* kernel, size_t bytes) 
     return e;
 }
 
+// Compute units of the current device and the number of XCDs (L2 domains) they form: workgroups are
+// dealt round-robin to the XCDs, 32 CUs each on gfx950 (256 CUs = 8 XCDs; a partitioned device has
+// fewer of both).  Cached per device; {256, 8} if the query fails.
+struct QrDevice {
+    int cus, xcds;
+};
+static inline QrDevice qr_device() {
+    constexpr int kMax = 64;
+    static QrDevice table[kMax];
+    static std::mutex guard;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMax) return QrDevice{256, 8};
+    std::lock_guard<std::mutex> lock(guard);
+    if (table[dev].cus == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = 256;
+        table[dev] = QrDevice{cus, cus >= 64 ? cus / 32 : 1};
+    }
+    return table[dev];
+}
+
 // Resident workgroups per CU for a kernel at a given block size and dynamic LDS size (cached; used
 // to size the grid of persistent kernels so that every workgroup is resident at once).
 static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) {
