@@ -75,7 +75,7 @@ WORKLOADS = {
 for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
-PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6"]
+PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 HBM_PEAK_GBS = 8000.0
 
@@ -91,6 +91,8 @@ PROFILE_OF = {
     "c4m8": "decode_i4_c4m8_decode_8_tokens_70b_down_proj.txt", "c4m32": "decode_i4_c4m32_decode_32_tokens_70b_down_proj.txt",
     "c4m64": "decode_i4_c4m64_decode_64_tokens_70b_down_proj.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
     "c6": "paged_decode_i4_c6_decode_attention_32x4096x8x128.txt",
+    "b13v": "gemm_sp256_b13v_2048x5120x5120.txt", "b70v": "gemm_sp256_b70v_2048x8192x8192.txt",
+    "b13d": "gemm_sp256_b13d_2048x13824x5120.txt", "b70d": "gemm_sp256_b70d_2048x28672x8192.txt",
 }
 
 
