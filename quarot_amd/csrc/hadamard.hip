@@ -494,7 +494,8 @@ bool km_applies(int n, int K, bool mode32) {
 template <bool MODE32, bool QUANT, int LOG2M, int KS2, bool XLDS>
 __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
                                                          int n, int K, const void* __restrict__ hadK, float scale,
-                                                         float clip, u32* __restrict__ q, f16* __restrict__ scales) {
+                                                         float clip, u32* __restrict__ q, f16* __restrict__ scales,
+                                                         int ident) {
     constexpr int M_ = 1 << LOG2M;
     constexpr int KS1 = M_ / 32;                 // contraction steps of stage 1
     constexpr int CT = M_ / 16;                  // 16-column tiles of T / Y
@@ -573,7 +574,11 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
                 for (int e = 0; e < 4; ++e) hf[t][ks][hh * 4 + e] = v[e];
             }
     }
-    // Sylvester fragments: H_m[r][r'] = (-1)^popcount(r & r')
+    // Sylvester fragments: H_m[r][r'] = (-1)^popcount(r & r').  With `ident` the inner factor is the
+    // identity instead, y = x . (hadK (x) I_m)^T * scale: the transform ACROSS m-wide groups, which is what
+    // OnlineHadamard(num_heads) on the transposed attention output computes (e2e/quantized_llama/
+    // modeling_llama.py:108-110), with the same staging as the reference (x * scale rounded to fp16, then
+    // hadK @ .: quarot/functional/hadamard.py:94-101 with n / K = 1).
     f16x8 b1[NCT][KS1];
 #pragma unroll
     for (int c = 0; c < NCT; ++c)
@@ -583,7 +588,8 @@ __global__ __launch_bounds__(HT) void hadamard_mm_kernel(const f16* __restrict__
             for (int j = 0; j < 8; ++j) {
                 const int rp = (wave + 4 * c) * 16 + l16;
                 const int r = ks * 32 + g * 8 + j;
-                b1[c][ks][j] = (__builtin_popcount(r & rp) & 1) ? (f16)-1.0f : (f16)1.0f;
+                const f16 sylv = (__builtin_popcount(r & rp) & 1) ? (f16)-1.0f : (f16)1.0f;
+                b1[c][ks][j] = ident ? (r == rp ? (f16)1.0f : (f16)0.0f) : sylv;
             }
 
     // stage-1 A-fragments for the tile pair s2 of a row: [2 tiles][KS1] 16-byte loads
@@ -1326,10 +1332,10 @@ bool mm_applies(int n, int K) {
 
 template <bool MODE32, bool QUANT>
 int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
-                       void* q, void* scales, hipStream_t st) {
+                       void* q, void* scales, hipStream_t st, int ident = 0) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
-    if (m == 64 && K >= 64) {
+    if (m == 64 && K >= 64 && !ident) {
         // the latency-organised kernel (it relies on every wave's first tile lying inside hadK), while
         // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
@@ -1396,7 +1402,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, lds);                                      \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), lds, st>>>((const f16*)x, (f16*)y, rows, n, K, hadK, scale, clip, (u32*)q,        \
-                                                (f16*)scales);                                                         \
+                                                (f16*)scales, ident);                                                  \
     } while (0)
 #define QR_MM_X(L2M, KS)                 \
     if (xlds) QR_MM(L2M, KS, true);      \
@@ -1861,4 +1867,15 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (mode == QR_DTYPE_F16) return launch_hadamard<f16, false, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     if (mode == QR_DTYPE_F32) return launch_hadamard<f16, true, true>(x, y_or_null, rows, n, K, hadK, scale, clip, q, scales, st);
     return QR_E_DTYPE;
+}
+
+// quant.hip: Hadamard across `heads` groups of 128 + quantiser for head counts that are orders of the
+// reference's tables: the fused two-stage kernel with the identity as inner factor
+__attribute__((visibility("hidden"))) int qr_internal_heads_matrix_quantize(const void* x, int64_t rows, int heads,
+                                                                            const void* hadK, float clip, void* q,
+                                                                            void* scales, void* y_or_null, hipStream_t st) {
+    const int n = heads * 128;
+    if (!mm_applies(n, heads)) return QR_E_UNSUPPORTED;
+    return launch_hadamard_mm<false, true>(x, y_or_null, rows, n, heads, hadK, 1.0f / __builtin_sqrtf((float)heads), clip, q,
+                                           scales, st, 1);
 }

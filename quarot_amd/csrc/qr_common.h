@@ -93,6 +93,10 @@ static inline int qr_blocks_per_cu(const void* kernel, int threads, size_t lds) 
 // kv.hip: y = x . H_128 * scale on rows of 128 halves (matrix-core kernel shared with the K-cache quantiser)
 int qr_internal_hadamard128_f16(const void* x, void* y, int64_t rows, float scale, hipStream_t st);
 
+// hadamard.hip: y = x . (hadK (x) I_128)^T / sqrt(heads) on rows of heads * 128 halves, then the quantiser
+int qr_internal_heads_matrix_quantize(const void* x, int64_t rows, int heads, const void* hadK, float clip, void* q,
+                                      void* scales, void* y_or_null, hipStream_t st);
+
 static inline int qr_launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? QR_OK : (int)e;

@@ -261,80 +261,6 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
     for (int i = 0; i < NC; ++i) qr[lane + i * QR_WAVE] = sym_codes8(v[i], s, rs, fast);
 }
 
-// The same chain for head counts that are not powers of two but orders of the reference's tables
-// (had_40 for the 40 heads of Llama-2-13B, had_52 for the 52 of Llama-30B, ...): OnlineHadamard(H) is
-// then hadK alone, y[g, d] = fp16( sum_h hadK[g, h] * fp16(x[h, d] / sqrt(H)) ) -- the reference's
-// two-step form rounds the scaled input to fp16 before the matrix product
-// (quarot/functional/hadamard.py:99-100).  One workgroup per row: the scaled row in LDS as floats,
-// hadK transposed in LDS; thread (d, half) forms four consecutive outputs g per pass (one 16-byte
-// broadcast of coefficients and one 4-byte read of x per four multiply-adds), the fp16 results go
-// back to LDS in row order and are quantised from there like any other row.
-__global__ __launch_bounds__(QT) void heads_matrix_quant_rows_kernel(const u32x4* __restrict__ x, int H,
-                                                                     const f16* __restrict__ hadK, float hscale,
-                                                                     float clip, u32* __restrict__ q,
-                                                                     f16* __restrict__ scale_out,
-                                                                     u32x4* __restrict__ y) {
-    static_assert(QT == 256, "two halves of 128 positions");
-    constexpr int LD = 129;                                  // floats per staged head: odd, positions hit distinct banks
-    extern __shared__ f32x4 hm_lds[];
-    float* Xs = (float*)hm_lds;                              // [H][LD]
-    float* Mt = Xs + ((H * LD + 3) & ~3);                    // [H][H], Mt[h][g] = hadK[g][h]; 16-byte aligned (H % 4 == 0)
-    f16* Ys = (f16*)(Mt + H * H);                            // [H][128]
-    __shared__ u32 red[QT / QR_WAVE];
-    const int64_t row = blockIdx.x;
-    const int lane = threadIdx.x & (QR_WAVE - 1), wave = threadIdx.x / QR_WAVE;
-    const int cols8 = H * 16;
-    const u32x4* xr = x + row * (int64_t)cols8;
-    for (int c = threadIdx.x; c < cols8; c += QT) {
-        const u32x4 v = xr[c];
-        float* dst = Xs + (c >> 4) * LD + (c & 15) * 8;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const f16x2 h = as_f16x2(v[w]);
-            dst[2 * w] = (float)narrow_f16((float)h[0] * hscale);
-            dst[2 * w + 1] = (float)narrow_f16((float)h[1] * hscale);
-        }
-    }
-    for (int i = threadIdx.x; i < H * H; i += QT) Mt[(i % H) * H + i / H] = (float)hadK[i];
-    __syncthreads();
-    const int d = threadIdx.x & 127, half = threadIdx.x >> 7;
-    for (int g0 = half * 4; g0 < H; g0 += 8) {
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        for (int h = 0; h < H; ++h) {
-            const f32x4 m4 = *(const f32x4*)(Mt + h * H + g0);
-            const float xv = Xs[h * LD + d];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = __builtin_fmaf(m4[e], xv, acc[e]);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) Ys[(g0 + e) * 128 + d] = (f16)acc[e];
-    }
-    __syncthreads();
-    u32 m = 0;
-    for (int c = threadIdx.x; c < cols8; c += QT) {
-        const u32 mi = absmax_bits8(*(const u32x4*)(Ys + c * 8));
-        m = m > mi ? m : mi;
-    }
-    m = wave_max_u32_dpp(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
-    const f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
-    if (threadIdx.x == 0) scale_out[row] = sh;
-    const float s = (float)sh;
-    u32* qr = q + row * (int64_t)cols8;
-    const bool lean = fast_quant_ok(m, s);
-    const FastRecip fr = make_fast_recip(lean ? s : 1.0f);
-    const bool fast = scale_fast_ok(s);
-    const float rs = fast ? 1.0f / s : 0.0f;
-    for (int c = threadIdx.x; c < cols8; c += QT) {
-        const u32x4 v = *(const u32x4*)(Ys + c * 8);
-        qr[c] = lean ? sym_codes8_fast(v, fr) : sym_codes8(v, s, rs, fast);
-        if (y) y[row * (int64_t)cols8 + c] = v;
-    }
-}
-
 // Any column count (odd included), any alignment: one workgroup per row, scalar accesses, the row
 // is read twice when the scale has to be derived.  Used only when the vector kernel's
 // preconditions (cols % 8 == 0, cols <= 32768, 16-byte aligned x, 4-byte aligned q) do not hold.
@@ -483,17 +409,9 @@ extern "C" int qr_heads_hadamard_quantize_f16_i4(const void* x, int64_t rows, in
     const bool table = hadK_or_null && heads % 4 == 0 && heads <= 64 && !pow2;
     if (head_dim != 128 || !(pow2 || table)) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 3)) return QR_E_ALIGN;
-    if (table) {
-        const size_t lds = ((size_t)((heads * 129 + 3) & ~3) + (size_t)heads * heads) * 4 + (size_t)heads * 256;
-        if (lds > 48 * 1024) {
-            hipError_t e = qr_allow_dynamic_lds((const void*)heads_matrix_quant_rows_kernel, lds);
-            if (e != hipSuccess) return (int)e;
-        }
-        heads_matrix_quant_rows_kernel<<<dim3((unsigned)rows), dim3(QT), lds, (hipStream_t)stream>>>(
-            (const u32x4*)x, heads, (const f16*)hadK_or_null, 1.0f / __builtin_sqrtf((float)heads), clip, (u32*)q,
-            (f16*)scales, (u32x4*)y_or_null);
-        return qr_launch_status();
-    }
+    if (table)
+        return qr_internal_heads_matrix_quantize(x, rows, heads, hadK_or_null, clip, q, scales, y_or_null,
+                                                 (hipStream_t)stream);
     dim3 grid((unsigned)((rows + QT / QR_WAVE - 1) / (QT / QR_WAVE))), block(QT);
     hipStream_t st = (hipStream_t)stream;
     const float hscale = 1.0f / __builtin_sqrtf((float)heads);
