@@ -193,6 +193,25 @@ int qr_linear_i4_f16_static(const void* A, const void* sA, const void* W, const 
                             void* stream);
 
 /*
+ * Linear4bit.forward (quarot/nn/linear.py:42-56) for prefill shapes on the FP6 matrix path: the same
+ * product and the same fp16 epilogue as qr_linear_i4_f16, bit for bit (every int4 code is a value of
+ * FP6 E3M2, products and sums stay integers below 2^24, so the fp32 accumulators are exact), at a higher
+ * matrix-instruction rate.  Both operands must first be converted to the 6-bit stage-major layout this
+ * kernel reads; the reference has no counterpart (its CUTLASS call takes the packed nibbles,
+ * quarot/kernels/gemm.cu:16-41).
+ *   qr_f6_bytes(rows, K): bytes of a converted operand (rows * K * 3 / 4; K % 64 == 0).
+ *   qr_convert_i4_f6: codes uint8 [rows, K/2] (16-byte aligned) -> out (8-byte aligned, qr_f6_bytes bytes).
+ *     Weights are converted once after loading, activations after the quantiser.
+ *   qr_linear_f6_f16: A6 = converted codes of x [M, K], W6 = converted weight [N, K] (both 16-byte
+ *     aligned, each below 4 GiB, else QR_E_UNSUPPORTED), sA fp16 [M], sW fp16 [N], bias fp16 [N] or NULL
+ *     -> y fp16 [M, N] (8-byte aligned).  Any M, N; meant for M >= 1024 (256 x 256 tiles).
+ */
+size_t qr_f6_bytes(int64_t rows, int64_t K);
+int qr_convert_i4_f6(const void* codes, int64_t rows, int64_t K, void* out, void* stream);
+int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, const void* sW,
+                     const void* bias_or_null, int64_t M, int64_t N, int64_t K, void* y, void* stream);
+
+/*
  * A whole quantised linear layer in one host call: the module chain
  *   torch.nn.Sequential(OnlineHadamard(K), Quantizer(clip), Linear4bit)        (had_K >= 1)
  *   torch.nn.Sequential(Quantizer(clip), Linear4bit)                           (had_K == 0)

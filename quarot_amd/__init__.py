@@ -17,7 +17,7 @@ from . import nn
 
 __all__ = [
     "matmul", "sym_quant", "sym_dequant", "PackedQuantizedTensor",      # the reference's names
-    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "heads_hadamard_quantize", "linear_i4", "quantized_linear",   # fused entry points
+    "quantize_rows", "hadamard_quantize", "rmsnorm_quantize", "heads_hadamard_quantize", "linear_i4", "quantized_linear", "convert_i4_f6", "linear_f6",   # fused entry points
 ]
 
 
@@ -249,6 +249,41 @@ def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
             _lib.check(L.qr_linear_i4_f16(_ptr(a2), _ptr(sx), _ptr(weight), _ptr(sw), _ptr(bias), M, N, K, _ptr(y),
                                           _lib.stream_ptr(dev)))
     return y.view(*lead, N)
+
+
+def convert_i4_f6(codes):
+    """Packed int4 codes uint8 [..., K/2] (K % 64 == 0) -> the 6-bit operand layout of linear_f6: uint8
+    [K/64, rows, 48], every code as its FP6 E3M2 value, stage-major.  For weights once after loading, for
+    activations after the quantiser."""
+    c2, lead = _flat2d(codes)
+    dev = _require_gpu_contiguous("convert_i4_f6", codes=c2)
+    rows, K = c2.shape[0], c2.shape[1] * 2
+    assert K % 64 == 0, "in_features: {} must be a multiple of 64".format(K)
+    out = torch.empty((K // 64, rows, 48), dtype=torch.uint8, device=dev)
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_convert_i4_f6(_ptr(c2), rows, K, _ptr(out), _lib.stream_ptr(dev)))
+    return out
+
+
+def linear_f6(x6, scales_x, weight6, weight_scales, bias=None):
+    """Linear4bit.forward (quarot/nn/linear.py:42-56) on operands converted by convert_i4_f6: the int4
+    product on the FP6 matrix path (exact: every code is an FP6 value, sums stay integers below 2^24) with the
+    same fused fp16 epilogue as linear_i4, bit for bit.  x6 [K/64, M, 48], weight6 [K/64, N, 48] -> fp16 [M, N]."""
+    assert scales_x.dtype == weight_scales.dtype == torch.float16
+    sx, sw = scales_x.view(-1), weight_scales.view(-1)
+    dev = _require_gpu_contiguous("linear_f6", x6=x6, scales_x=sx, weight6=weight6, weight_scales=sw, bias=bias)
+    if x6.dim() != 3 or weight6.dim() != 3 or x6.shape[0] != weight6.shape[0] or x6.shape[2] != 48 or weight6.shape[2] != 48:
+        raise RuntimeError("linear_f6: operands must be [K/64, rows, 48] from convert_i4_f6 with the same K")
+    M, N, K = x6.shape[1], weight6.shape[1], x6.shape[0] * 64
+    if sx.shape[0] != M or sw.shape[0] != N:
+        raise RuntimeError("linear_f6: inconsistent operand sizes")
+    if bias is not None and (bias.dtype != torch.float16 or bias.numel() != N):
+        raise RuntimeError("linear_f6: bias must be fp16 of size out_features")
+    y = torch.empty((M, N), dtype=torch.float16, device=dev)
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_linear_f6_f16(_ptr(x6), _ptr(sx), _ptr(weight6), _ptr(sw), _ptr(bias), M, N, K, _ptr(y),
+                                               _lib.stream_ptr(dev)))
+    return y
 
 
 @functools.lru_cache(maxsize=4096)

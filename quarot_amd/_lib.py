@@ -30,6 +30,9 @@ SIGNATURES = {
                                        _c.c_size_t, _ptr)),
     "qr_linear_i4_f16_ws": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr, _c.c_size_t, _ptr)),
     "qr_linear_i4_f16_static": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
+    "qr_f6_bytes": (_c.c_size_t, (_i64, _i64)),
+    "qr_convert_i4_f6": (_int, (_ptr, _i64, _i64, _ptr, _ptr)),
+    "qr_linear_f6_f16": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr)),
     "qr_kv_quant_f16_i4": (_int, (_ptr, _i64, _int, _int, _ptr, _ptr, _ptr, _ptr)),
     "qr_kv_dequant_i4_f16": (_int, (_ptr, _ptr, _ptr, _i64, _int, _ptr, _ptr)),
     "qr_kv_append_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int,

@@ -9,7 +9,7 @@ import sys
 PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libquarot_hip.so"
-SOURCES = ("api.hip", "quant.hip", "gemm.hip", "hadamard.hip", "kv.hip", "attn.hip")
+SOURCES = ("api.hip", "quant.hip", "gemm.hip", "gemm_f6.hip", "hadamard.hip", "kv.hip", "attn.hip")
 FLAGS = ("--offload-arch=gfx950", "-O3", "-fPIC", "-shared", "-std=c++17", "-fno-gpu-rdc",
          # every fp16/fp32 operation must round on its own (the reference's results are defined that
          # way): no fused multiply-add contraction unless a kernel spells fma out

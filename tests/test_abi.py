@@ -30,7 +30,8 @@ def test_header_declares_expected_entry_points():
     for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
                  "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
                  "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4", "qr_quantized_linear_workspace_bytes", "qr_quantized_linear_f16",
-                 "qr_workspace_bytes", "qr_linear_i4_f16_ws", "qr_linear_i4_f16_static"):
+                 "qr_workspace_bytes", "qr_linear_i4_f16_ws", "qr_linear_i4_f16_static", "qr_f6_bytes", "qr_convert_i4_f6",
+                 "qr_linear_f6_f16"):
         assert must in syms
 
 
@@ -91,6 +92,22 @@ def test_workspace_query_needs_no_gpu(lib):
     one = ctypes.c_void_p(16)
     assert lib.qr_linear_i4_f16_ws(one, None, one, one, None, 4, 4, 64, one, None, 0, None) == -1
     assert lib.qr_linear_i4_f16_ws(one, one, one, one, None, 4, 4, 100, one, None, 0, None) == -2
+
+
+def test_fp6_path_sizes_and_argument_errors_need_no_gpu(lib):
+    """The FP6 matrix path: a converted operand is 6 bits per value; argument errors come back before any launch."""
+    assert lib.qr_f6_bytes(2048, 11008) == 2048 * 11008 * 3 // 4
+    assert lib.qr_f6_bytes(0, 4096) == 0 and lib.qr_f6_bytes(16, 100) == 0
+    one = ctypes.c_void_p(16)
+    assert lib.qr_convert_i4_f6(one, 4, 100, one, None) == -2                   # K % 64 != 0
+    assert lib.qr_convert_i4_f6(None, 4, 64, one, None) == -1
+    assert lib.qr_convert_i4_f6(ctypes.c_void_p(8), 4, 64, one, None) == -4
+    assert lib.qr_convert_i4_f6(one, 0, 64, one, None) == 0
+    assert lib.qr_linear_f6_f16(one, one, one, one, None, 4, 4, 100, one, None) == -2
+    assert lib.qr_linear_f6_f16(one, None, one, one, None, 4, 4, 64, one, None) == -1
+    assert lib.qr_linear_f6_f16(ctypes.c_void_p(8), one, one, one, None, 4, 4, 64, one, None) == -4
+    assert lib.qr_linear_f6_f16(one, one, one, one, None, 1 << 20, 4, 8192, one, None) == -3   # operand beyond 32-bit offsets
+    assert lib.qr_linear_f6_f16(one, one, one, one, None, 0, 4, 64, one, None) == 0
 
 
 def test_quantized_linear_workspace_and_argument_errors_need_no_gpu(lib):

@@ -205,6 +205,78 @@ def test_decode_with_many_weight_rows_shares_the_tokens_through_lds(n):
             assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw))), (m, n, k)
 
 
+def f6_value(code):
+    """The real value of a 6-bit FP6 E3M2 code (sign, 3 exponent bits with bias 3, 2 mantissa bits)."""
+    s, e, f = code >> 5, (code >> 2) & 7, code & 3
+    mag = f * 0.0625 if e == 0 else (1 + f / 4) * 2.0 ** (e - 3)
+    return -mag if s else mag
+
+
+def test_fp6_conversion_holds_every_code_exactly():
+    """convert_i4_f6 against the format's definition: every 6-bit field of the converted operand decodes to
+    an int4 value, and each (row, stage, half) group of 32 fields holds exactly the 32 codes of that part of
+    the row (the order inside a group is the converter's own: both GEMM operands share it)."""
+    rng = np.random.default_rng(6)
+    rows, k = 37, 192
+    vals = rng.integers(-8, 8, (rows, k))
+    vals[0, :16] = np.arange(-8, 8)
+    out = quarot_amd.convert_i4_f6(gpu(o.pack_i4(vals))).cpu().numpy()
+    assert out.shape == (k // 64, rows, 48) and out.dtype == np.uint8
+    bits = np.unpackbits(out.reshape(k // 64, rows, 2, 24), axis=-1, bitorder="little")      # [stage, row, half, 192 bits]
+    for half in (0, 1):
+        b = bits[:, :, half, :]
+        if half == 1:                                       # stored as [last 8 bytes][first 16 bytes]
+            b = np.concatenate([b[..., 64:], b[..., :64]], axis=-1)
+        fields = (b.reshape(k // 64, rows, 32, 6) * (1 << np.arange(6))).sum(-1)
+        decoded = np.vectorize(f6_value)(fields)
+        for st in range(k // 64):
+            want = vals[:, st * 64 + half * 32: st * 64 + half * 32 + 32]
+            assert np.array_equal(np.sort(decoded[st], axis=-1), np.sort(want, axis=-1)), (st, half)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 64), (33, 65, 128), (256, 256, 64), (300, 520, 192), (257, 511, 320),
+                                   (1024, 768, 4096), (2048, 4096, 11008), (4100, 4090, 448)])
+def test_linear_on_the_fp6_matrix_path_bit_exact(m, n, k):
+    """qr_linear_f6_f16 on converted operands: the fused fp16 output against the oracle bit for bit (small shapes:
+    every element; large: the int8 path, itself checked against the oracle elsewhere, plus oracle rows), ragged
+    tiles, one and many K stages, extreme codes, with and without bias."""
+    rng = np.random.default_rng(m + n + k)
+    av, wv = rng.integers(-8, 8, (m, k)), rng.integers(-8, 8, (n, k))
+    av[0, :], wv[0, :] = -8, -8                          # the largest possible sum: 64 k
+    a, w = o.pack_i4(av), o.pack_i4(wv)
+    sa = (np.abs(rng.standard_normal(m)) * 0.2 + 0.01).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01 + 0.001).astype(F16)
+    bias = rng.standard_normal(n).astype(F16)
+    ga, gw, gsa, gsw, gb = gpu(a), gpu(w), gpu(sa), gpu(sw), gpu(bias)
+    a6, w6 = quarot_amd.convert_i4_f6(ga), quarot_amd.convert_i4_f6(gw)
+    for b, nb in ((gb, bias), (None, None)):
+        y = quarot_amd.linear_f6(a6, gsa, w6, gsw, b)
+        assert y.dtype == torch.float16 and y.shape == (m, n)
+        if m * n * k <= 1 << 27:
+            assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(o.int4_matmul(a, w), sa, sw, nb)))
+        else:
+            assert torch.equal(y, quarot_amd.linear_i4(ga, gsa, gw, gsw, b))
+            rows = sorted(set([0, m - 1] + [int(v) for v in rng.integers(0, m, 6)]))
+            want = o.sym_dequant(o.int4_matmul(a[rows], w), sa[rows], sw, nb)
+            assert np.array_equal(bits(y[rows].cpu().numpy()), bits(want))
+
+
+def test_linear4bit_opt_in_fp6_prefill_equals_the_default_path():
+    lin = quarot_amd.nn.Linear4bit(512, 384, bias=True).half().cuda()
+    rng = np.random.default_rng(5)
+    lin.weight.copy_(gpu(o.pack_i4(rng.integers(-8, 8, (384, 512)))))
+    lin.weight_scales.copy_(gpu((np.abs(rng.standard_normal((384, 1))) * 0.01 + 0.001).astype(F16)))
+    lin.bias.copy_(gpu(rng.standard_normal(384).astype(F16)))
+    x = quarot_amd.nn.Quantizer()(gpu(rng.standard_normal((600, 512)).astype(F16)))
+    want = lin(x)
+    lin.prefill_fp6, lin.fp6_min_rows = True, 256
+    assert torch.equal(lin(x), want)
+    lin.weight.copy_(gpu(o.pack_i4(rng.integers(-8, 8, (384, 512)))))      # new weights: the 6-bit copy is rebuilt
+    got = lin(x)
+    lin.prefill_fp6 = False
+    assert torch.equal(got, lin(x))
+
+
 def test_matmul_known_answers_and_leading_dims():
     k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
     a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
