@@ -73,21 +73,27 @@ __global__ __launch_bounds__(256) void convert_i4_f6_kernel(const u32x4* __restr
 }
 
 // ------------------------------------------------------------------------------------------------
-// 256 x 256 tile, four waves (one per SIMD) as 2 (M) x 2 (N), each a 128 x 128 wave tile = 16 accumulator
-// tiles of 32 x 32.  A stage is 64 k: 12 KB of X6 and 12 KB of W6, each one contiguous run, loaded
-// straight into LDS (buffer_load ... lds: a wave's 64 lanes fill 1 KB of consecutive LDS); six stage
-// buffers, loads five stages ahead.  Rows are 48 bytes apart in LDS: the 16 rows that a quarter-wave
+// TM x 256 tile (TM = 256, or 128 when 256-row tiles would leave compute units idle), four waves (one per
+// SIMD) as 2 (M) x 2 (N), each a TM/2 x 128 wave tile = TM/64 x 4 accumulator tiles of 32 x 32.  A stage
+// is 64 k: TM * 48 bytes of X6 and 12 KB of W6, each one contiguous run, loaded straight into LDS
+// (buffer_load ... lds: a wave's 64 lanes fill 1 KB of consecutive LDS); six stage buffers, loads five
+// stages ahead.  (At TM = 128 the X6 run is 1.5 rounds of the workgroup's 4 KB: waves 2 and 3 aim the
+// second round past the end of the operand, which fetches nothing, and at a spare 2 KB of LDS, so that
+// every wave has the same number of loads in flight and one wait count serves all.)  Rows are 48 bytes apart in LDS: the 16 rows that a quarter-wave
 // reads at one offset start in 16 different groups of four banks (12 r mod 64), so the 16-byte and 8-byte
 // reads that assemble an operand (24 bytes: halves of the row at byte 0 / 16 and 32 / 24) have no bank
 // conflicts and nothing is padded or swizzled.  Nothing is unpacked: fragments go from LDS to the
 // matrix instruction; the fragments of the next stage are read while the 16 MFMAs of the current one run.
-template <bool DEQ_BIAS>
+template <int TM, bool DEQ_BIAS>
 __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict__ A6, const uint8_t* __restrict__ B6, int M,
                                                       int N, int stages, f16* __restrict__ Y, const f16* __restrict__ sA,
                                                       const f16* __restrict__ sB, const f16* __restrict__ bias, int tiles_m,
                                                       int tiles_n, int nxcd) {
     constexpr int NBUF = 6, AHEAD = 5;
-    constexpr int BUF = 1536;                               // 16-byte slots per stage buffer: 768 of X6, 768 of W6
+    constexpr int IM = TM / 64;                             // accumulator tiles of a wave along M
+    constexpr int ASLOTS = TM * 3, AROUNDS = (ASLOTS + 255) / 256;
+    constexpr int BUF = ASLOTS + 768;                       // 16-byte slots per stage buffer: X6, then 768 of W6
+    constexpr int LOADS = AROUNDS + 3;                      // loads per wave and stage
     extern __shared__ u32x4 f6_lds[];
     const int per_xcd = gridDim.x / nxcd;
     const int tile = (blockIdx.x % nxcd) * per_xcd + blockIdx.x / nxcd;
@@ -99,7 +105,7 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
     const int gh = (tiles_m - gm0) < GROUP_M ? (tiles_m - gm0) : GROUP_M;
     const int tm = gm0 + (tile - g * group_sz) % gh;
     const int tn = (tile - g * group_sz) / gh;
-    const int m0 = tm * 256, n0 = tn * 256;
+    const int m0 = tm * TM, n0 = tn * 256;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -113,21 +119,26 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
         const int sc = st < stages ? st : stages - 1;       // past the end: repeat the last stage into a buffer nobody reads
         const u32 sa = ((u32)sc * (u32)M + (u32)m0) * 48u, sb = ((u32)sc * (u32)N + (u32)n0) * 48u;
 #pragma unroll
+        for (int i = 0; i < AROUNDS; ++i) {
+            const bool spare = (i * 256 + 256 > ASLOTS) && wave >= (ASLOTS - i * 256) / 64;    // wave-uniform
+            __attribute__((address_space(3))) void* da = (__attribute__((address_space(3))) void*)(
+                spare ? f6_lds + NBUF * BUF + (wave & 1) * 64 : f6_lds + buf * BUF + i * 256 + wave * 64);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, da, 16, spare ? 0xFFFFFF00u : (u32)(tid * 16 + i * 4096),
+                                                     spare ? 0u : sa, 0, 0);
+        }
+#pragma unroll
         for (int i = 0; i < 3; ++i) {
-            __attribute__((address_space(3))) void* da =
-                (__attribute__((address_space(3))) void*)(f6_lds + buf * BUF + i * 256 + wave * 64);
             __attribute__((address_space(3))) void* db =
-                (__attribute__((address_space(3))) void*)(f6_lds + buf * BUF + 768 + i * 256 + wave * 64);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, da, 16, (u32)(tid * 16 + i * 4096), sa, 0, 0);
+                (__attribute__((address_space(3))) void*)(f6_lds + buf * BUF + ASLOTS + i * 256 + wave * 64);
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, db, 16, (u32)(tid * 16 + i * 4096), sb, 0, 0);
         }
     };
     // fragment (row, kh): 16 bytes at row * 48 + (kh ? 32 : 0) and 8 bytes at row * 48 + (kh ? 24 : 16)
     struct Frags {
-        i32x8 a[4], b[4];
+        i32x8 a[IM], b[4];
     };
-    const int a16 = (wm * 128 + r) * 3 + (kh ? 2 : 0), a8 = (wm * 128 + r) * 6 + (kh ? 3 : 2);
-    const int b16 = 768 + (wn * 128 + r) * 3 + (kh ? 2 : 0), b8 = 1536 + (wn * 128 + r) * 6 + (kh ? 3 : 2);
+    const int a16 = (wm * (TM / 2) + r) * 3 + (kh ? 2 : 0), a8 = (wm * (TM / 2) + r) * 6 + (kh ? 3 : 2);
+    const int b16 = ASLOTS + (wn * 128 + r) * 3 + (kh ? 2 : 0), b8 = ASLOTS * 2 + (wn * 128 + r) * 6 + (kh ? 3 : 2);
     auto read_a = [&](int buf, int t, Frags& f) {
         const u32x4 q = f6_lds[buf * BUF + a16 + t * 96];
         const u32x2 e = ((const u32x2*)f6_lds)[buf * BUF * 2 + a8 + t * 192];
@@ -138,9 +149,9 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
         const u32x2 e = ((const u32x2*)f6_lds)[buf * BUF * 2 + b8 + t * 192];
         f.b[t] = i32x8{(int)q[0], (int)q[1], (int)q[2], (int)q[3], (int)e[0], (int)e[1], 0, 0};
     };
-    f32x16 acc[4][4];
+    f32x16 acc[IM][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < IM; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -149,27 +160,26 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
 #define QR_F6_BARRIER(ALLOWED) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(ALLOWED) : "memory")
 #pragma unroll
     for (int s = 0; s < AHEAD; ++s) dma(s, s);
-    QR_F6_BARRIER(18);                                      // stages 0 and 1 have landed (three stages of 6 loads may be out)
+    QR_F6_BARRIER(3 * LOADS);                               // stages 0 and 1 have landed (three stages of loads may be out)
     Frags fr[2];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-        read_a(0, t, fr[0]);
-        read_b(0, t, fr[0]);
-    }
-    // One stage: the 16 MFMAs of `cur`, one fragment read of the next stage (already landed: the barrier
-    // before this stage waited for it) behind each of the first eight, the loads of stage s + 5 into the
+    for (int t = 0; t < IM; ++t) read_a(0, t, fr[0]);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) read_b(0, t, fr[0]);
+    // One stage: the IM * 4 MFMAs of `cur`, one fragment read of the next stage (already landed: the barrier
+    // before this stage waited for it) behind each of the first IM + 4, the loads of stage s + 5 into the
     // buffer of stage s - 1 (last read during stage s - 2) behind the next ones.
     auto stage = [&](int s, int bnext, int bfill, const Frags& cur, Frags& nxt) {
 #pragma unroll
-        for (int q = 0; q < 16; ++q) {
+        for (int q = 0; q < IM * 4; ++q) {
             const int i = q >> 2, j = q & 3;
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.b[j], cur.a[i], acc[i][j], 3, 3, 0, 127, 0, 127);
-            if (q < 4) read_a(bnext, q, nxt);
-            else if (q < 8) read_b(bnext, q - 4, nxt);
-            if (q == 8) dma(s + AHEAD, bfill);
+            if (q < IM) read_a(bnext, q, nxt);
+            else if (q < IM + 4) read_b(bnext, q - IM, nxt);
+            if (q == (IM == 4 ? 8 : 6)) dma(s + AHEAD, bfill);
             __builtin_amdgcn_sched_barrier(0);
         }
-        QR_F6_BARRIER(18);                                  // stage s + 2 has landed; every wave is done reading stage s
+        QR_F6_BARRIER(3 * LOADS);                                 // stage s + 2 has landed; every wave is done reading stage s
     };
     int b = 0;                                              // buffer of the current stage
     auto next = [](int v) { return v == NBUF - 1 ? 0 : v + 1; };
@@ -189,8 +199,8 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
 
     // ---- epilogue: lane l, register v -> column (v/4)*8 + (l/32)*4 + v%4 of the W tile, token l%32
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row0 = m0 + wm * 128 + i * 32;
+    for (int i = 0; i < IM; ++i) {
+        const int row0 = m0 + wm * (TM / 2) + i * 32;
         const int row = row0 + r;
         const bool rows_whole = row0 + 32 <= M;
 #pragma unroll
@@ -261,27 +271,25 @@ extern "C" int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, 
     if (!A6 || !W6 || !sA || !sW || !y) return QR_E_NULL;
     if (((uintptr_t)A6 & 15) || ((uintptr_t)W6 & 15) || ((uintptr_t)y & 7)) return QR_E_ALIGN;
     // operands are addressed through 32-bit buffer offsets
-    if ((double)M * (double)K * 0.75 >= 4294967296.0 || (double)N * (double)K * 0.75 >= 4294967296.0) return QR_E_UNSUPPORTED;
-    const int tiles_m = (int)((M + 255) / 256), tiles_n = (int)((N + 255) / 256);
+    if ((double)M * (double)K * 0.75 >= 4294901760.0 || (double)N * (double)K * 0.75 >= 4294901760.0) return QR_E_UNSUPPORTED;
+    const int nxcd = qr_device().xcds, cus = qr_device().cus;
+    const int tiles_n = (int)((N + 255) / 256);
+    // 256-row tiles unless 128-row ones fill the device in fewer rounds (a 128-row tile costs ~0.6 of a 256-row one)
+    const int64_t t256 = (M + 255) / 256 * tiles_n, t128 = (M + 127) / 128 * tiles_n;
+    const bool narrow = (double)((t128 + cus - 1) / cus) * 0.6 < (double)((t256 + cus - 1) / cus);
+    const int tiles_m = (int)(narrow ? (M + 127) / 128 : (M + 255) / 256);
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
-    const int nxcd = qr_device().xcds;
     const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
-    constexpr size_t LDS = (size_t)6 * 1536 * 16;
     hipStream_t st = (hipStream_t)stream;
-    hipError_t e;
-    if (bias_or_null) {
-        e = qr_allow_dynamic_lds((const void*)gemm_f6_kernel<true>, LDS);
+    auto launch = [&](auto kernel, size_t lds) -> int {
+        hipError_t e = qr_allow_dynamic_lds((const void*)kernel, lds);
         if (e != hipSuccess) return (int)e;
-        gemm_f6_kernel<true><<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A6, (const uint8_t*)W6, (int)M, (int)N,
-                                                                 (int)(K / 64), (f16*)y, (const f16*)sA, (const f16*)sW,
-                                                                 (const f16*)bias_or_null, tiles_m, tiles_n, nxcd);
-    } else {
-        e = qr_allow_dynamic_lds((const void*)gemm_f6_kernel<false>, LDS);
-        if (e != hipSuccess) return (int)e;
-        gemm_f6_kernel<false><<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A6, (const uint8_t*)W6, (int)M, (int)N,
-                                                                  (int)(K / 64), (f16*)y, (const f16*)sA, (const f16*)sW, nullptr,
-                                                                  tiles_m, tiles_n, nxcd);
-    }
-    return qr_launch_status();
+        kernel<<<dim3(grid), dim3(256), lds, st>>>((const uint8_t*)A6, (const uint8_t*)W6, (int)M, (int)N, (int)(K / 64), (f16*)y,
+                                                   (const f16*)sA, (const f16*)sW, (const f16*)bias_or_null, tiles_m, tiles_n, nxcd);
+        return qr_launch_status();
+    };
+    constexpr size_t LDS256 = (size_t)6 * (768 + 768) * 16, LDS128 = (size_t)(6 * (384 + 768) + 128) * 16;
+    if (narrow) return bias_or_null ? launch(gemm_f6_kernel<128, true>, LDS128) : launch(gemm_f6_kernel<128, false>, LDS128);
+    return bias_or_null ? launch(gemm_f6_kernel<256, true>, LDS256) : launch(gemm_f6_kernel<256, false>, LDS256);
 }

@@ -235,7 +235,7 @@ def test_fp6_conversion_holds_every_code_exactly():
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1, 64), (33, 65, 128), (256, 256, 64), (300, 520, 192), (257, 511, 320),
-                                   (1024, 768, 4096), (2048, 4096, 11008), (4100, 4090, 448)])
+                                   (1024, 768, 4096), (2048, 4096, 11008), (4100, 4090, 448), (8200, 8190, 128)])
 def test_linear_on_the_fp6_matrix_path_bit_exact(m, n, k):
     """qr_linear_f6_f16 on converted operands: the fused fp16 output against the oracle bit for bit (small shapes:
     every element; large: the int8 path, itself checked against the oracle elsewhere, plus oracle rows), ragged
