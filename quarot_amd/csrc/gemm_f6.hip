@@ -158,9 +158,18 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
 #define QR_F6_BARRIER(ALLOWED) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(ALLOWED) : "memory")
+    // The epilogue's scales (and bias) of this tile's columns and rows are fetched first and parked in LDS
+    // behind the stage buffers, so that the epilogue finds them without waiting for memory (indices clamped
+    // to the matrix: values of rows and columns beyond it are never stored).
+    f16* const scale_lds = (f16*)(f6_lds + NBUF * BUF + (TM == 128 ? 128 : 0));     // [256] sB, [256] bias, [TM] sA
+    const int ccol = n0 + tid < N ? n0 + tid : N - 1, crow = m0 + tid < M ? m0 + tid : M - 1;
+    const f16 pre_sb = sB[ccol], pre_bi = DEQ_BIAS ? bias[ccol] : (f16)0, pre_sa = sA[crow];
 #pragma unroll
     for (int s = 0; s < AHEAD; ++s) dma(s, s);
     QR_F6_BARRIER(3 * LOADS);                               // stages 0 and 1 have landed (three stages of loads may be out)
+    scale_lds[tid] = pre_sb;                                // (published by the barriers of the K loop)
+    scale_lds[256 + tid] = pre_bi;
+    if (tid < TM) scale_lds[512 + tid] = pre_sa;
     Frags fr[2];
 #pragma unroll
     for (int t = 0; t < IM; ++t) read_a(0, t, fr[0]);
@@ -173,7 +182,7 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
 #pragma unroll
         for (int q = 0; q < IM * 4; ++q) {
             const int i = q >> 2, j = q & 3;
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.b[j], cur.a[i], acc[i][j], 3, 3, 0, 127, 0, 127);
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.b[j], cur.a[i], acc[i][j], 3, 3, 0, 0, 0, 0);
             if (q < IM) read_a(bnext, q, nxt);
             else if (q < IM + 4) read_b(bnext, q - IM, nxt);
             if (q == (IM == 4 ? 8 : 6)) dma(s + AHEAD, bfill);
@@ -198,33 +207,32 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
     __syncthreads();                                        // ... before the stage buffers become output slabs
 
     // ---- epilogue: lane l, register v -> column (v/4)*8 + (l/32)*4 + v%4 of the W tile, token l%32
+    f16x4 sbh[4][4], bih[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            const int c = wn * 128 + j * 32 + gq * 8 + kh * 4;
+            sbh[j][gq] = *(const f16x4*)(scale_lds + c);
+            bih[j][gq] = *(const f16x4*)(scale_lds + 256 + c);
+        }
+    const bool lines = (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
 #pragma unroll
     for (int i = 0; i < IM; ++i) {
         const int row0 = m0 + wm * (TM / 2) + i * 32;
         const int row = row0 + r;
-        const bool rows_whole = row0 + 32 <= M;
+        const f16 sa = scale_lds[512 + wm * (TM / 2) + i * 32 + r];
 #pragma unroll
         for (int jb = 0; jb < 4; jb += 2) {
             const int col0 = n0 + wn * 128 + jb * 32;
-            const bool by_rows = rows_whole && col0 + 64 <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
             f16x4 o[2][4];
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-                for (int gq = 0; gq < 4; ++gq) {
-                    const int col = col0 + jj * 32 + gq * 8 + kh * 4;
-                    f16x4 sb4, bi4;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int cc = col + e < N ? col + e : N - 1;
-                        sb4[e] = sB[cc];
-                        bi4[e] = DEQ_BIAS ? bias[cc] : (f16)0;
-                    }
-                    const f16 sa = sA[row < M ? row : M - 1];
+                for (int gq = 0; gq < 4; ++gq)
                     o[jj][gq] = dequant4_f32(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
-                                             acc[i][jb + jj][gq * 4 + 3], sa, sb4, bi4, DEQ_BIAS);
-                }
-            if (by_rows) {
+                                             acc[i][jb + jj][gq * 4 + 3], sa, sbh[jb + jj][gq], bih[jb + jj][gq], DEQ_BIAS);
+            if (lines && row0 + 32 <= M && col0 + 64 <= N) {
                 store_slab_rows<2>((u32x2*)(f6_lds + wave * 256), o, lane, Y + (int64_t)row0 * N + col0, N);
             } else if (row < M) {
 #pragma unroll
@@ -289,7 +297,8 @@ extern "C" int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, 
                                                    (const f16*)sA, (const f16*)sW, (const f16*)bias_or_null, tiles_m, tiles_n, nxcd);
         return qr_launch_status();
     };
-    constexpr size_t LDS256 = (size_t)6 * (768 + 768) * 16, LDS128 = (size_t)(6 * (384 + 768) + 128) * 16;
+    // six stage buffers (+ the spare 2 KB that idle loads of 128-row tiles aim at) + 1.5 KB of scales for the epilogue
+    constexpr size_t LDS256 = (size_t)(6 * (768 + 768) + 96) * 16, LDS128 = (size_t)(6 * (384 + 768) + 128 + 96) * 16;
     if (narrow) return bias_or_null ? launch(gemm_f6_kernel<128, true>, LDS128) : launch(gemm_f6_kernel<128, false>, LDS128);
     return bias_or_null ? launch(gemm_f6_kernel<256, true>, LDS256) : launch(gemm_f6_kernel<256, false>, LDS256);
 }
