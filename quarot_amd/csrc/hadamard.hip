@@ -1426,11 +1426,22 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
 
 // ---- K > 1 with a long power-of-two factor (m = 512 or 1024), fp16 I/O ---------------------------
 // Decode-sized inputs have few rows, so the row itself must supply the parallelism: 1024 threads per
-// row.  A wave transforms whole segments in registers (8 values per chunk, 64 lanes, CPL chunks per
-// lane: 3 + 6 + log2(CPL) butterfly levels, no LDS), scatters the scaled fp16 results into LDS in
-// MFMA-fragment order, and the hadK factor then runs on the matrix cores as in hadamard_mm_kernel
-// (T^T as first operand, hadK fragments in registers, 8-byte result writes).  All of a row's loads are
-// issued at once and the next row's are requested before the matrix stage.
+// row.  The power-of-two factor comes first, segment by segment (a segment = the m values of one k):
+//   m = 1024 on the matrix cores, as H_32 (x) H_32 over the segment viewed as [b][c] = [32][32]:
+//     stage A  T[b][c'] = sum_c X[b][c] H_32[c][c']: the first operand is a 16 x 32 tile of X exactly as
+//              it lies in memory (16 bytes per lane, 1 KB per wave and load), fp32 accumulation;
+//     stage B  U[b'][c'] = sum_b H_32[b'][b] T[b][c']: with the contraction index taken in the order
+//              b = 16 (t / 4) + 4 (lane / 16) + t % 4, the accumulators of stage A's two row tiles ARE the
+//              second operand (no exchange between lanes); T is split into fp16 hi + lo (two MFMAs), so
+//              the result has fp32 accuracy and is rounded to fp16 once, after the scale, as in the
+//              butterfly form;
+//     a wave takes four k and one half of c', and packs its four results per position into one 8-byte
+//     LDS write in the fragment order of the hadK stage;
+//   m = 512 with butterflies in registers (8 values per chunk, 64 lanes: 3 + 6 levels, no LDS), scattered
+//     into the same order as 2-byte writes.
+// The hadK factor then runs on the matrix cores as in hadamard_mm_kernel (T^T as first operand, hadK
+// fragments in registers, 8-byte result writes).  All of a row's loads are issued at once and the next
+// row's are requested before the matrix stage.
 template <bool QUANT, int CPL>
 __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict__ x, f16* __restrict__ y, int64_t rows,
                                                            int n, int K, const f16* __restrict__ hadK, float scale,
@@ -1468,22 +1479,84 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
     // slots of T for k >= K are never written afterwards: clear once
     for (int i = tid; i < KS2 * 4 * CT * TS; i += BT) Tl[i] = u32x4{0, 0, 0, 0};
 
-    u32x4 raw[SPW][CPL];
+    // m = 1024: unit (wave / 2) = four k, wave % 2 = the half of c'; Sylvester fragments of both stages
+    constexpr int XL = CPL == 2 ? 8 : SPW * CPL;
+    const int unit = wave >> 1, cth = wave & 1;
+    const bool works = CPL == 2 && unit * 4 < K;
+    f16x8 ha, hb[2];
+    if (CPL == 2) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            ha[t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+            const int b = 16 * (t >> 2) + 4 * g + (t & 3);
+#pragma unroll
+            for (int bt = 0; bt < 2; ++bt) hb[bt][t] = (__builtin_popcount(b & (bt * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+        }
+    }
+    u32x4 raw[XL];
     auto request = [&](int64_t row) {
+        if (CPL == 2) {
+#pragma unroll
+            for (int ai = 0; ai < 4; ++ai)
+#pragma unroll
+                for (int bt = 0; bt < 2; ++bt)
+                    raw[ai * 2 + bt] = works ? *((const u32x4*)(x + row * (int64_t)n) + (unit * 4 + ai) * 128 + bt * 64 + l16 * 4 + g)
+                                             : u32x4{0, 0, 0, 0};
+            return;
+        }
 #pragma unroll
         for (int sg = 0; sg < SPW; ++sg) {
             const int k = wave + NW * sg;
 #pragma unroll
             for (int i = 0; i < CPL; ++i)
-                raw[sg][i] = k < K ? *((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
-                                   : u32x4{0, 0, 0, 0};
+                raw[sg * CPL + i] = k < K ? *((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
+                                          : u32x4{0, 0, 0, 0};
         }
     };
     int64_t row = blockIdx.x;
     if (row < rows) request(row);
     __syncthreads();
     for (; row < rows; row += gridDim.x) {
-        // ---- phase 1: per-segment transform in registers, scatter to fragment order
+        // ---- phase 1: the power-of-two factor of every segment, results in fragment order in LDS
+        if (CPL == 2) {
+            if (works) {
+                u32 o[4][2][2];                          // [k of the unit][b' tile][pair of e]: fp16 pairs
+#pragma unroll
+                for (int ai = 0; ai < 4; ++ai) {
+                    f16x8 thi, tlo;
+#pragma unroll
+                    for (int bt = 0; bt < 2; ++bt) {
+                        const f32x4 da = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, raw[ai * 2 + bt]), ha,
+                                                                              f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const f16 hi = narrow_f16(da[e]);
+                            thi[bt * 4 + e] = hi;
+                            tlo[bt * 4 + e] = narrow_f16(da[e] - (float)hi);
+                        }
+                    }
+#pragma unroll
+                    for (int bt = 0; bt < 2; ++bt) {
+                        f32x4 db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], thi, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], tlo, db, 0, 0, 0);
+                        o[ai][bt][0] = narrow_f16x2(db[0] * scale, db[1] * scale);
+                        o[ai][bt][1] = narrow_f16x2(db[2] * scale, db[3] * scale);
+                    }
+                }
+                // position (b' = 16 bt + 4 g + e, c' = 16 cth + l16) = column tile 2 b' + cth, column l16
+                u32x2* const dst = (u32x2*)(Tl + ((unit >> 1) * CT + cth) * TS + l16) + (unit & 1);
+#pragma unroll
+                for (int bt = 0; bt < 2; ++bt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const u32 sel = (e & 1) ? 0x07060302u : 0x05040100u;      // high or low halves of two dwords
+                        u32x2 v;
+                        v[0] = __builtin_amdgcn_perm(o[1][bt][e >> 1], o[0][bt][e >> 1], sel);
+                        v[1] = __builtin_amdgcn_perm(o[3][bt][e >> 1], o[2][bt][e >> 1], sel);
+                        dst[(2 * (16 * bt + 4 * g + e)) * TS * 2] = v;
+                    }
+            }
+        } else {
 #pragma unroll
         for (int sg = 0; sg < SPW; ++sg) {
             const int k = wave + NW * sg;
@@ -1493,8 +1566,8 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                 for (int i = 0; i < CPL; ++i) {
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        v[i][2 * w] = (float)f16_from_bits((unsigned short)(raw[sg][i][w] & 0xffffu));
-                        v[i][2 * w + 1] = (float)f16_from_bits((unsigned short)(raw[sg][i][w] >> 16));
+                        v[i][2 * w] = (float)f16_from_bits((unsigned short)(raw[sg * CPL + i][w] & 0xffffu));
+                        v[i][2 * w + 1] = (float)f16_from_bits((unsigned short)(raw[sg * CPL + i][w] >> 16));
                     }
                     reg_fwht8(v[i]);
                     lane_stage<1>(v[i], lane);
@@ -1503,14 +1576,6 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                     lane_stage<8>(v[i], lane);
                     lane_stage<16>(v[i], lane);
                     lane_stage<32>(v[i], lane);
-                }
-                if (CPL == 2) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float a = v[0][e], b = v[CPL - 1][e];
-                        v[0][e] = a + b;
-                        v[CPL - 1][e] = a - b;
-                    }
                 }
                 const int ks = k >> 5, kgp = (k & 31) >> 3, kj = k & 7;
 #pragma unroll
@@ -1521,6 +1586,7 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                     for (int e = 0; e < 8; ++e) dst[e * 8] = narrow_f16(v[i][e] * scale);
                 }
             }
+        }
         }
         const int64_t nrow = row + gridDim.x;
         if (nrow < rows) request(nrow);
