@@ -75,8 +75,10 @@ WORKLOADS = {
 for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
-PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d"]
+PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
+              "c2_fp6", "c3d_fp6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
+FP6_MFMA_PEAK_TOPS = 10100.0     # MI355X dense fp6, published (the opt-in exact int4 GEMM on 6-bit operands)
 HBM_PEAK_GBS = 8000.0
 
 # Profile summaries that hold the FETCH_SIZE / WRITE_SIZE readings of a workload's dominant kernel
@@ -93,6 +95,7 @@ PROFILE_OF = {
     "c6": "paged_decode_i4_c6_decode_attention_32x4096x8x128.txt",
     "b13v": "gemm_sp256_b13v_2048x5120x5120.txt", "b70v": "gemm_sp256_b70v_2048x8192x8192.txt",
     "b13d": "gemm_sp256_b13d_2048x13824x5120.txt", "b70d": "gemm_sp256_b70d_2048x28672x8192.txt",
+    "c2_fp6": "gemm_f6_c2_down_proj_7b.txt", "c3d_fp6": "gemm_f6_c3d_down_proj_32768_tokens.txt",
 }
 
 
@@ -203,10 +206,11 @@ class LinearWorkload:
     """One quantised linear layer: front (quantiser, optionally behind a Hadamard / RMSNorm / heads
     Hadamard) + Linear4bit, operands resident in HBM."""
 
-    def __init__(self, name, dev, on_gpu_data=False):
+    def __init__(self, name, dev, on_gpu_data=False, fp6=False):
         import quarot_amd
         self.q = quarot_amd
         self.name = name
+        self.fp6 = fp6
         self.m, self.k, self.n, self.front_kind = WORKLOADS[name]
         m, k, n = self.m, self.k, self.n
         self.decode = m <= 64
@@ -234,7 +238,12 @@ class LinearWorkload:
         self.i = 0
         # front kernel and GEMM go out in ONE call into the library (decode steps, and the shorter prefill
         # steps, are otherwise bound by the host's per-call cost)
-        self.one_call = self.front_kind in ("had", "quant")
+        self.one_call = self.front_kind in ("had", "quant") and not fp6
+        if fp6:
+            # the opt-in FP6 matrix path: the step converts the activations' codes and runs the GEMM on 6-bit
+            # operands (the weights' 6-bit copy is made once, at the first call)
+            assert not self.decode and k % 64 == 0
+            self.lin.prefill_fp6, self.lin.fp6_min_rows = True, 0
         self.had_args = (self.front.had_rem_dim, self.front.rem_dim) if self.front_kind == "had" else (None, 0)
         self.ops = 2.0 * m * n * k
 
@@ -244,12 +253,16 @@ class LinearWorkload:
         return w
 
     def step(self):
+        if self.fp6:
+            return self.lin(self.front(self.x))
         if self.one_call:
             return self.q.quantized_linear(self.x, self.weight(), self.lin.weight_scales, self.lin.bias, *self.had_args)
         p = self.front(self.x)
         return self.q.linear_i4(p.quantized_x, p.scales_x, self.weight(), self.lin.weight_scales, self.lin.bias)
 
     def gemm(self, p):
+        if self.fp6:
+            return self.q.linear_f6(self.p6, p.scales_x, self.lin._weight_f6(), self.lin.weight_scales, self.lin.bias)
         return self.q.linear_i4(p.quantized_x, p.scales_x, self.weight(), self.lin.weight_scales, self.lin.bias)
 
     def staged_step(self):
@@ -272,6 +285,9 @@ class LinearWorkload:
         """(front kernel ms, GEMM kernel ms), each from a pass of its own (decode: the weights still
         rotating among their copies)."""
         p = self.front(self.x)
+        if self.fp6:
+            self.p6 = self.q.convert_i4_f6(p.quantized_x)
+            self.convert_ms = kernel_ms(lambda: self.q.convert_i4_f6(p.quantized_x), reps)
         return kernel_ms(lambda: self.front(self.x), reps), kernel_ms(lambda: self.gemm(p), reps)
 
     def front_bytes(self):
@@ -282,13 +298,16 @@ class LinearWorkload:
         return n * k / 2 + m * k / 2 + 2 * m + 2 * n + 2 * m * n
 
     def rooflines(self, front_ms, gemm_ms):
-        kern = gemm_kernel_name(self.m, self.n)
-        if self.decode:
+        kern = "gemm_f6_kernel" if self.fp6 else gemm_kernel_name(self.m, self.n)
+        if self.fp6:
+            g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": FP6_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                 "convert_kernel_ms": round(self.convert_ms, 5)}
+        elif self.decode:
             g = {"bound": "hbm", "achieved": round(self.gemm_bytes() / (gemm_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
         else:
             g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s"}
         g["frac"] = round(g["achieved"] / g["peak"], 4)
-        g["kernel"] = kern + " (int4 GEMM + dequant epilogue)"
+        g["kernel"] = kern + (" (exact int4 GEMM on FP6 operands + dequant epilogue)" if self.fp6 else " (int4 GEMM + dequant epilogue)")
         g["kernel_ms"] = round(gemm_ms, 5)
         f = {"bound": "hbm", "achieved": round(self.front_bytes() / (front_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
              "kernel": FRONT_KERNEL[self.front_kind], "kernel_ms": round(front_ms, 5)}
@@ -302,8 +321,8 @@ class LinearWorkload:
         return f"{self.name}: Linear4bit X[{self.m},{self.k}] fp16 ({data}) . W int4[{self.n},{self.k}]" + tail
 
 
-def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, graph=False):
-    wl = LinearWorkload(name, dev, on_gpu_data)
+def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, graph=False, fp6=False):
+    wl = LinearWorkload(name, dev, on_gpu_data, fp6=fp6)
     extra = {}
     if graph:
         # one graph per weight copy would defeat the rotation: capture a run of len(copies) steps
@@ -323,14 +342,15 @@ def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, grap
         extra["launch"] = "hip graph replay"
     else:
         loops = timed_loops(wl.step, steps, warmup, repeats)
-        extra["launch"] = "eager" + (" (one library call per step)" if wl.one_call else "")
+        extra["launch"] = "eager" + (" (one library call per step)" if wl.one_call else "") + (
+            " (front, conversion to 6-bit operands, GEMM)" if wl.fp6 else "")
     sp = spread(loops)
     ms = sp["median_ms"]
     front_ms, gemm_ms = wl.kernel_times(kernel_reps)
     groof, froof = wl.rooflines(front_ms, gemm_ms)
     staged = timed_loops(wl.staged_step, max(5, steps // 4), 3, min(repeats, 3))
     res = {"ms": ms, "value": round(wl.ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": groof,
-           "front": froof, "kernels_ms_sum": round(front_ms + gemm_ms, 5),
+           "front": froof, "kernels_ms_sum": round(front_ms + gemm_ms + (wl.convert_ms if wl.fp6 else 0.0), 5),
            "staged_reference_api_ms": round(float(np.median(staged)), 5), "workload": wl.describe(), **extra}
     return wl, res
 
@@ -538,6 +558,9 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time replays of the step captured in a HIP graph (decode steps are host-launch-bound when "
                          "launched eagerly from Python); the first replay is checked against the eager result")
+    ap.add_argument("--fp6", action="store_true",
+                    help="prefill linear workloads only: run the GEMM on the opt-in FP6 matrix path (Linear4bit.prefill_fp6); "
+                         "the step then includes the conversion of the activations' codes to 6-bit operands")
     ap.add_argument("--cpu-rows", type=int, default=64)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of a workload, run a plain 256 MiB device copy 20 times (known traffic: 256 MiB read, "
@@ -548,6 +571,9 @@ def main():
               "run one process per GPU and add the values (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
 
+    if args.fp6 and (WORKLOADS[args.workload] is None or WORKLOADS[args.workload][0] <= 64):
+        print("--fp6 applies to the prefill linear workloads (c1, c2, c3a-c3d, b13*, b70*)", file=sys.stderr)
+        sys.exit(2)
     from quarot_amd import _lib
     if not _lib.LIB_PATH.exists():
         from quarot_amd import build
@@ -566,6 +592,8 @@ def main():
     def measure(name, headline):
         """headline: the protocol's full step / repeat counts; per-config: a fifth of the steps (at least 20 per
         loop, at most ~60 ms of GPU time per loop) and 5 loops."""
+        fp6 = name.endswith("_fp6") or (args.fp6 and headline)      # per-config names "<workload>_fp6": the opt-in FP6 matrix path
+        name = name[:-4] if name.endswith("_fp6") else name
         spec = WORKLOADS[name]
         big = name.startswith("c3") or name in ("c5", "c6")
         steps = args.steps if headline else max(20, args.steps // 5)
@@ -581,12 +609,12 @@ def main():
         if name in ("c6", "c6b"):
             return None, run_attention(name, dev, steps, warm, repeats, kreps, headline and not args.no_cpu_baseline), steps, repeats
         assert spec is not None
-        wl, res = run_linear(name, dev, steps, warm, repeats, kreps, on_gpu_data=not headline, graph=args.graph and headline)
+        wl, res = run_linear(name, dev, steps, warm, repeats, kreps, on_gpu_data=not headline, graph=args.graph and headline, fp6=fp6)
         return wl, res, steps, repeats
 
     wl, res, steps, repeats = measure(args.workload, True)
     roof = dict(res["roofline"])
-    traffic, source = traffic_from_profile(args.workload, roof["kernel"])
+    traffic, source = traffic_from_profile(args.workload + ("_fp6" if args.fp6 else ""), roof["kernel"])
     if traffic is not None and args.workload == "c3":
         traffic *= 4                                       # the step is four launches; the summary holds their average
     roof["traffic"] = traffic
@@ -599,7 +627,9 @@ def main():
         "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": steps, "warmup": args.warmup, "repeats": repeats,
         "ms_per_step": res["ms"], "ms_per_step_mean": res["timing"]["mean_ms"], "ms_per_step_ci95": res["timing"]["ci95_ms"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 -> u4 (fp32 Hadamard, fp16 quantiser)" if kv_line else "int4 x int4 -> int32 (int8 MFMA), fp16 scales",
+        "dtype": ("f16 -> u4 (fp32 Hadamard, fp16 quantiser)" if kv_line
+                  else "int4 x int4 -> exact integers in fp32 (FP6 MFMA), fp16 scales" if args.fp6
+                  else "int4 x int4 -> int32 (int8 MFMA), fp16 scales"),
         "data": "synthetic",
         "config": {"workload": res["workload"], "launch": res.get("launch", "eager"),
                    "timing": "median of `repeats` loops of `steps` steps, each loop between two synchronisations; kernel times from a "
