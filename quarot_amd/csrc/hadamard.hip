@@ -1462,6 +1462,41 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
     const int l16 = lane & 15, g = lane >> 4;
     const int nchunks = n >> 3;
 
+    // m = 1024: unit (wave / 2) = four k, wave % 2 = the half of c'; Sylvester fragments of both stages
+    constexpr int XL = CPL == 2 ? 8 : SPW * CPL;
+    const int unit = wave >> 1, cth = wave & 1;
+    const bool works = CPL == 2 && unit * 4 < K;
+    u32x4 raw[XL];
+    auto request = [&](int64_t row) {
+        if (CPL == 2) {
+#pragma unroll
+            for (int ai = 0; ai < 4; ++ai)          // (waves beyond the last unit repeat unit 0's loads and drop them: no branch)
+#pragma unroll
+                for (int bt = 0; bt < 2; ++bt)
+                    raw[ai * 2 + bt] = *((const u32x4*)(x + row * (int64_t)n) + ((works ? unit : 0) * 4 + ai) * 128 + bt * 64 + l16 * 4 + g);
+            return;
+        }
+#pragma unroll
+        for (int sg = 0; sg < SPW; ++sg) {
+            const int k = wave + NW * sg;
+#pragma unroll
+            for (int i = 0; i < CPL; ++i)
+                raw[sg * CPL + i] = k < K ? *((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
+                                          : u32x4{0, 0, 0, 0};
+        }
+    };
+    int64_t row = blockIdx.x;
+    if (row < rows) request(row);           // in flight while the fragments are made and T is cleared
+    f16x8 ha, hb[2];
+    if (CPL == 2) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            ha[t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+            const int b = 16 * (t >> 2) + 4 * g + (t & 3);
+#pragma unroll
+            for (int bt = 0; bt < 2; ++bt) hb[bt][t] = (__builtin_popcount(b & (bt * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+        }
+    }
     // hadK fragments (second MFMA operand): column k' = rt*16 + l16, contraction k = ks*32 + g*8 + j
     f16x8 hf[RT][KS2];
 #pragma unroll
@@ -1479,42 +1514,6 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
     // slots of T for k >= K are never written afterwards: clear once
     for (int i = tid; i < KS2 * 4 * CT * TS; i += BT) Tl[i] = u32x4{0, 0, 0, 0};
 
-    // m = 1024: unit (wave / 2) = four k, wave % 2 = the half of c'; Sylvester fragments of both stages
-    constexpr int XL = CPL == 2 ? 8 : SPW * CPL;
-    const int unit = wave >> 1, cth = wave & 1;
-    const bool works = CPL == 2 && unit * 4 < K;
-    f16x8 ha, hb[2];
-    if (CPL == 2) {
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            ha[t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
-            const int b = 16 * (t >> 2) + 4 * g + (t & 3);
-#pragma unroll
-            for (int bt = 0; bt < 2; ++bt) hb[bt][t] = (__builtin_popcount(b & (bt * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
-        }
-    }
-    u32x4 raw[XL];
-    auto request = [&](int64_t row) {
-        if (CPL == 2) {
-#pragma unroll
-            for (int ai = 0; ai < 4; ++ai)
-#pragma unroll
-                for (int bt = 0; bt < 2; ++bt)
-                    raw[ai * 2 + bt] = works ? *((const u32x4*)(x + row * (int64_t)n) + (unit * 4 + ai) * 128 + bt * 64 + l16 * 4 + g)
-                                             : u32x4{0, 0, 0, 0};
-            return;
-        }
-#pragma unroll
-        for (int sg = 0; sg < SPW; ++sg) {
-            const int k = wave + NW * sg;
-#pragma unroll
-            for (int i = 0; i < CPL; ++i)
-                raw[sg * CPL + i] = k < K ? *((const u32x4*)(x + row * (int64_t)n) + k * (M_ / 8) + i * 64 + lane)
-                                          : u32x4{0, 0, 0, 0};
-        }
-    };
-    int64_t row = blockIdx.x;
-    if (row < rows) request(row);
     __syncthreads();
     for (; row < rows; row += gridDim.x) {
         // ---- phase 1: the power-of-two factor of every segment, results in fragment order in LDS
@@ -1523,18 +1522,22 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                 u32 o[4][2][2];                          // [k of the unit][b' tile][pair of e]: fp16 pairs
 #pragma unroll
                 for (int ai = 0; ai < 4; ++ai) {
-                    f16x8 thi, tlo;
+                    // T = hi + lo, both fp16, as packed pairs (the difference is exact in fp32, so one rounding each)
+                    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                    u32x4 whi, wlo;
 #pragma unroll
                     for (int bt = 0; bt < 2; ++bt) {
                         const f32x4 da = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, raw[ai * 2 + bt]), ha,
                                                                               f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const f16 hi = narrow_f16(da[e]);
-                            thi[bt * 4 + e] = hi;
-                            tlo[bt * 4 + e] = narrow_f16(da[e] - (float)hi);
+                        for (int pr = 0; pr < 2; ++pr) {
+                            const f16x2 hi = __builtin_convertvector(f32x2_t{da[2 * pr], da[2 * pr + 1]}, f16x2);
+                            const f16x2 lo = __builtin_convertvector(f32x2_t{da[2 * pr] - (float)hi[0], da[2 * pr + 1] - (float)hi[1]}, f16x2);
+                            whi[bt * 2 + pr] = __builtin_bit_cast(u32, hi);
+                            wlo[bt * 2 + pr] = __builtin_bit_cast(u32, lo);
                         }
                     }
+                    const f16x8 thi = __builtin_bit_cast(f16x8, whi), tlo = __builtin_bit_cast(f16x8, wlo);
 #pragma unroll
                     for (int bt = 0; bt < 2; ++bt) {
                         f32x4 db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], thi, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
@@ -1591,7 +1594,9 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
         const int64_t nrow = row + gridDim.x;
         if (nrow < rows) request(nrow);
         __syncthreads();
-        // ---- stage 2: Y^T = T^T . hadK^T
+        // ---- stage 2: Y^T = T^T . hadK^T (the row's largest magnitude is taken on the way: packed unsigned maxima
+        // of the fp16 bit patterns without their signs, so that a NaN still wins)
+        u16x2 mx2 = {0, 0};
         for (int ct = wave * (CT / NW); ct < (wave + 1) * (CT / NW); ++ct) {
             f16x8 th[KS2];
 #pragma unroll
@@ -1609,22 +1614,23 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
                         o[0] = narrow_f16x2(acc[0], acc[1]);
                         o[1] = narrow_f16x2(acc[2], acc[3]);
                         *(u32x2*)(Yl + kp * YS + ct * 16 + g * 4) = o;
+                        if (QUANT) {
+                            mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[0] & 0x7fff7fffu));
+                            mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, o[1] & 0x7fff7fffu));
+                        }
                     }
                 }
             }
         }
+        u32 mx = 0;
+        if (QUANT) {
+            mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+            mx = wave_max_u32(mx);
+            if (lane == 0) red[wave] = mx;          // (last read before the barrier that follows the previous row's phase 1)
+        }
         __syncthreads();
         // ---- stage 3
         if (QUANT) {
-            u32 mx = 0;
-            for (int c = tid; c < nchunks; c += BT) {
-                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
-                const u32 mc = absmax_bits8(h);
-                mx = mx > mc ? mx : mc;
-            }
-            mx = wave_max_u32(mx);
-            if (lane == 0) red[wave] = mx;
-            __syncthreads();
 #pragma unroll
             for (int w = 0; w < NW; ++w) mx = mx > red[w] ? mx : red[w];
             const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
