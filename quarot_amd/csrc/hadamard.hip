@@ -1054,11 +1054,13 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 //     v_permlane16_swap, byte permutes: a 4 x 4 transpose of pieces across the lanes l16 + 16 g) so
 //     that every lane stores 8 contiguous bytes and a wave 32 contiguous bytes per output row.
 // Only T (stage 1's output, read by every wave in stage 2) lives in LDS: 4 KB per 32 hadK columns.
-template <int KS2>
+template <int KS2, int LOG2M = 6, bool SMALLK = false>
 __global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
                                                              const f16* __restrict__ hadK, float scale, float clip,
                                                              u32* __restrict__ q, f16* __restrict__ scales) {
-    constexpr int CT = 4;
+    constexpr int M_ = 1 << LOG2M;                           // the power-of-two factor: 64, or 128 (hadK of 64 .. 128)
+    constexpr int CT = M_ / 16;                              // column tiles
+    constexpr int S1K = M_ / 32;                             // k steps of stage 1
     constexpr int NT = 2 * KS2;
     constexpr int TPW = (NT + 3) / 4;
     extern __shared__ f32x4 smem_raw[];
@@ -1096,22 +1098,22 @@ __global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restr
             sb[o][0][j] = neg ? (f16)-1.0f : (f16)1.0f;
             sb[o][1][j] = neg ? (f16)1.0f : (f16)-1.0f;
         }
-    // fragment (tile i, k step c) of a row: 16-byte piece 4 c + g of row (wave + 4 i) 16 + l16 of X[K][64]
-    int goff[TPW][2];
+    // fragment (tile i, k step c) of a row: 16-byte piece 4 c + g of row (wave + 4 i) 16 + l16 of X[K][M_]
+    int goff[TPW][S1K];
     bool dval[TPW];
 #pragma unroll
     for (int i = 0; i < TPW; ++i) {
         const int r = (wave + 4 * i) * 16 + l16;
         dval[i] = r < K;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) goff[i][c] = dval[i] ? r * 8 + 4 * c + g : 0;
+        for (int c = 0; c < S1K; ++c) goff[i][c] = dval[i] ? r * (M_ / 8) + 4 * c + g : 0;
     }
-    u32x4 xr[TPW][2];
+    u32x4 xr[TPW][S1K];
     auto load_row = [&](const f16* src) {
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) xr[i][c] = *((const u32x4*)src + goff[i][c]);
+            for (int c = 0; c < S1K; ++c) xr[i][c] = *((const u32x4*)src + goff[i][c]);
     };
     u32 amask[TPW];                                          // magnitude bits of this lane's output row in tile i, 0 beyond K:
 #pragma unroll                                               // those rows are zero except when the row holds an infinity (0 . inf)
@@ -1172,54 +1174,69 @@ __global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restr
         quant_part(p, 2);
     };
     auto finish_prev = [&](bool fast) {                      // pack, exchange pieces between lanes, store
-        u32 c01[TPW], c23[TPW];
+        constexpr int HV = CT / 4;                           // groups of four column tiles (64 columns) per row
+        u32 c01[TPW][HV], c23[TPW][HV];
         if (fast) {
 #pragma unroll
-            for (int i = 0; i < TPW; ++i) {
-                const u32 b0[4] = {pb[i][0][0], pb[i][0][1], pb[i][1][0], pb[i][1][1]};
-                const u32 b1[4] = {pb[i][2][0], pb[i][2][1], pb[i][3][0], pb[i][3][1]};
-                c01[i] = pack_nibbles8(b0);
-                c23[i] = pack_nibbles8(b1);
-            }
+            for (int i = 0; i < TPW; ++i)
+#pragma unroll
+                for (int hv = 0; hv < HV; ++hv) {
+                    const u32 b0[4] = {pb[i][4 * hv][0], pb[i][4 * hv][1], pb[i][4 * hv + 1][0], pb[i][4 * hv + 1][1]};
+                    const u32 b1[4] = {pb[i][4 * hv + 2][0], pb[i][4 * hv + 2][1], pb[i][4 * hv + 3][0], pb[i][4 * hv + 3][1]};
+                    c01[i][hv] = pack_nibbles8(b0);
+                    c23[i][hv] = pack_nibbles8(b1);
+                }
         } else {
             const bool fs = scale_fast_ok(sp);
             const float rs = fs ? 1.0f / sp : 0.0f;
 #pragma unroll
-            for (int i = 0; i < TPW; ++i) {
-                c01[i] = sym_codes8(u32x4{yp[i][0][0], yp[i][0][1], yp[i][1][0], yp[i][1][1]}, sp, rs, fs);
-                c23[i] = sym_codes8(u32x4{yp[i][2][0], yp[i][2][1], yp[i][3][0], yp[i][3][1]}, sp, rs, fs);
-            }
+            for (int i = 0; i < TPW; ++i)
+#pragma unroll
+                for (int hv = 0; hv < HV; ++hv) {
+                    c01[i][hv] = sym_codes8(u32x4{yp[i][4 * hv][0], yp[i][4 * hv][1], yp[i][4 * hv + 1][0], yp[i][4 * hv + 1][1]}, sp, rs, fs);
+                    c23[i][hv] = sym_codes8(u32x4{yp[i][4 * hv + 2][0], yp[i][4 * hv + 2][1], yp[i][4 * hv + 3][0], yp[i][4 * hv + 3][1]}, sp, rs, fs);
+                }
         }
         u32x2* qrow = (u32x2*)(q + prow * (int64_t)nchunks);
-        u32x2 outv[TPW];
+        u32x2 outv[TPW][HV];
 #pragma unroll
-        for (int i = 0; i < TPW; ++i) {
-            // lanes l16 + 16 g: piece (g, ct) -> lane ct.  First the halves of the wave (g and g ^ 2) ...
-            const auto s1 = __builtin_amdgcn_permlane32_swap(c01[i], c23[i], false, false);
-            const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);     // the even column tile of this lane's pair
-            const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);     // the odd one
-            // ... then neighbouring rows of 16 lanes (g and g ^ 1)
-            const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
-            const u32 lo = __builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u);     // pieces of g = 0, 1
-            const u32 hi = __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u);     // pieces of g = 2, 3
-            outv[i] = u32x2{lo, hi};
-        }
-        // lanes on rows beyond K store their first tile's piece once more (K >= 64: that row exists)
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) {
+                // lanes l16 + 16 g: piece (g, ct) -> lane ct % 4.  First the halves of the wave (g and g ^ 2) ...
+                const auto s1 = __builtin_amdgcn_permlane32_swap(c01[i][hv], c23[i][hv], false, false);
+                const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);     // the even column tile of this lane's pair
+                const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);     // the odd one
+                // ... then neighbouring rows of 16 lanes (g and g ^ 1)
+                const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
+                const u32 lo = __builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u);     // pieces of g = 0, 1
+                const u32 hi = __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u);     // pieces of g = 2, 3
+                outv[i][hv] = u32x2{lo, hi};
+            }
+        // lanes on rows beyond K store their first tile's piece once more (K >= 64: that row exists; SMALLK: hadK
+        // is smaller than that, a wave's first tile may lie outside it, and the stores are conditional)
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
             const int kp = (wave + 4 * i) * 16 + l16;
             const bool ok = kp < K;
-            qrow[(ok ? kp : wave * 16 + l16) * 4 + g] = ok ? outv[i] : outv[0];
+#pragma unroll
+            for (int hv = 0; hv < HV; ++hv) {
+                if (SMALLK) {
+                    if (ok) qrow[kp * CT + hv * 4 + g] = outv[i][hv];
+                } else {
+                    qrow[(ok ? kp : wave * 16 + l16) * CT + hv * 4 + g] = ok ? outv[i][hv] : outv[0][hv];
+                }
+            }
         }
     };
     for (; row < rows; row += gridDim.x) {
         const int64_t nrow = row + gridDim.x;
         // ---- stage 1: T = X . H_64 for this wave's tiles (rows beyond K are zero fragments)
-        u32x4 af[TPW][2];
+        u32x4 af[TPW][S1K];
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) af[i][c] = dval[i] ? xr[i][c] : u32x4{0, 0, 0, 0};
+            for (int c = 0; c < S1K; ++c) af[i][c] = dval[i] ? xr[i][c] : u32x4{0, 0, 0, 0};
         // (unconditional, like every store below: with a fixed number of memory operations per turn the wait
         // for these loads, a turn later, need not include the stores issued after them; the last turn re-reads
         // its own row)
@@ -1231,8 +1248,12 @@ __global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restr
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][0]), sb[ct & 1][0], acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][1]), sb[ct & 1][ct >> 1], acc, 0, 0, 0);
+                    // H[k][col] = (-1)^popcount(k & col): the fragment of (k step c, column tile ct) is the base tile of
+                    // ct & 1, negated when c and ct / 2 share an odd number of bits
+#pragma unroll
+                    for (int c = 0; c < S1K; ++c)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[i][c]),
+                                                                   sb[ct & 1][__builtin_popcount(c & (ct >> 1)) & 1], acc, 0, 0, 0);
                     u32x2 hi;
                     hi[0] = narrow_f16x2(acc[0] * scale, acc[1] * scale);
                     hi[1] = narrow_f16x2(acc[2] * scale, acc[3] * scale);
@@ -1335,6 +1356,24 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
                        void* q, void* scales, hipStream_t st, int ident = 0) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
+    if (m == 128 && (KS2 == 2 || KS2 == 4) && !ident && !MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
+        // m = 128 behind one of the reference's tables of order 36 .. 60 or 108 (Llama-2-13B: 5120 = 40 x 128, 13824 =
+        // 108 x 128): the lean fused kernel with eight column tiles.  (Orders 140 .. 172 would need more registers than a
+        // wave has -- 231 .. 260 spilled -- and stay with hadamard_mm_kernel.)
+        const size_t ldsq = (size_t)8192 * KS2;
+#define QR_M128Q(KS, SMALL)                                                                                            \
+    do {                                                                                                               \
+        auto kern = hadamard_m64q_kernel<KS, 7, SMALL>;                                                                \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                  \
+        const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
+        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \
+                                                 (f16*)scales);                                                        \
+    } while (0)
+        if (KS2 == 2) QR_M128Q(2, true);
+        else QR_M128Q(4, false);
+#undef QR_M128Q
+        return qr_launch_status();
+    }
     if (m == 64 && K >= 64 && !ident) {
         // the latency-organised kernel (it relies on every wave's first tile lying inside hadK), while
         // two workgroups still fit on a CU
