@@ -1055,7 +1055,7 @@ __global__ __launch_bounds__(HT, (KS2 <= 2 ? 4 : 2)) void hadamard_m64_kernel(
 //     that every lane stores 8 contiguous bytes and a wave 32 contiguous bytes per output row.
 // Only T (stage 1's output, read by every wave in stage 2) lives in LDS: 4 KB per 32 hadK columns.
 template <int KS2, int LOG2M = 6, bool SMALLK = false>
-__global__ __launch_bounds__(HT, 2) void hadamard_m64q_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
+__global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard_m64q_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
                                                              const f16* __restrict__ hadK, float scale, float clip,
                                                              u32* __restrict__ q, f16* __restrict__ scales) {
     constexpr int M_ = 1 << LOG2M;                           // the power-of-two factor: 64, or 128 (hadK of 64 .. 128)
@@ -1356,10 +1356,10 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
                        void* q, void* scales, hipStream_t st, int ident = 0) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
-    if (m == 128 && (KS2 == 2 || KS2 == 4) && !ident && !MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
-        // m = 128 behind one of the reference's tables of order 36 .. 60 or 108 (Llama-2-13B: 5120 = 40 x 128, 13824 =
-        // 108 x 128): the lean fused kernel with eight column tiles.  (Orders 140 .. 172 would need more registers than a
-        // wave has -- 231 .. 260 spilled -- and stay with hadamard_mm_kernel.)
+    if (m == 128 && KS2 >= 2 && KS2 != 3 && !ident && !MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
+        // m = 128 behind one of the reference's tables of order 36 and more (Llama-2-13B: 5120 = 40 x 128, 13824 =
+        // 108 x 128): the lean fused kernel with eight column tiles.  Orders 140 .. 172 need more registers than two
+        // workgroups per CU leave a wave (231 .. 260 spilled) and run one workgroup per CU.
         const size_t ldsq = (size_t)8192 * KS2;
 #define QR_M128Q(KS, SMALL)                                                                                            \
     do {                                                                                                               \
@@ -1369,8 +1369,12 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \
                                                  (f16*)scales);                                                        \
     } while (0)
-        if (KS2 == 2) QR_M128Q(2, true);
-        else QR_M128Q(4, false);
+        switch (KS2) {
+            case 2: QR_M128Q(2, true); break;
+            case 4: QR_M128Q(4, false); break;
+            case 5: QR_M128Q(5, false); break;
+            default: QR_M128Q(6, false); break;
+        }
 #undef QR_M128Q
         return qr_launch_status();
     }

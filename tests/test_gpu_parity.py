@@ -465,7 +465,7 @@ def test_hadamard_short_rows_many_per_workgroup(n):
         assert bool((err <= 2e-3 * x.float().abs().amax(dim=1) + 1e-3).all())
 
 
-@pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 16384, 224, 3840, 6912, 8960, 11008, 28672, 13824, 5120, 6656, 4608, 7680, 17920])
+@pytest.mark.parametrize("n", [64, 1024, 4096, 8192, 16384, 224, 3840, 6912, 8960, 11008, 28672, 13824, 5120, 6656, 4608, 7680, 17920, 22016])
 @pytest.mark.parametrize("fp32", [False, True])
 def test_fused_hadamard_quantize_equals_staged(n, fp32):
     """Codes of the fused kernel are judged on the kernel's OWN fp16 Hadamard output (returned on
@@ -491,7 +491,7 @@ def test_fused_hadamard_quantize_equals_staged(n, fp32):
     assert close(y2.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
 
 
-@pytest.mark.parametrize("n", [11008, 8960, 6912, 13824, 5120, 4608])
+@pytest.mark.parametrize("n", [11008, 8960, 6912, 13824, 5120, 4608, 17920])
 def test_fused_hadamard_quantize_lean_kernel_rows_of_every_kind(n):
     """Without the copy of the transformed rows the m = 64 widths (and m = 128 behind a table of order 36 .. 60 or
     108: the 13B widths 13824 and 5120; 4608 = 36 x 128 has hadK rows in only part of a wave's tile) take a kernel of their own (results of
