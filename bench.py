@@ -76,7 +76,7 @@ for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
 PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
-              "c2_fp6", "c3d_fp6"]
+              "c2_fp6", "c3_fp6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 FP6_MFMA_PEAK_TOPS = 10100.0     # MI355X dense fp6, published (the opt-in exact int4 GEMM on 6-bit operands)
 HBM_PEAK_GBS = 8000.0
@@ -96,6 +96,7 @@ PROFILE_OF = {
     "b13v": "gemm_sp256_b13v_2048x5120x5120.txt", "b70v": "gemm_sp256_b70v_2048x8192x8192.txt",
     "b13d": "gemm_sp256_b13d_2048x13824x5120.txt", "b70d": "gemm_sp256_b70d_2048x28672x8192.txt",
     "c2_fp6": "gemm_f6_c2_down_proj_7b.txt", "c3d_fp6": "gemm_f6_c3d_down_proj_32768_tokens.txt",
+    "c3_fp6": "gemm_f6_c3_prefill_layer_set_32768_tokens.txt",
 }
 
 
@@ -355,9 +356,10 @@ def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, grap
     return wl, res
 
 
-def run_layer(dev, steps, warmup, repeats, kernel_reps):
+def run_layer(dev, steps, warmup, repeats, kernel_reps, fp6=False):
     """Workload c3: the four W4A4 linears of a Llama-2-7B decoder layer at M = 32768 tokens (prefill,
-    16 x 2048) as one step; operands generated on the GPU, resident in HBM."""
+    16 x 2048) as one step; operands generated on the GPU, resident in HBM.  fp6: the GEMMs on the opt-in
+    FP6 matrix path (each step then also converts the activations' codes to 6-bit operands)."""
     import quarot_amd
     m = 32768
     parts = [("qkv", 4096, 12288, "quant", 10), ("o", 4096, 4096, "quant", 11), ("gate_up", 4096, 22016, "quant", 12),
@@ -369,6 +371,8 @@ def run_layer(dev, steps, warmup, repeats, kernel_reps):
         lin = quarot_amd.nn.Linear4bit(k, n).half().to(dev)
         lin.weight.copy_(w)
         lin.weight_scales.copy_(sw)
+        if fp6:
+            lin.prefill_fp6, lin.fp6_min_rows = True, 0
         front = (quarot_amd.nn.OnlineHadamardQuantizer(k) if kind == "had" else quarot_amd.nn.Quantizer()).to(dev)
         mods.append((xs[k], front, lin))
     ops = sum(2.0 * m * k * n for _, k, n, _, _ in parts)
@@ -376,30 +380,41 @@ def run_layer(dev, steps, warmup, repeats, kernel_reps):
     def step():
         for x, front, lin in mods:
             p = front(x)
-            y = quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None)
+            y = lin(p) if fp6 else quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None)
             del y                                           # 0.3 - 1.4 GB each: returned to the pool before the next one
 
     sp = spread(timed_loops(step, steps, warmup, repeats))
     ms = sp["median_ms"]
     per, gemm_total, front_total = {}, 0.0, 0.0
+    peak = FP6_MFMA_PEAK_TOPS if fp6 else INT8_MFMA_PEAK_TOPS
     for (name, k, n, kind, _), (x, front, lin) in zip(parts, mods):
         p = front(x)
         f_ms = kernel_ms(lambda: front(x), kernel_reps)
-        g_ms = kernel_ms(lambda: quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None), kernel_reps)
+        if fp6:
+            p6 = quarot_amd.convert_i4_f6(p.quantized_x)
+            c_ms = kernel_ms(lambda: quarot_amd.convert_i4_f6(p.quantized_x), kernel_reps)
+            g_ms = kernel_ms(lambda: quarot_amd.linear_f6(p6, p.scales_x, lin._weight_f6(), lin.weight_scales, None), kernel_reps)
+            del p6
+            front_total += c_ms
+        else:
+            g_ms = kernel_ms(lambda: quarot_amd.linear_i4(p.quantized_x, p.scales_x, lin.weight, lin.weight_scales, None), kernel_reps)
         del p
         gemm_total += g_ms
         front_total += f_ms
         per[name] = {"gemm_ms": round(g_ms, 4), "gemm_TOPS": round(2.0 * m * k * n / (g_ms * 1e-3) / 1e12, 1),
-                     "gemm_frac": round(2.0 * m * k * n / (g_ms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS, 4),
+                     "gemm_frac": round(2.0 * m * k * n / (g_ms * 1e-3) / 1e12 / peak, 4),
                      "front_ms": round(f_ms, 4), "front_GBs": round((2.5 * m * k + 2 * m) / (f_ms * 1e-3) / 1e9, 1)}
-    roof = {"bound": "mfma", "achieved": round(ops / (gemm_total * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s"}
+        if fp6:
+            per[name]["convert_ms"] = round(c_ms, 4)
+    roof = {"bound": "mfma", "achieved": round(ops / (gemm_total * 1e-3) / 1e12, 1), "peak": peak, "unit": "TOP/s"}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = "gemm_sp256_kernel (int4 GEMM + dequant epilogue), four launches"
+    roof["kernel"] = ("gemm_f6_kernel (exact int4 GEMM on FP6 operands + dequant epilogue), four launches" if fp6
+                      else "gemm_sp256_kernel (int4 GEMM + dequant epilogue), four launches")
     roof["kernel_ms"] = round(gemm_total, 4)
     return {"ms": ms, "value": round(ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": roof,
             "per_linear": per, "kernels_ms_sum": round(gemm_total + front_total, 4), "total_TOP": round(ops / 1e12, 2),
             "workload": "c3: Llama-2-7B decoder-layer linear set at M=32768 (qkv 4096->12288, o 4096->4096, gate_up 4096->22016, "
-                        "down 11008->4096 with online Hadamard), W4A4, one step = 8 launches"}
+                        "down 11008->4096 with online Hadamard), W4A4, one step = " + ("12 launches (fronts, conversions to 6-bit operands, GEMMs)" if fp6 else "8 launches")}
 
 
 def run_kv(dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
@@ -571,8 +586,8 @@ def main():
               "run one process per GPU and add the values (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
 
-    if args.fp6 and (WORKLOADS[args.workload] is None or WORKLOADS[args.workload][0] <= 64):
-        print("--fp6 applies to the prefill linear workloads (c1, c2, c3a-c3d, b13*, b70*)", file=sys.stderr)
+    if args.fp6 and args.workload != "c3" and (WORKLOADS[args.workload] is None or WORKLOADS[args.workload][0] <= 64):
+        print("--fp6 applies to the prefill linear workloads (c1, c2, c3, c3a-c3d, b13*, b70*)", file=sys.stderr)
         sys.exit(2)
     from quarot_amd import _lib
     if not _lib.LIB_PATH.exists():
@@ -603,7 +618,7 @@ def main():
         kreps = args.kernel_reps if not big else max(5, args.kernel_reps // 5)
         warm = args.warmup if not big else max(2, args.warmup // 5)
         if name == "c3":
-            return None, run_layer(dev, steps, warm, repeats, kreps), steps, repeats
+            return None, run_layer(dev, steps, warm, repeats, kreps, fp6=fp6), steps, repeats
         if name == "c5":
             return None, run_kv(dev, steps, warm, repeats, kreps, headline and not args.no_cpu_baseline), steps, repeats
         if name in ("c6", "c6b"):
@@ -654,7 +669,7 @@ def main():
             per[name] = brief(r)
             t, s = traffic_from_profile(name, r["roofline"]["kernel"])
             if t is not None:
-                per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = (4 * t if name == "c3" else t), s
+                per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = (4 * t if name in ("c3", "c3_fp6") else t), s
         out["per_config"] = per
         out["per_config_note"] = ("same step definition as the headline; operands generated on the GPU, a fifth of the steps per loop "
                                   "(c3, c5: fewer still) and half the repeats")

@@ -1,6 +1,7 @@
 import torch
 
 import quarot_amd
+from .hadamard import OnlineHadamard
 
 
 def _pack_weight(weight, weight_scales):
@@ -88,7 +89,6 @@ class Linear4bitSequential(torch.nn.Sequential):
     module like the base class."""
 
     def _plan(self):
-        from .hadamard import OnlineHadamard
         from .quantization import Quantizer
         mods = list(self)
         had = None
@@ -104,8 +104,30 @@ class Linear4bitSequential(torch.nn.Sequential):
                 or not x.is_contiguous() or x.shape[-1] % 64 != 0):
             return super().forward(x)
         had, quantizer, lin = plan
+        if lin.prefill_fp6 and x.numel() // x.shape[-1] >= lin.fp6_min_rows and lin.in_features % 64 == 0:
+            # long prompt on the opt-in FP6 matrix path: the fused front, then Linear4bit's own route
+            if had is None:
+                return lin(quantizer(x))
+            return lin(quarot_amd.hadamard_quantize(x, had.had_rem_dim, had.rem_dim, quantizer.input_clip_ratio,
+                                                    force_fp32=had.fp32_had))
         if had is None:
             return quarot_amd.quantized_linear(x, lin.weight, lin.weight_scales, lin.bias,
                                                clip_ratio=quantizer.input_clip_ratio)
         return quarot_amd.quantized_linear(x, lin.weight, lin.weight_scales, lin.bias, had.had_rem_dim, had.rem_dim,
                                            quantizer.input_clip_ratio, force_fp32=had.fp32_had)
+
+
+def enable_fp6_prefill(module, min_rows=4096, convert_now=True):
+    """Opt every Linear4bit under `module` into the FP6 matrix path for inputs of at least `min_rows`
+    rows (long prompts): the same results bit for bit, the GEMM 15-25 % faster at 32768 rows, for a
+    6-bit copy of each weight (1.5 x its packed size, kept beside the 4-bit one that decode streams)
+    and a conversion pass over the activations' codes.  convert_now: make the copies here rather
+    than at the first long input.  Returns the number of layers switched."""
+    count = 0
+    for m in module.modules():
+        if isinstance(m, Linear4bit) and m.in_features % 64 == 0:
+            m.prefill_fp6, m.fp6_min_rows = True, int(min_rows)
+            if convert_now and m.weight.is_cuda:
+                m._weight_f6()
+            count += 1
+    return count

@@ -277,6 +277,30 @@ def test_linear4bit_opt_in_fp6_prefill_equals_the_default_path():
     assert torch.equal(got, lin(x))
 
 
+def test_enable_fp6_prefill_on_a_module_tree_changes_no_result():
+    """enable_fp6_prefill switches every Linear4bit of a model; the reference-shaped chains (Linear4bitSequential with
+    and without the online Hadamard) then take the FP6 route for long inputs and the usual one for short ones,
+    with identical outputs."""
+    nn_ = quarot_amd.nn
+    rng = np.random.default_rng(11)
+    def lin(k, n):
+        m = nn_.Linear4bit(k, n).half().cuda()
+        m.weight.copy_(gpu(o.pack_i4(rng.integers(-8, 8, (n, k)))))
+        m.weight_scales.copy_(gpu((np.abs(rng.standard_normal((n, 1))) * 0.01 + 0.001).astype(F16)))
+        return m
+    model = torch.nn.ModuleDict({
+        "down": nn_.Linear4bitSequential(nn_.OnlineHadamard(2304), nn_.Quantizer(0.9), lin(2304, 320)),
+        "q": nn_.Linear4bitSequential(nn_.Quantizer(), lin(512, 384)),
+    }).cuda()
+    xs = {"down": gpu(synth_x(700, 2304, seed=3)), "q": gpu(synth_x(700, 512, seed=4))}
+    want = {k: model[k](xs[k]) for k in xs}
+    assert nn_.enable_fp6_prefill(model, min_rows=256) == 2
+    for k in xs:
+        assert model[k][-1]._f6_cache is not None                       # converted at once
+        assert torch.equal(model[k](xs[k]), want[k])                    # long input: FP6 route
+        assert torch.equal(model[k](xs[k][:100]), want[k][:100])        # short input: the usual route
+
+
 def test_matmul_known_answers_and_leading_dims():
     k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
     a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
