@@ -204,7 +204,8 @@ int qr_linear_i4_f16_static(const void* A, const void* sA, const void* W, const 
  *     Weights are converted once after loading, activations after the quantiser.
  *   qr_linear_f6_f16: A6 = converted codes of x [M, K], W6 = converted weight [N, K] (both 16-byte
  *     aligned, each below 4 GiB, else QR_E_UNSUPPORTED), sA fp16 [M], sW fp16 [N], bias fp16 [N] or NULL
- *     -> y fp16 [M, N] (8-byte aligned).  Any M, N; meant for M >= 1024 (256 x 256 tiles).
+ *     -> y fp16 [M, N] (8-byte aligned).  Any M, N; meant for long prompts (256 x 256 tiles, or 128 x 256 when
+ *     those fill the compute units in fewer rounds).
  */
 size_t qr_f6_bytes(int64_t rows, int64_t K);
 int qr_convert_i4_f6(const void* codes, int64_t rows, int64_t K, void* out, void* stream);
