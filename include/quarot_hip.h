@@ -313,6 +313,20 @@ int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, const void* 
                        int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/*
+ * qr_batch_decode_i4 with the query's Hadamard inside: what the reference's decode step does as two calls,
+ * matmul_had_cuda(q, torch.float16) (quarot/transformers/kv_cache.py:30-33,113: fast_hadamard_transform over
+ * the head dimension, scale 1 / sqrt(128), result in fp16) and then batch_decode_i4, in ONE launch -- every
+ * workgroup transforms its own query vector (128 values, fp32 butterflies, rounded to fp16 as that function's
+ * result is) before it walks the cache.  Same arguments and tolerance as qr_batch_decode_i4; q is the
+ * untransformed query.
+ */
+int qr_batch_decode_qhad_i4(void* o, const void* q, const void* kv_data, const void* kv_param,
+                            const void* kv_indptr, const void* kv_indices, const void* last_page_offset,
+                            int64_t num_pages, int num_layers, int layer_idx, int num_heads, int page_size,
+                            int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,8 @@ SIGNATURES = {
     "qr_batch_decode_workspace_bytes": (_c.c_size_t, (_i64, _int, _i64)),
     "qr_batch_decode_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int, _i64, _i64, _ptr,
                                   _c.c_size_t, _ptr)),
+    "qr_batch_decode_qhad_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int, _i64, _i64, _ptr,
+                                       _c.c_size_t, _ptr)),
 }
 
 QR_DTYPE_F16, QR_DTYPE_F32 = 0, 1

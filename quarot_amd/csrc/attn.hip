@@ -92,7 +92,8 @@ __device__ __forceinline__ float row_rotate(float v) {   // DPP row_ror within e
 // NW: waves per workgroup (4 or 16): a (sequence, head) gets NW * splits waves in all.
 template <bool ALIGNED, int NW>
 __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void paged_decode_i4_kernel(
-    const f16* __restrict__ q, PagedKV c, f16* __restrict__ o, float sm_scale_log2, int splits, float* __restrict__ part) {
+    const f16* __restrict__ q, PagedKV c, f16* __restrict__ o, float sm_scale_log2, int splits, float* __restrict__ part,
+    int q_had) {
     __shared__ float st[NW * 4 * 4 * 36];                  // [wave * 4 + row][quarter][m, d, -, -, acc[32]]
     __shared__ float st2[(NW / 2) * 128 * 3];              // second merge level: [part][dimension][m, d, o]
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -108,9 +109,48 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
     float ql = 0.f;                                        // sum of this lane's 32 values
     {
         const u32x4* qsrc = (const u32x4*)(q + (int64_t)bh * 128 + c4 * 32);
+        u32x4 qw[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qw[j] = qsrc[j];
+        if (q_had) {
+            // The query's Hadamard over the head dimension (matmul_had_cuda on q, kv_cache.py:30-33,113) here instead of
+            // in a launch of its own: 128-point transform in fp32 -- five butterfly levels over the lane's 32 values,
+            // two across the four lanes of a position group -- times 1 / sqrt(128), rounded to fp16 like that
+            // function's result.
+            float t[32];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const f16x2 pr = as_f16x2(qw[j][k]);
+                    t[8 * j + 2 * k] = (float)pr[0];
+                    t[8 * j + 2 * k + 1] = (float)pr[1];
+                }
+#pragma unroll
+            for (int hb = 1; hb < 32; hb <<= 1)
+#pragma unroll
+                for (int i = 0; i < 32; ++i)
+                    if ((i & hb) == 0) {
+                        const float a = t[i], b = t[i + hb];
+                        t[i] = a + b;
+                        t[i + hb] = a - b;
+                    }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                const float o1 = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, t[i]), 0xB1, 0xF, 0xF, true));
+                t[i] = (c4 & 1) ? o1 - t[i] : t[i] + o1;                // lanes ^ 1: index bit 5
+                const float o2 = __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, t[i]), 0x4E, 0xF, 0xF, true));
+                t[i] = (c4 & 2) ? o2 - t[i] : t[i] + o2;                // lanes ^ 2: index bit 6
+            }
+            const float hs = 0.08838834764831845f;                       // 1 / sqrt(128)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) qw[j][k] = narrow_f16x2(t[8 * j + 2 * k] * hs, t[8 * j + 2 * k + 1] * hs);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const u32x4 w = qsrc[j];
+            const u32x4 w = qw[j];
             f16 e[8];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -446,10 +486,11 @@ extern "C" size_t qr_batch_decode_workspace_bytes(int64_t batch_size, int num_he
     return s > 1 ? (size_t)batch_size * num_heads * s * 132 * sizeof(float) : 0;
 }
 
-extern "C" int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, const void* kv_param, const void* kv_indptr,
-                                  const void* kv_indices, const void* last_page_offset, int64_t num_pages, int num_layers,
-                                  int layer_idx, int num_heads, int page_size, int head_dim, int64_t batch_size,
-                                  int64_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream) {
+namespace {
+int batch_decode(void* o, const void* q, const void* kv_data, const void* kv_param, const void* kv_indptr,
+                 const void* kv_indices, const void* last_page_offset, int64_t num_pages, int num_layers, int layer_idx,
+                 int num_heads, int page_size, int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
+                 size_t workspace_bytes, void* stream, int q_had) {
     const int rc = check_cache(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
                                num_heads, page_size, head_dim, batch_size);
     if (rc != QR_OK) return rc;
@@ -469,7 +510,7 @@ extern "C" int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, c
     hipStream_t st = (hipStream_t)stream;
 #define QR_DECODE(AL, NWV)                                                                                              \
     paged_decode_i4_kernel<AL, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits,      \
-                                                                          (float*)workspace)
+                                                                          (float*)workspace, q_had)
     if (page_size % 16 == 0) {
         if (plan.nw == 16) QR_DECODE(true, 16);
         else if (plan.nw == 8) QR_DECODE(true, 8);
@@ -485,4 +526,21 @@ extern "C" int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, c
     paged_decode_merge_kernel<<<dim3((unsigned)(batch_size * num_heads)), dim3(128), 0, st>>>((const float*)workspace, splits,
                                                                                              (f16*)o);
     return qr_launch_status();
+}
+}  // namespace
+
+extern "C" int qr_batch_decode_i4(void* o, const void* q, const void* kv_data, const void* kv_param, const void* kv_indptr,
+                                  const void* kv_indices, const void* last_page_offset, int64_t num_pages, int num_layers,
+                                  int layer_idx, int num_heads, int page_size, int head_dim, int64_t batch_size,
+                                  int64_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream) {
+    return batch_decode(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
+                        num_heads, page_size, head_dim, batch_size, max_seq_len, workspace, workspace_bytes, stream, 0);
+}
+
+extern "C" int qr_batch_decode_qhad_i4(void* o, const void* q, const void* kv_data, const void* kv_param, const void* kv_indptr,
+                                       const void* kv_indices, const void* last_page_offset, int64_t num_pages, int num_layers,
+                                       int layer_idx, int num_heads, int page_size, int head_dim, int64_t batch_size,
+                                       int64_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream) {
+    return batch_decode(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
+                        num_heads, page_size, head_dim, batch_size, max_seq_len, workspace, workspace_bytes, stream, 1);
 }

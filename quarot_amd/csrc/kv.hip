@@ -279,7 +279,8 @@ template <bool QUANT, bool PAGED = false>
 __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4* __restrict__ x, int64_t vectors,
                                                                      float hscale, u32x4* __restrict__ q,
                                                                      f16* __restrict__ scale, f16* __restrict__ zero,
-                                                                     u32x4* __restrict__ y, PagedDst pd) {
+                                                                     u32x4* __restrict__ y, PagedDst pd,
+                                                                     const u32x4* __restrict__ x2, int plain_mask) {
     __shared__ u32x4 km_lds[KM_WAVES * 512];                       // 8 KB per wave
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int v = lane & 31, h = lane >> 5;
@@ -296,17 +297,30 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
             hn[o][e] = neg ? (f16)1.0f : (f16)-1.0f;
         }
 
-    const int64_t blocks = (vectors + 31) >> 5;
+    // Identity tiles (PAGED only): a part that is quantised WITHOUT the transform -- the values of an append, or
+    // keys when the caller wants none -- goes through the same matrix instructions with I in place of H_128
+    // (exact: one non-zero product per sum), so that keys and values of an append are ONE launch: blocks
+    // [0, blocks1) take x, blocks [blocks1, 2 blocks1) take x2 into the value slots.
+    f16x8 ib[2];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ib[o][e] = (PAGED && v == 16 * o + 8 * h + e) ? (f16)1.0f : (f16)0.0f;
+    const int64_t blocks1 = (vectors + 31) >> 5;
+    const int64_t blocks = (PAGED && x2) ? 2 * blocks1 : blocks1;
     const int64_t wstride = (int64_t)gridDim.x * KM_WAVES;
     int64_t blk = (int64_t)blockIdx.x * KM_WAVES + wave;
     // block of 32 rows = 512 pieces of 16 bytes; load c takes pieces 64 c + lane: row 4 c + lane / 16
     u32x4 pre[8];
     auto fetch = [&](int64_t b) {
+        const bool second = PAGED && b >= blocks1;
+        const u32x4* src = second ? x2 : x;
+        if (second) b -= blocks1;
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             int64_t row = b * 32 + 4 * c + (lane >> 4);
             row = row < vectors ? row : vectors - 1;               // the last block may be short: repeat its last row
-            pre[c] = x[row * 16 + (lane & 15)];
+            pre[c] = src[row * 16 + (lane & 15)];
         }
     };
     if (blk < blocks) fetch(blk);
@@ -318,17 +332,29 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
         u32x4 xf[8];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) xf[ks] = stage[km_slot(v, 2 * ks + h)];
+        const bool second = PAGED && blk >= blocks1;               // wave-uniform
+        const bool plain = PAGED && ((plain_mask >> (second ? 1 : 0)) & 1);
+        const float oscale = plain ? 1.0f : hscale;
         f32x16 acc[4];
 #pragma unroll
-        for (int jt = 0; jt < 4; ++jt) {
+        for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[jt][r] = 0.f;
+        if (plain) {
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                const bool neg = (__builtin_popcount(jt & (ks >> 1)) & 1) != 0;     // compile-time after unrolling
-                acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(neg ? hn[ks & 1] : hb[ks & 1],
-                                                                 __builtin_bit_cast(f16x8, xf[ks]), acc[jt], 0, 0, 0);
-            }
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int o = 0; o < 2; ++o)
+                    acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ib[o], __builtin_bit_cast(f16x8, xf[2 * jt + o]), acc[jt], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) {
+                    const bool neg = (__builtin_popcount(jt & (ks >> 1)) & 1) != 0;     // compile-time after unrolling
+                    acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(neg ? hn[ks & 1] : hb[ks & 1],
+                                                                     __builtin_bit_cast(f16x8, xf[ks]), acc[jt], 0, 0, 0);
+                }
         }
         // scaled, rounded outputs: yq[jt][qq] = the four outputs j = 32 jt + 8 qq + 4 h + (0..3), two per word
         u32 yw[4][4][2];
@@ -336,10 +362,11 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
         for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
             for (int qq = 0; qq < 4; ++qq) {
-                yw[jt][qq][0] = narrow_f16x2(acc[jt][4 * qq] * hscale, acc[jt][4 * qq + 1] * hscale);
-                yw[jt][qq][1] = narrow_f16x2(acc[jt][4 * qq + 2] * hscale, acc[jt][4 * qq + 3] * hscale);
+                yw[jt][qq][0] = narrow_f16x2(acc[jt][4 * qq] * oscale, acc[jt][4 * qq + 1] * oscale);
+                yw[jt][qq][1] = narrow_f16x2(acc[jt][4 * qq + 2] * oscale, acc[jt][4 * qq + 3] * oscale);
             }
-        const int64_t vec = blk * 32 + v;
+        const int64_t blk1 = second ? blk - blocks1 : blk;
+        const int64_t vec = blk1 * 32 + v;
         if (!QUANT) {
             // back through the staging region (all fragment reads are done): 8-byte pieces in, rows out
 #pragma unroll
@@ -464,7 +491,7 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                 int64_t page;
                 int entry;
                 if (paged_locate(pd.c, pd.append_indptr, token, page, entry)) {
-                    const int64_t s = paged_slot(pd.c, page, pd.kv, (int)(vec - token * pd.c.num_heads), entry);
+                    const int64_t s = paged_slot(pd.c, page, second ? 1 : pd.kv, (int)(vec - token * pd.c.num_heads), entry);
                     u32x4* dst = (u32x4*)pd.c.data + s * 4 + 2 * h;
                     dst[0] = u32x4{W[0], W[1], W[2], W[3]};
                     dst[1] = u32x4{W[4], W[5], W[6], W[7]};
@@ -484,14 +511,14 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
 
 template <bool QUANT, bool PAGED = false>
 int launch_had128(const void* x, int64_t vectors, float hscale, void* q, void* scale, void* zero, void* y, hipStream_t st,
-                  const PagedDst& pd = PagedDst{}) {
+                  const PagedDst& pd = PagedDst{}, const void* x2 = nullptr, int plain_mask = 0) {
     auto kern = kv_had128_kernel<QUANT, PAGED>;
-    const int64_t blocks = (vectors + 31) >> 5;
+    const int64_t blocks = ((vectors + 31) >> 5) * (x2 ? 2 : 1);
     const int64_t want = (blocks + KM_WAVES - 1) / KM_WAVES;
     const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, 64 * KM_WAVES, 0);
     const unsigned grid = (unsigned)(want < cap ? want : cap);
     kern<<<dim3(grid), dim3(64 * KM_WAVES), 0, st>>>((const u32x4*)x, vectors, hscale, (u32x4*)q, (f16*)scale, (f16*)zero,
-                                                    (u32x4*)y, pd);
+                                                    (u32x4*)y, pd, (const u32x4*)x2, plain_mask);
     return qr_launch_status();
 }
 
@@ -588,20 +615,11 @@ extern "C" int qr_kv_quant_append_f16_i4(const void* k, const void* v, int64_t t
     pd.c = qr_internal_paged_kv(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
                                 num_heads, page_size, batch_size);
     pd.append_indptr = (const int32_t*)append_indptr_or_null;
-    const int64_t vectors = tokens * num_heads, nchunks = vectors * 16;
+    const int64_t vectors = tokens * num_heads;
     const float hs = (float)(1.0 / __builtin_sqrt(128.0));
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(grid_for(nchunks, 4 * KT)), block(KT);
+    // keys (through H_128, or through the identity when the caller wants them untransformed) and values (identity) in
+    // ONE launch of the matrix-core kernel: bit for bit the codes, scales and zeros of the separate quantisers
     pd.kv = 0;
-    if (k_had_mode) {
-        const int rc = launch_had128<true, true>(k, vectors, hs, nullptr, nullptr, nullptr, nullptr, st, pd);
-        if (rc != QR_OK) return rc;
-    } else {
-        kv_quant_kernel<4, false, true><<<grid, block, 0, st>>>((const u32x4*)k, nchunks, hs, nullptr, nullptr, nullptr, pd);
-        const int rc = qr_launch_status();
-        if (rc != QR_OK) return rc;
-    }
-    pd.kv = 1;
-    kv_quant_kernel<4, false, true><<<grid, block, 0, st>>>((const u32x4*)v, nchunks, hs, nullptr, nullptr, nullptr, pd);
-    return qr_launch_status();
+    return launch_had128<true, true>(k, vectors, hs, nullptr, nullptr, nullptr, nullptr, st, pd, v, k_had_mode ? 2 : 3);
 }

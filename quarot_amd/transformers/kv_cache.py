@@ -168,11 +168,14 @@ def _decode_workspace_bytes(batch, heads, max_seq_len):
     return _lib.lib().qr_batch_decode_workspace_bytes(batch, heads, max_seq_len)
 
 
-def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, max_seq_len=0):
+def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, max_seq_len=0,
+                    q_hadamard=False):
     """o[b, h] = softmax(q[b, h] . K^T / sqrt(128)) . V over the int4 cache of sequence b, dequantised in
     registers as float(code) * scale - zero (kv_cache.py:60-67 -> bindings.cpp:118-153).  Writes into `o`
     and returns None, like the reference's binding.  max_seq_len (optional, an upper bound of the
-    sequence lengths) lets a small batch be split along the sequence."""
+    sequence lengths) lets a small batch be split along the sequence.  q_hadamard: `q` is the
+    untransformed query and the kernel applies matmul_had_cuda(q, torch.float16) itself (one launch
+    instead of two)."""
     fn = "batch_decode_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     for name, t in (("o", o), ("q", q)):
@@ -188,7 +191,8 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
     ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len)) if max_seq_len else 0
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
     with _lib.on_device(dev):
-        _lib.check(_lib.lib().qr_batch_decode_i4(
+        entry = _lib.lib().qr_batch_decode_qhad_i4 if q_hadamard else _lib.lib().qr_batch_decode_i4
+        _lib.check(entry(
             o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
             last_page_offset.data_ptr(), pages, layers, int(layer_idx), heads, page_size, head_dim, batch, int(max_seq_len),
             None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
@@ -208,10 +212,11 @@ class _AttentionStub(object):
         batch_size, q_len, num_qo_heads, head_dim = q.shape
         assert q_len == 1
         q = q.view(batch_size, num_qo_heads, head_dim)
-        if self.hadamard_dtype is not None:
+        fused = self.hadamard_dtype == torch.float16 and q.dtype == torch.float16 and q.is_contiguous()
+        if self.hadamard_dtype is not None and not fused:
             q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
         attn_output = torch.empty_like(q)
-        batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len)
+        batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len, q_hadamard=fused)
         return attn_output.unsqueeze(1)
 
 

@@ -132,6 +132,39 @@ def test_decode_attention_against_the_oracle(page_size, lens):
         assert close(out[b].cpu().numpy(), o.paged_dequant(vc, vp)[0])
 
 
+@pytest.mark.parametrize("page_size,lens", [(16, [1, 33, 700, 4100]), (5, [11, 64])])
+def test_decode_attention_with_the_querys_hadamard_inside(page_size, lens):
+    """q_hadamard=True: the kernel transforms the raw query itself.  Against the oracle on the oracle's own
+    transform of q (kv_hadamard: float64 sums, 1 / sqrt(128), fp16), and against the two-launch form
+    (matmul_had_cuda, then batch_decode_i4) -- with and without the split along the sequence, and through
+    the C entry point."""
+    rng = np.random.default_rng(page_size + 9)
+    heads, layer = 6, 0
+    data, param, indptr, indices, last = paged_case(rng, heads, page_size, lens, layers=1)
+    q = (rng.standard_normal((len(lens), heads, 128)) * 2).astype(F16)
+    q[0, 0, :] = 0
+    q[1, 2, 5] = 40.0
+    qh = o.kv_hadamard(q)
+    want = o.paged_batch_decode(qh, data, param, indptr, indices, last, layer)
+    args = (gpu(data), gpu(param), gpu(indptr), gpu(indices), gpu(last))
+    two = torch.empty((len(lens), heads, 128), dtype=torch.float16, device="cuda:0")
+    kv.batch_decode_i4(two, kv.matmul_had_cuda(gpu(q), torch.float16), *args, layer)
+    for hint in (0, max(lens)):
+        out = torch.full_like(two, float("nan"))
+        kv.batch_decode_i4(out, gpu(q), *args, layer, max_seq_len=hint, q_hadamard=True)
+        assert close(out.cpu().numpy(), want)
+        assert close(out.cpu().numpy(), two.cpu().numpy())
+    L = _lib.lib()
+    out = torch.full_like(two, float("nan"))
+    gq = gpu(q)
+    rc = L.qr_batch_decode_qhad_i4(out.data_ptr(), gq.data_ptr(), args[0].data_ptr(), args[1].data_ptr(), args[2].data_ptr(),
+                                   args[3].data_ptr(), args[4].data_ptr(), args[0].shape[0], 1, 0, heads, page_size, 128, len(lens), 0,
+                                   None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and close(out.cpu().numpy(), want)
+    assert L.qr_batch_decode_qhad_i4(None, gq.data_ptr(), args[0].data_ptr(), args[1].data_ptr(), args[2].data_ptr(), args[3].data_ptr(),
+                                     args[4].data_ptr(), args[0].shape[0], 1, 0, heads, page_size, 128, len(lens), 0, None, 0, None) == -1
+
+
 def test_decode_attention_real_quantised_cache_and_split_workspace():
     """A cache filled by the quantiser from N(0,1) keys and values with outliers (config 5's statistics),
     page size 16, 2 sequences x 8 heads x 1500 tokens: few workgroups, so the entry point splits the
