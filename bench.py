@@ -76,7 +76,7 @@ for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
 PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
-              "c2_fp6", "c3_fp6"]
+              "c2_fp6", "c3_fp6", "b13v_fp6", "b70v_fp6", "b13d_fp6", "b70d_fp6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 FP6_MFMA_PEAK_TOPS = 10100.0     # MI355X dense fp6, published (the opt-in exact int4 GEMM on 6-bit operands)
 HBM_PEAK_GBS = 8000.0

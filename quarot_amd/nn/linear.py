@@ -38,11 +38,12 @@ class Linear4bit(torch.nn.Module):
     def extra_repr(self):
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
 
-    # Opt-in: long prompts through the FP6 matrix path (quarot_amd.linear_f6: bit-identical results, 10-25 %
-    # faster GEMM at 32768 tokens, at the price of a 6-bit copy of the weights -- 1.5 x their packed size,
-    # made at the first such call -- and of one conversion pass over the activations' codes).
+    # Opt-in: prompts of fp6_min_rows rows and more through the FP6 matrix path (quarot_amd.linear_f6:
+    # bit-identical results, the GEMM 20-30 % faster wherever its tiles fill the machine, at the price of
+    # a 6-bit copy of the weights -- 1.5 x their packed size, made at the first such call -- and of one
+    # conversion pass over the activations' codes).
     prefill_fp6 = False
-    fp6_min_rows = 4096
+    fp6_min_rows = 2048
 
     def _weight_f6(self):
         key = (self.weight.data_ptr(), self.weight._version)
@@ -117,9 +118,10 @@ class Linear4bitSequential(torch.nn.Sequential):
                                            quantizer.input_clip_ratio, force_fp32=had.fp32_had)
 
 
-def enable_fp6_prefill(module, min_rows=4096, convert_now=True):
+def enable_fp6_prefill(module, min_rows=2048, convert_now=True):
     """Opt every Linear4bit under `module` into the FP6 matrix path for inputs of at least `min_rows`
-    rows (long prompts): the same results bit for bit, the GEMM 15-25 % faster at 32768 rows, for a
+    rows (prompts): the same results bit for bit, whole steps 14-22 % faster at 2048 rows of the 13B / 70B
+    widths and 16 % at 32768 rows of the 7B ones (level at 2048 rows of the 7B widths), for a
     6-bit copy of each weight (1.5 x its packed size, kept beside the 4-bit one that decode streams)
     and a conversion pass over the activations' codes.  convert_now: make the copies here rather
     than at the first long input.  Returns the number of layers switched."""
