@@ -4,7 +4,7 @@
 // last-level cache holds) and reads a shared 1 MB region (the tokens' codes, L2 hits) XS 16-byte loads for
 // every 4 private ones: 4:1, 4:4, 4:8 are the byte ratios of 8, 32 and 64 tokens.  The times are the floor
 // for any kernel with that decomposition of the work.
-//   hipcc --offload-arch=gfx950 -O3 -o decode_traffic decode_traffic.hip && ./decode_traffic
+//   hipcc --offload-arch=gfx950 -O3 -Xclang -target-feature -Xclang -packed-fp32-ops -o decode_traffic decode_traffic.hip && ./decode_traffic
 #include <hip/hip_runtime.h>
 #include <cstdio>
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));

@@ -2,7 +2,7 @@
 // quantiser and of its inverse with NOTHING else -- 16-byte loads of RD bytes in all, 16-byte stores of RD / 4 bytes
 // (or the other way round), eight buffers in turn so that no launch re-reads what the last-level cache holds.
 // The times are the floor for quant_rows_kernel / kv_quant_kernel (4 : 1) and kv_dequant_kernel (1 : 4).
-//   hipcc --offload-arch=gfx950 -O3 -o quantiser_traffic quantiser_traffic.hip && ./quantiser_traffic
+//   hipcc --offload-arch=gfx950 -O3 -Xclang -target-feature -Xclang -packed-fp32-ops -o quantiser_traffic quantiser_traffic.hip && ./quantiser_traffic
 #include <hip/hip_runtime.h>
 #include <cstdio>
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));

@@ -2,7 +2,7 @@
 // from HBM (a 2 GiB buffer, every launch reads all of it) and from L2 (a 2 MB window read over and over), as a
 // function of waves per CU and 16-byte loads in flight per lane.  The ceilings that the memory-bound kernels
 // are measured against come from here.
-//   hipcc --offload-arch=gfx950 -O3 -o read_bandwidth read_bandwidth.hip && ./read_bandwidth
+//   hipcc --offload-arch=gfx950 -O3 -Xclang -target-feature -Xclang -packed-fp32-ops -o read_bandwidth read_bandwidth.hip && ./read_bandwidth
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstdlib>
