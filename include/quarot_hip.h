@@ -283,7 +283,7 @@ int qr_kv_append_i4(void* kv_data, void* kv_param, const void* kv_indptr, const 
  * The same from fp16 K and V, quantising on the way: what MultiLayerPagedKVCache4Bit.update runs as
  * matmul_had_cuda(K), asym_quantize_and_pack_i4 (K and V), two torch.cat of {scale, zero} and
  * init_kv_i4 / append_kv_i4 (quarot/transformers/kv_cache.py:174-251).  Codes, scales and zeros are those
- * of qr_kv_quant_f16_i4 bit for bit; they go straight to their pages (two launches).
+ * of qr_kv_quant_f16_i4 bit for bit; they go straight to their pages (one launch for keys and values).
  *   k, v fp16 [tokens, num_heads, 128]; k_had_mode as qr_kv_quant_f16_i4's had_mode (1: Hadamard over the
  *   head dimension first); append_indptr_or_null as above.
  */

@@ -139,7 +139,7 @@ def quantize_append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_of
                           hadamard=True):
     """fp16 K and V [tokens, heads, 128] -> (Hadamard over the head dimension of K) -> asymmetric int4 ->
     straight into the pages: matmul_had_cuda + asym_quantize_and_pack_i4 (twice) + the two torch.cat +
-    init_kv_i4 / append_kv_i4 of MultiLayerPagedKVCache4Bit.update (kv_cache.py:174-251) as two launches,
+    init_kv_i4 / append_kv_i4 of MultiLayerPagedKVCache4Bit.update (kv_cache.py:174-251) as one launch,
     with the same codes, scales and zeros.  seqlen_indptr None: one token per sequence."""
     fn = "quantize_append_kv_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
