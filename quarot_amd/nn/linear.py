@@ -43,7 +43,7 @@ class Linear4bit(torch.nn.Module):
     # a 6-bit copy of the weights -- 1.5 x their packed size, made at the first such call -- and of one
     # conversion pass over the activations' codes).
     prefill_fp6 = False
-    fp6_min_rows = 2048
+    fp6_min_rows = 1024          # (measured: ahead of the int8 path from 1024 rows on at every Llama-2 width, conversion included)
 
     def _weight_f6(self):
         key = (self.weight.data_ptr(), self.weight._version)
@@ -118,7 +118,7 @@ class Linear4bitSequential(torch.nn.Sequential):
                                            quantizer.input_clip_ratio, force_fp32=had.fp32_had)
 
 
-def enable_fp6_prefill(module, min_rows=2048, convert_now=True):
+def enable_fp6_prefill(module, min_rows=1024, convert_now=True):
     """Opt every Linear4bit under `module` into the FP6 matrix path for inputs of at least `min_rows`
     rows (prompts): the same results bit for bit, whole steps 14-22 % faster at 2048 rows of the 13B / 70B
     widths and 16 % at 32768 rows of the 7B ones (level at 2048 rows of the 7B widths), for a
