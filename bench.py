@@ -532,12 +532,17 @@ def cpu_baseline(wl, budget_rows):
     row sample of the same workload, all host threads; TOPS scaled to the sample's own work."""
     from oracle import cpu_baseline as cb
     rows = min(wl.m, budget_rows)
-    xs = wl.x_cpu[:rows].clone()
     wc = cb.unpacked_codes(wl.w_cpu.numpy())
     ws = wl.sw_cpu.view(-1)
     hadamard, rmsnorm, heads = wl.front_kind == "had", wl.front_kind == "rmsnorm", wl.heads
     torch.set_num_threads(os.cpu_count() or 1)
-    cb.linear4bit_path(xs[:2], wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
+    cb.linear4bit_path(wl.x_cpu[:2].clone(), wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
+    # size the sample for about 4 s per pass (three passes: 10-15 s of CPU work), starting from `budget_rows`
+    t0 = time.perf_counter()
+    cb.linear4bit_path(wl.x_cpu[:rows].clone(), wc, ws, hadamard, rmsnorm, heads)
+    t_probe = time.perf_counter() - t0
+    rows = min(wl.m, max(rows, int(rows * 4.0 / max(t_probe, 1e-3)) // 64 * 64))
+    xs = wl.x_cpu[:rows].clone()
     times = []
     for _ in range(3):
         t0 = time.perf_counter()
@@ -576,7 +581,8 @@ def main():
     ap.add_argument("--fp6", action="store_true",
                     help="prefill linear workloads only: run the GEMM on the opt-in FP6 matrix path (Linear4bit.prefill_fp6); "
                          "the step then includes the conversion of the activations' codes to 6-bit operands")
-    ap.add_argument("--cpu-rows", type=int, default=64)
+    ap.add_argument("--cpu-rows", type=int, default=64,
+                    help="rows of the first CPU-baseline pass; the timed sample is then sized for about 4 s per pass")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of a workload, run a plain 256 MiB device copy 20 times (known traffic: 256 MiB read, "
                          "256 MiB written per launch) for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters")
