@@ -189,11 +189,12 @@ def kernel_ms(fn, reps):
 def gemm_kernel_name(m, n):
     t256 = ((m + 255) // 256) * ((n + 255) // 256)
     t128 = ((m + 127) // 128) * ((n + 255) // 256)
-    if m <= 4:
+    groups = (n + 31) // 32                # the library's choice: enough groups of 32 rows to give every CU a workgroup
+    xs = any((groups + rg - 1) // rg >= 192 for rg in range(4, 9))
+    if m == 1 or (m <= 4 and not xs):
         return "gemv_i4_kernel"
     if m <= 64:
-        groups = (n + 31) // 32            # the library's choice: enough groups of 32 rows to give every CU a workgroup
-        return "decode_xs_kernel" if any((groups + rg - 1) // rg >= 192 for rg in range(4, 9)) else "decode_i4_kernel"
+        return "decode_xs_kernel" if xs else "decode_i4_kernel"
     if t128 >= 128:         # the library's choice between its two pipelined kernels, by rounds of tiles
         return "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
     return "gemm_ks_kernel<64,256>"

@@ -2161,7 +2161,9 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-    if (M <= 4) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    // one to four tokens: the dot-product kernel -- except two to four tokens against a weight with enough rows for the
+    // shared-token kernel, which is ahead there (57344 x 8192: 40.2 against 42.9 us)
+    if (M == 1 || (M <= 4 && decode_xs_groups(n) == 0)) return launch_gemv(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     // too few tiles for the CUs: split K across workgroups when the caller passed scratch for the
     // slices' partial sums
     const int split = ks_split(M, N, kb);
