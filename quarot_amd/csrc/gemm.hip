@@ -189,8 +189,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
 
     // Epilogue.  Accumulator layout (first operand = W rows, second = X rows): lane l, register v ->
     // n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
-    // Whole tiles of an fp16 output leave as full rows through LDS, 64 columns (one line) at a time.
-    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    // Tiles of an fp16 output whose columns all exist leave as full rows through LDS, 64 columns (one
+    // line) at a time; a last row tile stores the rows that exist.
+    const bool by_rows = DEQ && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
     if (DEQ && by_rows) {
         constexpr int NJ = JN > 2 ? 2 : JN;                 // MFMA tiles per slab
         __syncthreads();                                    // every wave is done with the stage buffers
@@ -207,7 +208,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
-                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                const int row0 = m0 + wm * TM + i * 32;       // (rows past M: computed on a clamped scale, not stored)
+                if (row0 >= M) continue;
+                const f16 sa = sA[min(row0 + (lane & 31), M - 1)];
                 f16x4 o[NJ][4];
 #pragma unroll
                 for (int jj = 0; jj < NJ; ++jj)
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_i4_kernel(
                         o[jj][gq] = dequant4(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
                                              acc[i][jb + jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<NJ>((u32x2*)(lds_raw + wave * SLAB), o, lane,
-                                    Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+                                    Y + (int64_t)row0 * N + n0 + wn * TN + jb * 32, N, M - row0);
             }
         }
         return;
@@ -541,14 +544,16 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
                 }
             }
     }
-    // whole tiles of an fp16 output leave as full rows through LDS (each K-group its 64 columns)
-    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    // tiles of an fp16 output whose columns all exist leave as full rows through LDS (each K-group its 64 columns)
+    const bool by_rows = DEQ && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
     if (DEQ && by_rows) __syncthreads();                    // the exchange buffers are no longer read
 #pragma unroll
     for (int i = 0; i < IM; ++i) {
         const int row = m0 + wm * TM + i * 32 + (lane & 31);
         if (DEQ && by_rows) {
-            const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+            const int row0 = m0 + wm * TM + i * 32;           // (rows past M: computed on a clamped scale, not stored)
+            if (row0 >= M) continue;
+            const f16 sa = sA[min(row, M - 1)];
             f16x4 o[JH][4];
 #pragma unroll
             for (int j = 0; j < JN; ++j) {
@@ -563,7 +568,7 @@ __global__ __launch_bounds__(128 * WAVES_M * WAVES_N) void gemm_ks_kernel(
                     }
             }
             store_slab_rows<JH>((u32x2*)(ks_lds + wave * (32 * JH * 32 * 2 / 16)), o, lane,
-                                Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + j_first * 32, N);
+                                Y + (int64_t)row0 * N + n0 + wn * TN + j_first * 32, N, M - row0);
             continue;
         }
         if (row >= M) continue;
@@ -859,7 +864,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     __syncthreads();                                        // stage buffers free for the output slabs
 
     // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
-    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    const bool by_rows = DEQ && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
     if (DEQ && by_rows) {
 #pragma unroll
         for (int jb = 0; jb < JN; jb += 2) {
@@ -874,7 +879,9 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
-                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                const int row0 = m0 + wm * TM + i * 32;       // (rows past M: computed on a clamped scale, not stored)
+                if (row0 >= M) continue;
+                const f16 sa = sA[min(row0 + (lane & 31), M - 1)];
                 f16x4 o[2][4];
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)
@@ -883,7 +890,7 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
                         o[jj][gq] = dequant4(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
                                              acc[i][jb + jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<2>((u32x2*)(sp2_lds + wave * 256), o, lane,
-                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+                                   Y + (int64_t)row0 * N + n0 + wn * TN + jb * 32, N, M - row0);
             }
         }
         return;
@@ -1198,7 +1205,7 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     __syncthreads();                                        // stage buffers free for the output slabs
 
     // Epilogue: lane l, register v -> n = (v/4)*8 + (l/32)*4 + v%4, m = l%32.
-    const bool by_rows = DEQ && m0 + BM <= M && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
+    const bool by_rows = DEQ && n0 + BN <= N && (N & 7) == 0 && (((uintptr_t)Y) & 15) == 0;
     if (DEQ && by_rows) {
         const int jb = 2 * kg;
         {
@@ -1213,7 +1220,9 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
                 }
 #pragma unroll
             for (int i = 0; i < IM; ++i) {
-                const f16 sa = sA[m0 + wm * TM + i * 32 + (lane & 31)];
+                const int row0 = m0 + wm * TM + i * 32;       // (rows past M: computed on a clamped scale, not stored)
+                if (row0 >= M) continue;
+                const f16 sa = sA[min(row0 + (lane & 31), M - 1)];
                 f16x4 o[2][4];
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)
@@ -1222,7 +1231,7 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
                         o[jj][gq] = dequant4(acc[i][jj][gq * 4], acc[i][jj][gq * 4 + 1], acc[i][jj][gq * 4 + 2],
                                              acc[i][jj][gq * 4 + 3], sa, sbh[jj][gq], bih[jj][gq], bias != nullptr);
                 store_slab_rows<2>((u32x2*)(spk_lds + wave * 256), o, lane,
-                                   Y + (int64_t)(m0 + wm * TM + i * 32) * N + n0 + wn * TN + jb * 32, N);
+                                   Y + (int64_t)row0 * N + n0 + wn * TN + jb * 32, N, M - row0);
             }
         }
         return;

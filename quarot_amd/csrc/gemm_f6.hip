@@ -232,8 +232,8 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
                 for (int gq = 0; gq < 4; ++gq)
                     o[jj][gq] = dequant4_f32(acc[i][jb + jj][gq * 4], acc[i][jb + jj][gq * 4 + 1], acc[i][jb + jj][gq * 4 + 2],
                                              acc[i][jb + jj][gq * 4 + 3], sa, sbh[jb + jj][gq], bih[jb + jj][gq], DEQ_BIAS);
-            if (lines && row0 + 32 <= M && col0 + 64 <= N) {
-                store_slab_rows<2>((u32x2*)(f6_lds + wave * 256), o, lane, Y + (int64_t)row0 * N + col0, N);
+            if (lines && col0 + 64 <= N) {                  // (a last row tile stores the rows that exist)
+                store_slab_rows<2>((u32x2*)(f6_lds + wave * 256), o, lane, Y + (int64_t)row0 * N + col0, N, M - row0);
             } else if (row < M) {
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)

@@ -14,8 +14,11 @@ namespace {
 //   o[jj][gq] = this lane's columns jj*32 + gq*8 + (lane/32)*4 .. +3 of row lane%32.
 //   region: 32 * NJ * 8 slots of 8 bytes; the 8-byte slot index within a row is XORed with a key made
 //   from the row so that the 32 rows written by one instruction spread over all banks.
+//   rows: how many of the slab's 32 rows exist in the output (the last row tile of a token count that
+//   is no multiple of the tile height); the others are computed on clamped inputs and not stored.
 template <int NJ>
-__device__ __forceinline__ void store_slab_rows(u32x2* region, const f16x4 (&o)[NJ][4], int lane, f16* ybase, int N) {
+__device__ __forceinline__ void store_slab_rows(u32x2* region, const f16x4 (&o)[NJ][4], int lane, f16* ybase, int N,
+                                                int rows = 32) {
     constexpr int U = NJ * 8;                   // 8-byte slots per row
     constexpr int LPR = U / 2;                  // lanes (16 bytes each) per row on the way out
     constexpr int RPP = 64 / LPR;               // rows per store instruction
@@ -35,7 +38,7 @@ __device__ __forceinline__ void store_slab_rows(u32x2* region, const f16x4 (&o)[
         const int key = (rr * U / 32) & (U - 1);
         u32x4 v = region16[rr * LPR + (s ^ (key >> 1))];
         if (key & 1) v = u32x4{v[2], v[3], v[0], v[1]};
-        *(u32x4*)(ybase + (int64_t)rr * N + s * 8) = v;
+        if (rr < rows) *(u32x4*)(ybase + (int64_t)rr * N + s * 8) = v;
     }
 }
 

@@ -181,6 +181,43 @@ def test_matmul_and_linear_random_shapes_across_every_kernel_boundary():
         assert np.array_equal(bits(y.cpu().numpy()), bits(o.sym_dequant(want, sa, sw, bias))), (m, n, k)
 
 
+@pytest.mark.parametrize("m,n,k", [(2047, 4096, 256), (2049, 4096, 320), (1900, 4096, 128), (1153, 8192, 128), (1025, 8192, 192),
+                                   (300, 512, 192), (130, 4096, 1024), (97, 1024, 2048), (65, 768, 64), (4001, 4096, 64),
+                                   (257, 2048, 448), (161, 256, 4096)])
+def test_linear_token_counts_that_end_inside_a_row_tile(m, n, k):
+    """Prompt lengths that are no multiple of the kernels' tile heights (32-row slabs of 64/128/256-row tiles)
+    against weights whose rows fill whole tiles: the last row tile stores exactly the rows that exist.  Through
+    the C-ABI into a buffer with a guard band behind the last row, with and without bias, on the int8 and the
+    FP6 matrix paths; the oracle decides bit for bit."""
+    from quarot_amd import _lib
+    rng = np.random.default_rng(m * 3 + n + k)
+    a, w = o.pack_i4(rng.integers(-8, 8, (m, k))), o.pack_i4(rng.integers(-8, 8, (n, k)))
+    sa = (np.abs(rng.standard_normal(m)) * 0.2 + 0.01).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01 + 0.001).astype(F16)
+    bias = rng.standard_normal(n).astype(F16)
+    acc = o.int4_matmul(a, w)
+    ga, gw, gsa, gsw, gb = gpu(a), gpu(w), gpu(sa), gpu(sw), gpu(bias)
+    a6, w6 = quarot_amd.convert_i4_f6(ga), quarot_amd.convert_i4_f6(gw)
+    L = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    guard = 40                                               # rows behind the output that no kernel may touch
+    for b, nb in ((gb, bias), (None, None)):
+        want = bits(o.sym_dequant(acc, sa, sw, nb))
+        for path in ("i8", "f6"):
+            buf = torch.full((m + guard, n), 12345.0, dtype=torch.float16, device="cuda")
+            bp = b.data_ptr() if b is not None else None
+            if path == "i8":
+                rc = L.qr_linear_i4_f16(ga.data_ptr(), gsa.data_ptr(), gw.data_ptr(), gsw.data_ptr(), bp, m, n, k,
+                                        buf.data_ptr(), stream)
+            else:
+                rc = L.qr_linear_f6_f16(a6.data_ptr(), gsa.data_ptr(), w6.data_ptr(), gsw.data_ptr(), bp, m, n, k,
+                                        buf.data_ptr(), stream)
+            assert rc == 0, (path, rc)
+            got = buf.cpu().numpy()
+            assert np.array_equal(bits(got[:m]), want), (path, nb is not None)
+            assert (got[m:] == 12345.0).all(), (path, "rows behind the output were written")
+
+
 @pytest.mark.parametrize("n", [25600, 35200, 44800, 57344, 65536, 57339, 65500])
 def test_decode_with_many_weight_rows_shares_the_tokens_through_lds(n):
     """Decode batches (5..64 tokens) against enough weight rows to give every CU a workgroup of 4..8 groups
