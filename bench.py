@@ -196,7 +196,7 @@ def gemm_kernel_name(m, n):
     if m <= 64:
         return "decode_xs_kernel" if xs else "decode_i4_kernel"
     if t128 >= 128:         # the library's choice between its two pipelined kernels, by rounds of tiles
-        return "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.61 else "gemm_spk_kernel"
+        return "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.57 else "gemm_spk_kernel"
     return "gemm_ks_kernel<64,256>"
 
 

@@ -2197,9 +2197,10 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (t128x256 >= cus / 2) {
         // 256x256 tiles run ~1.2x faster per unit of work (3 instead of 4.5 unpacking instructions per
         // MFMA) but quantise worse over the 256 CUs: compare rounds of tiles, a 128x256 tile costing
-        // 0.61 of a 256x256 one
+        // 0.57 of a 256x256 one (measured over 1152..3000 tokens against 4096..27648 weight rows: rounds of
+        // 27-29 us against 48-51 us at K = 4096; with 0.57 every one of those shapes gets the faster kernel)
         const double rounds256 = (double)((t256 + cus - 1) / cus);
-        const double rounds128 = (double)((t128x256 + cus - 1) / cus) * 0.61;
+        const double rounds128 = (double)((t128x256 + cus - 1) / cus) * 0.57;
         if (rounds256 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
         return launch_spk(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
