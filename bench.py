@@ -195,8 +195,10 @@ def gemm_kernel_name(m, n):
         return "gemv_i4_kernel"
     if m <= 64:
         return "decode_xs_kernel" if xs else "decode_i4_kernel"
-    if t128 >= 128:         # the library's choice between its two pipelined kernels, by rounds of tiles
-        return "gemm_sp256_kernel" if (t256 + 255) // 256 <= ((t128 + 255) // 256) * 0.57 else "gemm_spk_kernel"
+    if t128 >= 128:         # the library's choice between its pipelined kernels, by rounds of tiles (256-, 192- or 128-row)
+        t192 = ((m + 191) // 192) * ((n + 255) // 256)
+        r256, r192, r128 = (t256 + 255) // 256, ((t192 + 255) // 256) * 0.80, ((t128 + 255) // 256) * 0.57
+        return "gemm_sp256_kernel" if (r256 <= r128 and r256 <= r192) or r192 <= r128 else "gemm_spk_kernel"
     return "gemm_ks_kernel<64,256>"
 
 

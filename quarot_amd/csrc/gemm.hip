@@ -658,19 +658,24 @@ int launch_ks(const void* A, const void* B, int M, int N, int Kb, void* C, void*
 // (a 128-byte line per row); two LDS stage buffers; global loads are raw buffer loads (scalar
 // descriptor + scalar stage offset + constant 32-bit lane offset: no address arithmetic in the loop)
 // running ahead in registers; one workgroup barrier per stage.
-//   gemm_sp256_kernel  256x256 tile, waves 2 (M) x 2 (N), whole K per wave: shapes with many tiles.
+//   gemm_sp256_kernel  256x256 tile, waves 2 (M) x 2 (N), whole K per wave: shapes with many tiles.  Also as a
+//                      192x256 tile (wave tiles of 96x128: 12 MFMA tiles, 3.5 unpacking instructions per
+//                      MFMA) for shapes that 256-row tiles spread over a fraction of the CUs and 128-row
+//                      tiles over a round and a bit (2048 tokens against 5120 weight rows: 160 / 220 /
+//                      320 tiles of 256 / 192 / 128 rows on 256 CUs).
 //   gemm_spk_kernel    128x256 tile (one per CU at M = 2048, N = 4096), waves 2 (N) x 2 (K): the two
 //                      K-groups take alternate pairs of sub-steps and exchange half of their
 //                      accumulators through LDS at the end.
-template <bool DEQ, bool RAGGED>
+template <bool DEQ, bool RAGGED, int BM = 256>
 __global__ __launch_bounds__(256) void gemm_sp256_kernel(
     const uint8_t* __restrict__ A, const uint8_t* __restrict__ B, int M, int N, int Kb, int32_t* __restrict__ C,
     f16* __restrict__ Y, const f16* __restrict__ sA, const f16* __restrict__ sB, const f16* __restrict__ bias,
     int tiles_m, int tiles_n, int nxcd) {
-    constexpr int BM = 256, BN = 256, NT = 256;
-    constexpr int TM = 128, TN = 128, IM = 4, JN = 4;
+    static_assert(BM == 256 || BM == 192, "wave tiles of 4 or 3 accumulator tiles along M");
+    constexpr int BN = 256, NT = 256;
+    constexpr int TM = BM / 2, TN = 128, IM = TM / 32, JN = 4;
     constexpr int CH = (BM + BN) * 8;                       // 16-byte chunks per stage
-    constexpr int NL = CH / NT;                             // 16 per thread
+    constexpr int NL = CH / NT;                             // 16 (14) per thread
     constexpr int NF = IM + JN;                             // fragments per sub-step
     constexpr int NMF = 2 * IM * JN;                        // MFMAs (= slots) per sub-step
     constexpr int UNP = NF * 12;                            // unpacking instructions per sub-step
@@ -733,8 +738,11 @@ __global__ __launch_bounds__(256) void gemm_sp256_kernel(
         const int kb = (st < stages ? st : stages - 1) * 128;
         __attribute__((address_space(3))) void* dst =
             (__attribute__((address_space(3))) void*)(sp2_lds + buf * CH + i * NT + wave_u * 64);
-        if (i * 32 < BM) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, goff[i], kb, 0, 0);
-        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, goff[i], kb, 0, 0);
+        // (off: a plain u32 -- goff's bound depends on a template parameter, and with such an operand the
+        // host pass silently drops the kernel's stub)
+        const u32 off = goff[i];
+        if (i * 32 < BM) __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, dst, 16, off, kb, 0, 0);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, dst, 16, off, kb, 0, 0);
     };
 
     i32x16 acc[IM][JN];
@@ -1303,10 +1311,12 @@ template <int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_cfg(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
                const void* bias, hipStream_t st);
 
+// bm: rows of a tile, 256 or 192 (192: eleven row tiles instead of eight at 2048 tokens -- shapes whose
+// 256-row tiles would occupy a fraction of the CUs and whose 128-row tiles need a second round)
 int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA, const void* sB,
-                 const void* bias, hipStream_t st) {
-    constexpr size_t LDS = (size_t)2 * (256 + 256) * 8 * 16;
-    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+                 const void* bias, hipStream_t st, int bm = 256) {
+    const size_t LDS = (size_t)2 * (size_t)(bm + 256) * 8 * 16;
+    const int tiles_m = (M + bm - 1) / bm, tiles_n = (N + 255) / 256;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
@@ -1315,20 +1325,22 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
     // operands are addressed through 32-bit buffer offsets
     if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
         return launch_cfg<256, 256, 4, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
-    hipError_t e;
-    if (Y) {
-        auto kern = ragged ? gemm_sp256_kernel<true, true> : gemm_sp256_kernel<true, false>;
-        e = qr_allow_dynamic_lds((const void*)kern, LDS);
-        if (e != hipSuccess) return (int)e;
+    using Kern = void (*)(const uint8_t*, const uint8_t*, int, int, int, int32_t*, f16*, const f16*, const f16*, const f16*,
+                          int, int, int);
+    static const Kern table[2][2][2] = {
+        {{gemm_sp256_kernel<false, false, 256>, gemm_sp256_kernel<false, true, 256>},
+         {gemm_sp256_kernel<true, false, 256>, gemm_sp256_kernel<true, true, 256>}},
+        {{gemm_sp256_kernel<false, false, 192>, gemm_sp256_kernel<false, true, 192>},
+         {gemm_sp256_kernel<true, false, 192>, gemm_sp256_kernel<true, true, 192>}}};
+    const Kern kern = table[bm == 192 ? 1 : 0][Y ? 1 : 0][ragged ? 1 : 0];
+    const hipError_t e = qr_allow_dynamic_lds((const void*)kern, LDS);
+    if (e != hipSuccess) return (int)e;
+    if (Y)
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y,
                                                  (const f16*)sA, (const f16*)sB, (const f16*)bias, tiles_m, tiles_n, nxcd);
-    } else {
-        auto kern = ragged ? gemm_sp256_kernel<false, true> : gemm_sp256_kernel<false, false>;
-        e = qr_allow_dynamic_lds((const void*)kern, LDS);
-        if (e != hipSuccess) return (int)e;
+    else
         kern<<<dim3(grid), dim3(256), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C, nullptr,
                                                  nullptr, nullptr, nullptr, tiles_m, tiles_n, nxcd);
-    }
     return qr_launch_status();
 }
 
@@ -2195,13 +2207,17 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     const int64_t t128x256 = ((M + 127) / 128) * ((N + 255) / 256);
     const int64_t cus = qr_device().cus;
     if (t128x256 >= cus / 2) {
-        // 256x256 tiles run ~1.2x faster per unit of work (3 instead of 4.5 unpacking instructions per
-        // MFMA) but quantise worse over the 256 CUs: compare rounds of tiles, a 128x256 tile costing
-        // 0.57 of a 256x256 one (measured over 1152..3000 tokens against 4096..27648 weight rows: rounds of
-        // 27-29 us against 48-51 us at K = 4096; with 0.57 every one of those shapes gets the faster kernel)
+        // Taller tiles run faster per unit of work (3 unpacking instructions per MFMA at 256 rows, 3.5 at 192,
+        // 4.5 at 128) but quantise worse over the 256 CUs: compare rounds of tiles, a 128x256 tile costing 0.57
+        // and a 192x256 tile 0.80 of a 256x256 one (measured over 300..4096 tokens against 4096..27648 weight
+        // rows: rounds of 27-29 / 40-41 / 48-51 us at K = 4096; with these ratios every one of those shapes gets
+        // the fastest kernel).  Ties go to the taller tile.
+        const int64_t t192 = ((M + 191) / 192) * ((N + 255) / 256);
         const double rounds256 = (double)((t256 + cus - 1) / cus);
+        const double rounds192 = (double)((t192 + cus - 1) / cus) * 0.80;
         const double rounds128 = (double)((t128x256 + cus - 1) / cus) * 0.57;
-        if (rounds256 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        if (rounds256 <= rounds128 && rounds256 <= rounds192) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        if (rounds192 <= rounds128) return launch_sp256(A, B, m, n, kb, C, Y, sA, sB, bias, st, 192);
         return launch_spk(A, B, m, n, kb, C, Y, sA, sB, bias, st);
     }
     if (N > 128) return launch_ks<64, 256, 1, 4>(A, B, m, n, kb, C, Y, sA, sB, bias, st);

@@ -73,13 +73,13 @@ __global__ __launch_bounds__(256) void convert_i4_f6_kernel(const u32x4* __restr
 }
 
 // ------------------------------------------------------------------------------------------------
-// TM x 256 tile (TM = 256, or 128 when 256-row tiles would leave compute units idle), four waves (one per
+// TM x 256 tile (TM = 256, or 192 / 128 when taller tiles would leave compute units idle), four waves (one per
 // SIMD) as 2 (M) x 2 (N), each a TM/2 x 128 wave tile = TM/64 x 4 accumulator tiles of 32 x 32.  A stage
 // is 64 k: TM * 48 bytes of X6 and 12 KB of W6, each one contiguous run, loaded straight into LDS
 // (buffer_load ... lds: a wave's 64 lanes fill 1 KB of consecutive LDS); six stage buffers, loads five
-// stages ahead.  (At TM = 128 the X6 run is 1.5 rounds of the workgroup's 4 KB: waves 2 and 3 aim the
-// second round past the end of the operand, which fetches nothing, and at a spare 2 KB of LDS, so that
-// every wave has the same number of loads in flight and one wait count serves all.)  Rows are 48 bytes apart in LDS: the 16 rows that a quarter-wave
+// stages ahead.  (At TM = 128 the X6 run is 1.5 rounds of the workgroup's 4 KB, at TM = 192 2.25: the waves
+// without a share of the last round aim it past the end of the operand, which fetches nothing, and at a spare
+// 2 KB of LDS, so that every wave has the same number of loads in flight and one wait count serves all.)  Rows are 48 bytes apart in LDS: the 16 rows that a quarter-wave
 // reads at one offset start in 16 different groups of four banks (12 r mod 64), so the 16-byte and 8-byte
 // reads that assemble an operand (24 bytes: halves of the row at byte 0 / 16 and 32 / 24) have no bank
 // conflicts and nothing is padded or swizzled.  Nothing is unpacked: fragments go from LDS to the
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void gemm_f6_kernel(const uint8_t* __restrict_
     // The epilogue's scales (and bias) of this tile's columns and rows are fetched first and parked in LDS
     // behind the stage buffers, so that the epilogue finds them without waiting for memory (indices clamped
     // to the matrix: values of rows and columns beyond it are never stored).
-    f16* const scale_lds = (f16*)(f6_lds + NBUF * BUF + (TM == 128 ? 128 : 0));     // [256] sB, [256] bias, [TM] sA
+    f16* const scale_lds = (f16*)(f6_lds + NBUF * BUF + (TM == 256 ? 0 : 128));     // [256] sB, [256] bias, [TM] sA
     const int ccol = n0 + tid < N ? n0 + tid : N - 1, crow = m0 + tid < M ? m0 + tid : M - 1;
     const f16 pre_sb = sB[ccol], pre_bi = DEQ_BIAS ? bias[ccol] : (f16)0, pre_sa = sA[crow];
 #pragma unroll
@@ -282,10 +282,14 @@ extern "C" int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, 
     if ((double)M * (double)K * 0.75 >= 4294901760.0 || (double)N * (double)K * 0.75 >= 4294901760.0) return QR_E_UNSUPPORTED;
     const int nxcd = qr_device().xcds, cus = qr_device().cus;
     const int tiles_n = (int)((N + 255) / 256);
-    // 256-row tiles unless 128-row ones fill the device in fewer rounds (a 128-row tile costs ~0.6 of a 256-row one)
-    const int64_t t256 = (M + 255) / 256 * tiles_n, t128 = (M + 127) / 128 * tiles_n;
-    const bool narrow = (double)((t128 + cus - 1) / cus) * 0.6 < (double)((t256 + cus - 1) / cus);
-    const int tiles_m = (int)(narrow ? (M + 127) / 128 : (M + 255) / 256);
+    // 256-row tiles unless 192- or 128-row ones fill the device in fewer rounds (measured on single rounds at
+    // K = 4096 .. 13824: a 128-row tile costs 0.73 and a 192-row tile 0.87 of a 256-row one); ties go to the
+    // taller tile
+    const int64_t t256 = (M + 255) / 256 * tiles_n, t192 = (M + 191) / 192 * tiles_n, t128 = (M + 127) / 128 * tiles_n;
+    const double r256 = (double)((t256 + cus - 1) / cus), r192 = (double)((t192 + cus - 1) / cus) * 0.87,
+                 r128 = (double)((t128 + cus - 1) / cus) * 0.73;
+    int tm_rows = (r256 <= r192 && r256 <= r128) ? 256 : (r192 <= r128 ? 192 : 128);
+    const int tiles_m = (int)((M + tm_rows - 1) / tm_rows);
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
     if (tiles > 0x3fffffff) return QR_E_SHAPE;
     const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
@@ -297,8 +301,10 @@ extern "C" int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, 
                                                    (const f16*)sA, (const f16*)sW, (const f16*)bias_or_null, tiles_m, tiles_n, nxcd);
         return qr_launch_status();
     };
-    // six stage buffers (+ the spare 2 KB that idle loads of 128-row tiles aim at) + 1.5 KB of scales for the epilogue
-    constexpr size_t LDS256 = (size_t)(6 * (768 + 768) + 96) * 16, LDS128 = (size_t)(6 * (384 + 768) + 128 + 96) * 16;
-    if (narrow) return bias_or_null ? launch(gemm_f6_kernel<128, true>, LDS128) : launch(gemm_f6_kernel<128, false>, LDS128);
+    // six stage buffers (+ the spare 2 KB that idle loads of 128- and 192-row tiles aim at) + 1.5 KB of scales for the epilogue
+    constexpr size_t LDS256 = (size_t)(6 * (768 + 768) + 96) * 16, LDS192 = (size_t)(6 * (576 + 768) + 128 + 96) * 16,
+                     LDS128 = (size_t)(6 * (384 + 768) + 128 + 96) * 16;
+    if (tm_rows == 128) return bias_or_null ? launch(gemm_f6_kernel<128, true>, LDS128) : launch(gemm_f6_kernel<128, false>, LDS128);
+    if (tm_rows == 192) return bias_or_null ? launch(gemm_f6_kernel<192, true>, LDS192) : launch(gemm_f6_kernel<192, false>, LDS192);
     return bias_or_null ? launch(gemm_f6_kernel<256, true>, LDS256) : launch(gemm_f6_kernel<256, false>, LDS256);
 }

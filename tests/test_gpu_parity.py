@@ -183,7 +183,9 @@ def test_matmul_and_linear_random_shapes_across_every_kernel_boundary():
 
 @pytest.mark.parametrize("m,n,k", [(2047, 4096, 256), (2049, 4096, 320), (1900, 4096, 128), (1153, 8192, 128), (1025, 8192, 192),
                                    (300, 512, 192), (130, 4096, 1024), (97, 1024, 2048), (65, 768, 64), (4001, 4096, 64),
-                                   (257, 2048, 448), (161, 256, 4096)])
+                                   (257, 2048, 448), (161, 256, 4096),
+                                   # 192-row tiles (fewer rounds over the CUs than 128- or 256-row ones), whole K stages
+                                   (2049, 4096, 512), (1153, 8192, 256), (1920, 5120, 256), (2048, 5120, 768)])
 def test_linear_token_counts_that_end_inside_a_row_tile(m, n, k):
     """Prompt lengths that are no multiple of the kernels' tile heights (32-row slabs of 64/128/256-row tiles)
     against weights whose rows fill whole tiles: the last row tile stores exactly the rows that exist.  Through
