@@ -121,7 +121,7 @@ class Linear4bitSequential(torch.nn.Sequential):
 
 def enable_fp6_prefill(module, min_rows=1024, convert_now=True):
     """Opt every Linear4bit under `module` into the FP6 matrix path for inputs of at least `min_rows`
-    rows (prompts): the same results bit for bit, whole steps 14-22 % faster at 2048 rows of the 13B / 70B
+    rows (prompts): the same results bit for bit, whole steps 10-16 % faster at 2048 rows of the 13B / 70B
     widths and 16 % at 32768 rows of the 7B ones (level at 2048 rows of the 7B widths), for a
     6-bit copy of each weight (1.5 x its packed size, kept beside the 4-bit one that decode streams)
     and a conversion pass over the activations' codes.  convert_now: make the copies here rather
