@@ -52,6 +52,11 @@ __device__ __forceinline__ f16x2 kv_pair_min(f16x2 p) {
 // Eight codes clamp(round_half_even(fp16(fp16(x + zero) / scale)), 0, 15) for all-finite input: the
 // add is one packed fp16 add, the division the exact-product / fma form of sym_codes8_fast (the
 // shifted value has at most 11 significant bits), the rounding the +1536 trick.
+// CLAMP = false leaves the clamp out: the shifted values lie in [0, range] by construction, so with a
+// scale that is a NORMAL fp16 number (relative rounding error <= 2^-11: range >= 2^-10 is enough) the
+// quotient is at most 15 (1 + 2^-11) and rounds to 15 at most.  A subnormal scale can be off by several
+// per cent and needs the clamp (range / 15 = 10.5 units of 2^-24 -> scale 10 units -> quotient 15.75).
+template <bool CLAMP = true>
 __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) {
     const f16x2 z2 = {zero, zero};
     u32 b[4];
@@ -61,14 +66,18 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
         const float x0 = (float)sh[0], x1 = (float)sh[1];
         float q0 = __builtin_fmaf(x0, f.rl, __builtin_fmaf(x0, f.rh, 0.0f));
         float q1 = __builtin_fmaf(x1, f.rl, __builtin_fmaf(x1, f.rh, 0.0f));
-        q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
-        q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);
+        if (CLAMP) {
+            q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
+            q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);
+        }
         f16x2 h = {(f16)q0, (f16)q1};
         h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
         b[i] = __builtin_bit_cast(u32, h);
     }
     return pack_nibbles8(b);
 }
+// ranges from which the clamp-free form is exact (see above)
+__device__ __forceinline__ bool asym_range_normal(f16 rng) { return rng >= (f16)0.0009765625f; }
 
 // LG = log2(lanes per vector) = log2(dim) - 3, 1..5
 // PAGED (head dimension 128 only): codes and {scale, zero} go straight to the vector's place in the paged
@@ -145,7 +154,9 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
             rng = rng < floor_ ? floor_ : rng;
             sc = narrow_f16((float)rng * (1.0f / 15.0f));
             zp = -mn;
-            outw = asym_codes8_fast(hp, zp, make_fast_recip((float)sc));
+            const FastRecip fr = make_fast_recip((float)sc);
+            if (__builtin_amdgcn_ballot_w64(!asym_range_normal(rng)) == 0) outw = asym_codes8_fast<false>(hp, zp, fr);
+            else outw = asym_codes8_fast<true>(hp, zp, fr);
         } else {
             float v[8];
 #pragma unroll
@@ -207,7 +218,7 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
                       if ((lane & ((1 << LG) - 1)) == 0) pd.c.param[s] = pack_scale_zero(scs[u], zps[u]);
                   }
               } else {
-                  q[c] = outws[u];
+                  __builtin_nontemporal_store(outws[u], q + c);
                   if ((lane & ((1 << LG) - 1)) == 0) {
                       scale[c >> LG] = scs[u];
                       zero[c >> LG] = zps[u];
@@ -320,15 +331,31 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
         for (int c = 0; c < 8; ++c) {
             int64_t row = b * 32 + 4 * c + (lane >> 4);
             row = row < vectors ? row : vectors - 1;               // the last block may be short: repeat its last row
-            pre[c] = src[row * 16 + (lane & 15)];
+            pre[c] = __builtin_nontemporal_load(src + row * 16 + (lane & 15));     // (streamed once: 70 -> 65.5 us on 268 MB in, then 63 us with the codes leaving as nontemporal stores too)
         }
     };
-    if (blk < blocks) fetch(blk);
-    for (; blk < blocks; blk += wstride) {
-        // LDS operations of one wave execute in order: these writes follow the previous block's reads
-#pragma unroll
+    // The loop is rotated so that every turn issues the same memory operations in the same order, without a
+    // branch around any of them: [fragment reads] [transform, quantiser] [stores of block b] [wait for the loads
+    // of block b + 1, issued a turn earlier and therefore OLDER than those stores; stage them] [loads of block
+    // b + 2].  The wait then counts the stores as still allowed in flight; with a conditional load or store
+    // anywhere in the turn the compiler has to wait for everything, i.e. for the stores' round trip, every turn.
+    // (Past the end the last block is fetched again, and rows past the end repeat the last row: their lanes
+    // compute the last vector's values once more and store them to the last vector's place.)
+    auto stage_in = [&]() {                                        // LDS operations of one wave execute in order:
+#pragma unroll                                                     // these writes follow the current block's reads
         for (int c = 0; c < 8; ++c) stage[km_slot(4 * c + (lane >> 4), lane & 15)] = pre[c];
-        if (blk + wstride < blocks) fetch(blk + wstride);
+    };
+    auto turn_end = [&](int64_t b) {                               // b: the block just finished
+        stage_in();
+        const int64_t nb = b + 2 * wstride;
+        fetch(nb < blocks ? nb : blocks - 1);
+    };
+    if (blk < blocks) {
+        fetch(blk);
+        stage_in();
+        fetch(blk + wstride < blocks ? blk + wstride : blocks - 1);
+    }
+    for (; blk < blocks; blk += wstride) {
         u32x4 xf[8];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) xf[ks] = stage[km_slot(v, 2 * ks + h)];
@@ -380,50 +407,70 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
             for (int c = 0; c < 8; ++c) {
                 const int row = 4 * c + (lane >> 4);
                 const u32x4 o = stage[km_slot(row, lane & 15)];
-                if (blk * 32 + row < vectors) y[(blk * 32 + row) * 16 + (lane & 15)] = o;
+                int64_t grow = blk * 32 + row;
+                grow = grow < vectors ? grow : vectors - 1;        // (a repeat of the last row: the same values again)
+                y[grow * 16 + (lane & 15)] = o;                    // (plain: as a nontemporal store 81 -> 91 us on 2 x 268 MB)
             }
+            turn_end(blk);
             continue;
         }
-        // ---- quantiser on the lane's 64 values
-        u16x2 am2 = {0, 0};                                        // largest magnitude bits: >= 0x7c00 means inf or NaN
+        // ---- quantiser on the lane's 64 values: packed minimum and maximum first
+        f16x2 mn2 = as_f16x2(yw[0][0][0]), mx2 = mn2;
 #pragma unroll
         for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
             for (int qq = 0; qq < 4; ++qq)
 #pragma unroll
-                for (int w = 0; w < 2; ++w)
-                    am2 = __builtin_elementwise_max(am2, __builtin_bit_cast(u16x2, yw[jt][qq][w] & 0x7fff7fffu));
-        const u32 amax = am2[0] > am2[1] ? am2[0] : am2[1];
-        const bool finite = __builtin_amdgcn_ballot_w64(amax >= 0x7c00u) == 0;
-        f16 sc, zp;
-        u32 U[8];
-        if (finite) {
-            f16x2 mn2 = as_f16x2(yw[0][0][0]), mx2 = mn2;
+                for (int w = 0; w < 2; ++w) {
+                    mn2 = __builtin_elementwise_min(mn2, as_f16x2(yw[jt][qq][w]));
+                    mx2 = __builtin_elementwise_max(mx2, as_f16x2(yw[jt][qq][w]));
+                }
+        const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+        const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+        f16x2 pr = {mn0, -mx0};                                    // (min, -max): one packed min across the two lanes
+        const f16x2 other = as_f16x2((u32)__shfl_xor((int)__builtin_bit_cast(u32, pr), 32, 64));
+        pr = __builtin_elementwise_min(pr, other);
+        const f16 mn = pr[0], mx = -pr[1];
+        // Is every value finite?  Behind the transform that needs no pass over the values: an infinity or NaN in
+        // a vector reaches EVERY output of that vector (each is a sum of all 128 inputs times +-1), so one output
+        // tells; what is left is a finite sum too large for fp16, and that shows in the minimum or maximum.
+        // Parts that pass through the identity (appends) are looked at value by value.
+        bool bad;
+        if (PAGED) {
+            u16x2 am2 = {0, 0};                                    // largest magnitude bits: >= 0x7c00 means inf or NaN
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
                 for (int qq = 0; qq < 4; ++qq)
 #pragma unroll
-                    for (int w = 0; w < 2; ++w) {
-                        mn2 = __builtin_elementwise_min(mn2, as_f16x2(yw[jt][qq][w]));
-                        mx2 = __builtin_elementwise_max(mx2, as_f16x2(yw[jt][qq][w]));
-                    }
-            const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
-            const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
-            f16x2 pr = {mn0, -mx0};                                // (min, -max): one packed min across the two lanes
-            const f16x2 other = as_f16x2((u32)__shfl_xor((int)__builtin_bit_cast(u32, pr), 32, 64));
-            pr = __builtin_elementwise_min(pr, other);
-            const f16 mn = pr[0], mx = -pr[1];
+                    for (int w = 0; w < 2; ++w)
+                        am2 = __builtin_elementwise_max(am2, __builtin_bit_cast(u16x2, yw[jt][qq][w] & 0x7fff7fffu));
+            bad = (am2[0] > am2[1] ? am2[0] : am2[1]) >= 0x7c00u;
+        } else {
+            bad = (yw[0][0][0] & 0x7c00u) == 0x7c00u || (f16_bits(mn) & 0x7fffu) >= 0x7c00u || (f16_bits(mx) & 0x7fffu) >= 0x7c00u;
+        }
+        const bool finite = __builtin_amdgcn_ballot_w64(bad) == 0;
+        f16 sc, zp;
+        u32 U[8];
+        if (finite) {
             f16 rng = narrow_f16((float)mx - (float)mn);
             const f16 floor_ = (f16)1e-5f;
             rng = rng < floor_ ? floor_ : rng;
             sc = narrow_f16((float)rng * (1.0f / 15.0f));
             zp = -mn;
             const FastRecip fr = make_fast_recip((float)sc);
+            if (__builtin_amdgcn_ballot_w64(!asym_range_normal(rng)) == 0) {
 #pragma unroll
-            for (int m = 0; m < 8; ++m) {
-                const int jt = m >> 1, q0 = (m & 1) * 2;
-                U[m] = asym_codes8_fast(u32x4{yw[jt][q0][0], yw[jt][q0][1], yw[jt][q0 + 1][0], yw[jt][q0 + 1][1]}, zp, fr);
+                for (int m = 0; m < 8; ++m) {
+                    const int jt = m >> 1, q0 = (m & 1) * 2;
+                    U[m] = asym_codes8_fast<false>(u32x4{yw[jt][q0][0], yw[jt][q0][1], yw[jt][q0 + 1][0], yw[jt][q0 + 1][1]}, zp, fr);
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < 8; ++m) {
+                    const int jt = m >> 1, q0 = (m & 1) * 2;
+                    U[m] = asym_codes8_fast<true>(u32x4{yw[jt][q0][0], yw[jt][q0][1], yw[jt][q0 + 1][0], yw[jt][q0 + 1][1]}, zp, fr);
+                }
             }
         } else {
             // a NaN anywhere in a vector makes its range, scale and zero NaN and every code 0 (torch's
@@ -485,8 +532,14 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
             W[2 * m] = __builtin_amdgcn_perm(sw[1], sw[0], 0x05040100u);
             W[2 * m + 1] = __builtin_amdgcn_perm(sw[1], sw[0], 0x07060302u);
         }
-        if (vec < vectors) {
-            if (PAGED) {
+        if (!PAGED) {
+            const int64_t vc = vec < vectors ? vec : vectors - 1;  // (lanes past the end hold the last vector's values)
+            __builtin_nontemporal_store(u32x4{W[0], W[1], W[2], W[3]}, q + vc * 4 + 2 * h);
+            __builtin_nontemporal_store(u32x4{W[4], W[5], W[6], W[7]}, q + vc * 4 + 2 * h + 1);
+            scale[vc] = sc;                                        // both lanes of a vector: the same two values
+            zero[vc] = zp;
+        } else if (vec < vectors) {
+            {
                 const int64_t token = vec / pd.c.num_heads;
                 int64_t page;
                 int entry;
@@ -497,15 +550,9 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                     dst[1] = u32x4{W[4], W[5], W[6], W[7]};
                     if (h == 0) pd.c.param[s] = pack_scale_zero(sc, zp);
                 }
-            } else {
-                q[vec * 4 + 2 * h] = u32x4{W[0], W[1], W[2], W[3]};
-                q[vec * 4 + 2 * h + 1] = u32x4{W[4], W[5], W[6], W[7]};
-                if (h == 0) {
-                    scale[vec] = sc;
-                    zero[vec] = zp;
-                }
             }
         }
+        turn_end(blk);
     }
 }
 

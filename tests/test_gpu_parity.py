@@ -783,6 +783,44 @@ def test_kv_quant_dequant_bit_exact(dim, hadamard):
     assert bool((err <= s.float() / 2 + 0.004 * (15 * s.float() + z.float().abs()) + 1e-3).all())
 
 
+@pytest.mark.parametrize("dim", [64, 128])
+@pytest.mark.parametrize("hadamard", [False, True])
+def test_kv_tiny_ranges_and_sums_too_large_for_fp16(dim, hadamard):
+    """The corners of the quantiser's lean path: ranges so small that the scale is a subnormal fp16 number (its
+    rounding error then reaches several per cent and the largest quotient passes 15.5: the clamp decides), ranges
+    at the 1e-5 floor, and -- behind the Hadamard -- finite vectors whose transform overflows fp16 in SOME outputs
+    only (all elements 60000: the first output is 128 * 60000 / sqrt(128) = inf, every other one 0).  Mixed with
+    ordinary vectors in the same waves; codes, scales and zeros against the oracle bit for bit."""
+    rng = np.random.default_rng(dim + hadamard)
+    v = 640
+    x = rng.standard_normal((v, dim)).astype(np.float64)
+    for i in range(0, 200):                                  # ranges from 5e-6 to 2e-3 around various offsets
+        span = 5e-6 * (400.0 ** (i / 199.0))
+        base = (0.0, 0.01, -0.3, 1.0)[i % 4]
+        x[i] = base + span * rng.random(dim)
+        x[i, 0], x[i, 1] = base, base + span
+    if hadamard:                                             # (transformed ranges: scaled so that the outputs are tiny)
+        x[200:260] = rng.standard_normal((60, dim)) * (10.0 ** rng.uniform(-5.5, -2.5, (60, 1)))
+        x[300] = 60000.0
+        x[301] = -60000.0
+        x[302] = 60000.0 * np.where(np.arange(dim) % 2 == 0, 1.0, -1.0)
+        x[303, :] = 0.0
+        x[303, :4] = 65504.0
+    x = x.astype(F16)
+    q, s, z = kv.asym_quantize_and_pack_i4(gpu(x), hadamard=hadamard)
+    xin = x
+    if hadamard:
+        xin = kv.matmul_had_cuda(gpu(x), torch.float16).cpu().numpy()
+        with np.errstate(over="ignore", invalid="ignore"):
+            assert close(xin[:300], o.kv_hadamard(x[:300]))
+        assert np.isinf(xin[300]).sum() == 1 and np.isinf(xin[301]).sum() == 1 and np.isinf(xin[302]).sum() == 1
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore"):
+        wq, ws, wz = o.kv_asym_quant(xin)
+    assert np.array_equal(q.cpu().numpy(), wq)
+    assert np.array_equal(bits(s.cpu().numpy()), bits(ws)) and np.array_equal(bits(z.cpu().numpy()), bits(wz))
+    assert (wq[:200] >> 4).max() == 15 and (wq[:200] & 15).min() == 0
+
+
 def test_kv_vectors_with_infinities_take_the_ieee_path():
     """An infinite element makes range and scale infinite: every finite element then gets code 0 and
     inf / inf (NaN) converts to 0, as round/clamp/cast give in the reference; neighbouring finite
