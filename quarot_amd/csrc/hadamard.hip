@@ -1146,23 +1146,20 @@ __global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard
     for (int i = 0; i < TPW; ++i)
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) yp[i][ct] = u32x2{0, 0};
-    // One register pair of the previous row in three parts of two or three vector instructions (the
-    // arithmetic of sym_codes8_fast): each part goes behind one matrix instruction, whose 16 cycles leave
-    // room for about three vector instructions of the same wave.
+    // One register pair of the previous row in three parts of two vector instructions (the arithmetic
+    // of sym_codes8_fast): each part goes behind one matrix instruction, whose 16 cycles leave room for
+    // about three vector instructions of the same wave.
     float qa0 = 0.f, qa1 = 0.f;
     auto quant_part = [&](int p, int part) {
         const int i = p / (2 * CT), ct = (p / 2) % CT, w = p & 1;
         if (part == 0) {
             const f16x2 h2 = as_f16x2(yp[i][ct][w]);
-            qa0 = __builtin_fmaf((float)h2[0], fqp.rh, 0.0f);
-            qa1 = __builtin_fmaf((float)h2[1], fqp.rh, 0.0f);
+            qa0 = __builtin_fmaf((float)h2[0], fqp.r, 0.0f);
+            qa1 = __builtin_fmaf((float)h2[1], fqp.r, 0.0f);
         } else if (part == 1) {
-            const f16x2 h2 = as_f16x2(yp[i][ct][w]);
-            qa0 = __builtin_fmaf((float)h2[0], fqp.rl, qa0);
-            qa1 = __builtin_fmaf((float)h2[1], fqp.rl, qa1);
             qa0 = __builtin_amdgcn_fmed3f(qa0, -8.0f, 7.0f);
-        } else {
             qa1 = __builtin_amdgcn_fmed3f(qa1, -8.0f, 7.0f);
+        } else {
             f16x2 h = {(f16)qa0, (f16)qa1};
             h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
             pb[i][ct][w] = __builtin_bit_cast(u32, h);
@@ -1319,7 +1316,7 @@ __global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard
         sp = (float)sh;
         mxp = mx;
         prow = row;
-        fqp = fast_quant_ok(mx, sp) ? make_fast_recip(sp) : FastRecip{0.f, 0.f};
+        fqp = fast_quant_ok(mx, sp) ? make_fast_recip(sp) : FastRecip{0.f};
 #pragma unroll
         for (int i = 0; i < TPW; ++i)
 #pragma unroll

@@ -50,8 +50,8 @@ __device__ __forceinline__ f16x2 kv_pair_min(f16x2 p) {
 }
 
 // Eight codes clamp(round_half_even(fp16(fp16(x + zero) / scale)), 0, 15) for all-finite input: the
-// add is one packed fp16 add, the division the exact-product / fma form of sym_codes8_fast (the
-// shifted value has at most 11 significant bits), the rounding the +1536 trick.
+// add is one packed fp16 add, the division the one-multiplication form of sym_codes8_fast (the
+// shifted value is an fp16 number like any other), the rounding the +1536 trick.
 // CLAMP = false leaves the clamp out: the shifted values lie in [0, range] by construction, so with a
 // scale that is a NORMAL fp16 number (relative rounding error <= 2^-11: range >= 2^-10 is enough) the
 // quotient is at most 15 (1 + 2^-11) and rounds to 15 at most.  A subnormal scale can be off by several
@@ -64,8 +64,8 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
     for (int i = 0; i < 4; ++i) {
         const f16x2 sh = as_f16x2(v[i]) + z2;
         const float x0 = (float)sh[0], x1 = (float)sh[1];
-        float q0 = __builtin_fmaf(x0, f.rl, __builtin_fmaf(x0, f.rh, 0.0f));
-        float q1 = __builtin_fmaf(x1, f.rl, __builtin_fmaf(x1, f.rh, 0.0f));
+        float q0 = __builtin_fmaf(x0, f.r, 0.0f);
+        float q1 = __builtin_fmaf(x1, f.r, 0.0f);
         if (CLAMP) {
             q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
             q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);

@@ -225,25 +225,30 @@ __device__ __forceinline__ u32 sym_codes8(u32x4 v, float s, float rs, bool fast_
 }
 
 // ---- lean quantiser for rows known to be all-finite with a finite non-zero scale ------------------
-// 1/s is held as rh + rl with rh cut to 13 significant bits, so x * rh is EXACT in fp32 (x has 11)
-// and q = fma(x, rl, x * rh) is the correctly rounded fp32 quotient x / s up to a 2^-36 relative
-// perturbation: far inside the 2^-23 margin that separates a quotient of two fp16 numbers from an
-// fp16 rounding boundary (see sym_code), so (f16)q is the correctly rounded fp16 division.
-// Clamping to [-8, 7] before that conversion commutes with it (rounding is monotone and -8, 7 are
+// q = x * r with r the CORRECTLY ROUNDED fp32 reciprocal of the scale: one multiplication per value.
+// That (f16)q is the correctly rounded fp16 division wherever a code depends on it (quotients in
+// [0.25, 32): below, every candidate rounds to code 0; above, the clamp decides) was checked by brute
+// force over every pair of a finite fp16 value and a positive finite fp16 scale (31744 x 31743 pairs:
+// no difference; with r one ulp off in either direction a few thousand pairs differ, so the
+// reciprocal must be the correctly rounded one).  Why it works: a quotient of two fp16 numbers keeps
+// a relative distance above 2^-23 from every fp16 rounding boundary (see sym_code), and the two
+// roundings here (r, then the product) stay within 2^-23.
+// Clamping to [-8, 7] before the conversion commutes with it (rounding is monotone and -8, 7 are
 // representable).  Adding 1536 (ulp 1 in [1024, 2048)) in fp16 then rounds to the nearest integer,
 // ties to even, and leaves the two's-complement code in the low four mantissa bits.
 struct FastRecip {
-    float rh, rl;
+    float r;
 };
-// s: a finite non-zero fp16 value as float.  v_rcp_f32 + one Newton step give r1 ~ 1/s; rh = r1
-// cut to 13 bits makes s * rh exact (11 + 13 bits), so e2 = 1 - s rh is exact and rl = e2 r1
-// completes 1/s to a relative 2^-35.
+// s: a finite non-zero fp16 value as float.  v_rcp_f32 is good to one ulp; a Newton step in fma form
+// brings r1 within 2^-24 (1 + 2^-22) of 1 / s; in the second step e = 1 - s r1 is EXACT (s has 11
+// significant bits, the product 35, and all but 12 cancel), so fma(e, r1, r1) rounds
+// (1 / s) (1 - e^2) once: the correctly rounded reciprocal, because 1 / s for an 11-bit s keeps a
+// relative distance of at least 2^-36 from every fp32 rounding boundary and e^2 < 2^-46.
 __device__ __forceinline__ FastRecip make_fast_recip(float s) {
     const float r0 = __builtin_amdgcn_rcpf(s);
     const float r1 = __builtin_fmaf(__builtin_fmaf(-s, r0, 1.0f), r0, r0);
     FastRecip f;
-    f.rh = __builtin_bit_cast(float, __builtin_bit_cast(u32, r1) & 0xFFFFF800u);
-    f.rl = __builtin_fmaf(-s, f.rh, 1.0f) * r1;
+    f.r = __builtin_fmaf(__builtin_fmaf(-s, r1, 1.0f), r1, r1);
     return f;
 }
 // w[i] holds two fp16 values 1536 + code (codes in the low four bits of each half, element 2 i in
@@ -263,11 +268,10 @@ __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
     for (int i = 0; i < 4; ++i) {
         const float x0 = (float)f16_from_bits((unsigned short)(v[i] & 0xffffu));
         const float x1 = (float)f16_from_bits((unsigned short)(v[i] >> 16));
-        // x * rh written as fma(x, rh, 0): the same value (the product is exact; a zero of either sign
-        // ends as code 0), and it lets both steps take the half straight from the packed word
-        // (v_fma_mix_f32) instead of converting it first
-        float q0 = __builtin_fmaf(x0, f.rl, __builtin_fmaf(x0, f.rh, 0.0f));
-        float q1 = __builtin_fmaf(x1, f.rl, __builtin_fmaf(x1, f.rh, 0.0f));
+        // x * r written as fma(x, r, 0): the same value (a zero of either sign ends as code 0), and the
+        // instruction takes the half straight from the packed word (v_fma_mix_f32) instead of converting first
+        float q0 = __builtin_fmaf(x0, f.r, 0.0f);
+        float q1 = __builtin_fmaf(x1, f.r, 0.0f);
         q0 = __builtin_amdgcn_fmed3f(q0, -8.0f, 7.0f);
         q1 = __builtin_amdgcn_fmed3f(q1, -8.0f, 7.0f);
         f16x2 h = {(f16)q0, (f16)q1};

@@ -113,6 +113,27 @@ def test_sym_quant_every_fp16_value_times_many_scales():
     assert not got[~finite_scale].any()
 
 
+def test_sym_quant_every_fp16_value_against_every_positive_scale():
+    """The lean quantiser forms x / s as ONE fp32 multiplication by the correctly rounded reciprocal of s: every
+    finite fp16 value against every positive finite fp16 scale (2 x 31744 x 31743 pairs), judged on the GPU
+    against the IEEE sequence the reference's kernel runs (fp32 division, rounding to fp16, round half even,
+    clamp), and every 257th scale's rows against the oracle on the CPU as well."""
+    pos = torch.from_numpy(np.arange(0, 0x7c00, dtype=np.uint16).view(F16).copy()).cuda()
+    scales = pos[1:]
+    for sign in (1.0, -1.0):
+        vals = (pos * sign).contiguous()
+        for c0 in range(0, scales.numel(), 2048):
+            s = scales[c0:c0 + 2048].contiguous()
+            x = vals.unsqueeze(0).expand(s.numel(), -1).contiguous()
+            q = quarot_amd.sym_quant(x, s)
+            want = torch.clamp(torch.round((x.float() / s.float().unsqueeze(1)).half().float()), -8, 7).to(torch.int8)
+            got = torch.stack([(q & 15).to(torch.int8), (q >> 4).to(torch.int8)], dim=-1).reshape(s.numel(), -1)
+            got = torch.where(got > 7, got - 16, got)
+            assert torch.equal(got, want), (sign, c0)
+            rows = list(range(c0 % 257, s.numel(), 257))
+            assert np.array_equal(q[rows].cpu().numpy(), o.pack_i4(o.sym_quant_codes(x[rows].cpu().numpy(), s[rows].cpu().numpy())))
+
+
 def test_sym_quant_odd_columns_and_views():
     x = synth_x(11, 75, seed=3)
     s = o.quantizer_scales(x)
