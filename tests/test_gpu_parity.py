@@ -575,6 +575,47 @@ def test_fused_hadamard_quantize_equals_staged(n, fp32):
     assert close(y2.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
 
 
+def test_fused_fronts_random_shapes_scales_and_clips():
+    """Seeded random sweep over the fused Hadamard+quantise kernels: widths of every kernel family, 1 .. 1500 rows,
+    data from 1e-5 to 300 with outlier columns, clip ratios 1.0 / 0.95 / 0.9, both precisions, a zero row, rows
+    with an infinity, a NaN or saturating values.  The call without the transformed copy (the lean kernels), the
+    call with it and the standalone quantiser on that copy must agree bit for bit, and on every finite non-zero
+    row the codes and scales must be those of the IEEE sequence the reference runs (amax / 7, * clip, fp32
+    division, rounding to fp16, round half even, clamp), evaluated by torch on the GPU."""
+    rng = np.random.default_rng(11)
+    sizes = [64, 128, 1024, 4096, 8192, 224, 3840, 6912, 8960, 11008, 28672, 13824, 5120, 6656, 4608, 7680, 17920, 22016]
+
+    def unpack(p):
+        v = torch.stack([(p & 15).to(torch.int8), (p >> 4).to(torch.int8)], dim=-1).reshape(p.shape[0], -1)
+        return torch.where(v > 7, v - 16, v)
+
+    for case in range(48):
+        n = int(sizes[case % len(sizes)])
+        rows = int(rng.choice([rng.integers(1, 40), rng.integers(40, 1500)]))
+        clip = float(rng.choice([1.0, 1.0, 0.9, 0.95]))
+        fp32 = bool(rng.random() < 0.3)
+        x = torch.randn(rows, n, device="cuda") * float(rng.choice([1e-5, 1e-3, 1.0, 30.0, 300.0]))
+        x[:, ::int(rng.integers(50, 200))] *= 20
+        x = x.half()
+        if rows > 3:
+            x[1] = 0
+            x[2, int(rng.integers(0, n))] = float("inf")
+            x[3, int(rng.integers(0, n))] = float("nan")
+            x[0] = 60000.0
+        fused = quarot_amd.nn.OnlineHadamardQuantizer(n, force_fp32=fp32, input_clip_ratio=clip).cuda()
+        p2, y2 = quarot_amd.hadamard_quantize(x, fused.had_rem_dim, fused.rem_dim, clip, force_fp32=fp32, return_transformed=True)
+        p = fused(x)
+        tag = (n, rows, clip, fp32)
+        assert torch.equal(p.quantized_x, p2.quantized_x) and torch.equal(p.scales_x.view(torch.int16), p2.scales_x.view(torch.int16)), tag
+        st = quarot_amd.nn.Quantizer(clip)(y2)
+        assert torch.equal(st.quantized_x, p2.quantized_x) and torch.equal(st.scales_x.view(torch.int16), p2.scales_x.view(torch.int16)), tag
+        ok = torch.isfinite(y2).all(dim=1) & (y2.abs().amax(dim=1) > 0)
+        scale = ((y2.abs().amax(dim=1, keepdim=True).float() / 7).half().float() * clip).half()
+        want = torch.clamp(torch.round((y2.float() / scale.float()).half().float()), -8, 7).to(torch.int8)
+        assert torch.equal(unpack(p2.quantized_x)[ok], want[ok]), tag
+        assert torch.equal(p2.scales_x.reshape(-1)[ok].view(torch.int16), scale.reshape(-1)[ok].view(torch.int16)), tag
+
+
 @pytest.mark.parametrize("n", [11008, 8960, 6912, 13824, 5120, 4608, 17920])
 def test_fused_hadamard_quantize_lean_kernel_rows_of_every_kind(n):
     """Without the copy of the transformed rows the m = 64 widths (and m = 128 behind a table of order 36 .. 60 or
