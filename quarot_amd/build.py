@@ -34,27 +34,5 @@ def build(verbose=True):
     return LIB
 
 
-def build_ubench(out_dir=None, verbose=True):
-    """Compile the stand-alone microbenchmarks under csrc/ubench (not part of the library) into
-    `out_dir` (default: a temporary directory, i.e. a does-it-still-compile check)."""
-    import tempfile
-    made = []
-    with tempfile.TemporaryDirectory() as tmp:
-        dst = pathlib.Path(out_dir) if out_dir else pathlib.Path(tmp)
-        dst.mkdir(parents=True, exist_ok=True)
-        for src in sorted((CSRC / "ubench").glob("*.hip")):
-            cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                   "-Wno-unused-command-line-argument", str(src), "-o", str(dst / src.stem)]
-            if verbose:
-                print(" ".join(cmd), flush=True)
-            res = subprocess.run(cmd, capture_output=True, text=True)
-            if res.returncode != 0:
-                raise RuntimeError(f"hipcc failed ({res.returncode}) on {src.name}:\n{res.stderr}")
-            made.append(dst / src.stem)
-    return made
-
-
 if __name__ == "__main__":
     build()
-    if "--ubench" in sys.argv:
-        build_ubench(PKG.parent / "gpurun_out" / "ubench" if "--keep" in sys.argv else None)
