@@ -13,6 +13,7 @@ outlier channels that motivate the Hadamard):
     c1o o_proj 7B      attention output [2048, 32, 128] -> Hadamard across the 32 heads -> Quantizer
         (one fused kernel) -> W int4 [4096, 4096]
     c2  down_proj 7B   X [2048, 11008]  W int4 [4096, 11008]    Hadamard FWHT(64) (x) had_172   (default)
+    c2_fp32had  the same with OnlineHadamard(force_fp32=True): the reference benchmark's "+FP32had" column
     c3  the four linears of a 7B decoder layer at 32768 tokens as ONE step: fused qkv 4096->12288, o 4096->4096,
         gate_up 4096->22016 (Quantizer in front of each) and down 11008->4096 (Hadamard+Quantizer): 13.26 TOP
         (c3a, c3b, c3c, c3d: each of them on its own)
@@ -59,6 +60,7 @@ WORKLOADS = {
     "c1n": (2048, 4096, 4096, "rmsnorm"),     # input_layernorm -> Quantizer -> q_proj
     "c1o": (2048, 4096, 4096, "heads"),       # attention output -> Hadamard over heads -> Quantizer -> o_proj
     "c2": (2048, 11008, 4096, "had"),
+    "c2_fp32had": (2048, 11008, 4096, "had32"),   # the "+FP32had" chain of benchmarks/qlinear_benchmark.py:68-73 (force_fp32=True)
     "c3a": (32768, 4096, 12288, "quant"),     # fused qkv
     "c3b": (32768, 4096, 4096, "quant"),      # o_proj
     "c3c": (32768, 4096, 22016, "quant"),     # gate_up
@@ -75,7 +77,7 @@ WORKLOADS = {
 for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
-PER_CONFIG = ["c1", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
+PER_CONFIG = ["c1", "c2_fp32had", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
               "c2_fp6", "c3_fp6", "b13v_fp6", "b70v_fp6", "b13d_fp6", "b70d_fp6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 FP6_MFMA_PEAK_TOPS = 10100.0     # MI355X dense fp6, published (the opt-in exact int4 GEMM on 6-bit operands)
@@ -186,6 +188,75 @@ def kernel_ms(fn, reps):
     return e0.elapsed_time(e1) / reps
 
 
+def mfma_i8_rate(pattern, launches=10, iters=4096, workgroups=1024):
+    """TOP/s of the library's register-only loop of v_mfma_i32_32x32x32_i8 (qr_calib_mfma_i8: four waves per
+    workgroup, four accumulator chains per wave, no memory access): what the matrix pipe sustains with nothing
+    else going on.  pattern 0: zero operands, 1: random int4 codes as the GEMMs feed them, 2: random int8, 3: random int4 codes as
+    sign-extended int8."""
+    from quarot_amd import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    out = torch.empty(workgroups * 256, dtype=torch.int32, device=dev)
+    st = _lib.stream_ptr(dev)
+    ops = workgroups * 4 * iters * 16 * 65536.0
+    return ops / (kernel_ms(lambda: _lib.check(L.qr_calib_mfma_i8(pattern, iters, workgroups, out.data_ptr(), st)), launches) * 1e-3) / 1e12
+
+
+def gpu_clock_mhz():
+    """Current shader clock from rocm-smi (None when the tool is missing or prints something else)."""
+    import subprocess
+    try:
+        txt = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r"sclk clock level:?\s*\d*:?\s*\((\d+)Mhz\)", txt, flags=re.I)
+    return int(m.group(1)) if m else None
+
+
+def mfma_ceiling(seconds):
+    """The int8 matrix instruction alone (no loads, no LDS, no unpacking): short bursts, then `seconds` of back-to-back
+    launches per operand pattern with the shader clock sampled from rocm-smi while they run."""
+    import threading
+    from quarot_amd import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    res = {"instruction": "v_mfma_i32_32x32x32_i8", "published_peak_TOPS": INT8_MFMA_PEAK_TOPS, "patterns": {}}
+    wg, iters = 1024, 8192
+    out = torch.empty(wg * 256, dtype=torch.int32, device=dev)
+    st = _lib.stream_ptr(dev)
+    ops = wg * 4 * iters * 16 * 65536.0
+    for pattern, label in ((0, "zero operands"), (1, "random int4 codes x16 (what the GEMMs feed)"), (2, "random int8 bytes"),
+                           (3, "random int4 codes sign-extended to int8")):
+        burst = mfma_i8_rate(pattern, launches=5, iters=iters, workgroups=wg)
+        clocks, stop = [], threading.Event()
+
+        def sample():
+            while not stop.is_set():
+                c = gpu_clock_mhz()
+                if c:
+                    clocks.append(c)
+                time.sleep(0.25)
+
+        th = threading.Thread(target=sample)
+        torch.cuda.synchronize()
+        th.start()
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(20):
+                _lib.check(L.qr_calib_mfma_i8(pattern, iters, wg, out.data_ptr(), st))
+            torch.cuda.synchronize()
+            n += 20
+        t = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        tail = clocks[len(clocks) // 2:]
+        res["patterns"][label] = {"burst_TOPS": round(burst, 1), "sustained_TOPS": round(n * ops / t / 1e12, 1),
+                                  "sustained_seconds": round(t, 2), "frac_of_published_peak": round(n * ops / t / 1e12 / INT8_MFMA_PEAK_TOPS, 4),
+                                  "sclk_mhz_second_half": [min(tail), max(tail)] if tail else None, "sclk_samples": len(clocks)}
+    return res
+
+
 def gemm_kernel_name(m, n):
     t256 = ((m + 255) // 256) * ((n + 255) // 256)
     t128 = ((m + 127) // 128) * ((n + 255) // 256)
@@ -202,7 +273,8 @@ def gemm_kernel_name(m, n):
     return "gemm_ks_kernel<64,256>"
 
 
-FRONT_KERNEL = {"had": "hadamard kernel + quantiser (fused)", "quant": "quant_rows_kernel",
+FRONT_KERNEL = {"had": "hadamard kernel + quantiser (fused)", "had32": "hadamard kernel in fp32 precision + quantiser (fused)",
+                "quant": "quant_rows_kernel",
                 "rmsnorm": "rmsnorm_quant_rows_kernel", "heads": "heads_hadamard_quant_rows_kernel"}
 
 
@@ -232,7 +304,8 @@ class LinearWorkload:
         if self.heads:
             self.x = self.x.view(m, self.heads, k // self.heads)   # as attention writes it: [tokens, heads, head_dim]
         nn_ = quarot_amd.nn
-        self.front = {"had": lambda: nn_.OnlineHadamardQuantizer(k), "rmsnorm": lambda: nn_.RMSNormQuantizer(k),
+        self.front = {"had": lambda: nn_.OnlineHadamardQuantizer(k), "had32": lambda: nn_.OnlineHadamardQuantizer(k, force_fp32=True),
+                      "rmsnorm": lambda: nn_.RMSNormQuantizer(k),
                       "heads": lambda: nn_.HeadsHadamardQuantizer(self.heads), "quant": lambda: nn_.Quantizer()}[self.front_kind]().to(dev)
         # decode: identical weight copies used round-robin, more bytes in total than the last-level cache
         self.copies = [self.lin.weight]
@@ -242,13 +315,14 @@ class LinearWorkload:
         self.i = 0
         # front kernel and GEMM go out in ONE call into the library (decode steps, and the shorter prefill
         # steps, are otherwise bound by the host's per-call cost)
-        self.one_call = self.front_kind in ("had", "quant") and not fp6
+        self.one_call = self.front_kind in ("had", "had32", "quant") and not fp6
         if fp6:
             # the opt-in FP6 matrix path: the step converts the activations' codes and runs the GEMM on 6-bit
             # operands (the weights' 6-bit copy is made once, at the first call)
             assert not self.decode and k % 64 == 0
             self.lin.prefill_fp6, self.lin.fp6_min_rows = True, 0
-        self.had_args = (self.front.had_rem_dim, self.front.rem_dim) if self.front_kind == "had" else (None, 0)
+        self.had_args = (self.front.had_rem_dim, self.front.rem_dim) if self.front_kind in ("had", "had32") else (None, 0)
+        self.fp32_had = self.front_kind == "had32"
         self.ops = 2.0 * m * n * k
 
     def weight(self):
@@ -260,7 +334,8 @@ class LinearWorkload:
         if self.fp6:
             return self.lin(self.front(self.x))
         if self.one_call:
-            return self.q.quantized_linear(self.x, self.weight(), self.lin.weight_scales, self.lin.bias, *self.had_args)
+            return self.q.quantized_linear(self.x, self.weight(), self.lin.weight_scales, self.lin.bias, *self.had_args,
+                                           force_fp32=self.fp32_had)
         p = self.front(self.x)
         return self.q.linear_i4(p.quantized_x, p.scales_x, self.weight(), self.lin.weight_scales, self.lin.bias)
 
@@ -274,8 +349,8 @@ class LinearWorkload:
         nn_ = self.q.nn
         if not hasattr(self, "_staged"):
             dev = self.x.device
-            if self.front_kind == "had":
-                self._staged = torch.nn.Sequential(nn_.OnlineHadamard(self.k), nn_.Quantizer()).to(dev)
+            if self.front_kind in ("had", "had32"):
+                self._staged = torch.nn.Sequential(nn_.OnlineHadamard(self.k, force_fp32=self.fp32_had), nn_.Quantizer()).to(dev)
             elif self.front_kind == "rmsnorm":
                 self._staged = torch.nn.Sequential(nn_.RMSNorm(self.k), nn_.Quantizer()).to(dev)
             elif self.front_kind == "heads":
@@ -284,6 +359,13 @@ class LinearWorkload:
             else:
                 self._staged = nn_.Quantizer()
         return self.lin(self._staged(self.x))
+
+    def fp16_linear_ms(self, steps):
+        """Context only, never a target: torch's fp16 linear layer on the same shape (the reference's benchmark
+        prints its int4 chains beside it, benchmarks/qlinear_benchmark.py:60-66,102-106); random weights."""
+        w = torch.randn(self.n, self.k, device=self.x.device, dtype=torch.float16) * 0.02
+        x = self.x.reshape(self.m, self.k)
+        return float(np.median(timed_loops(lambda: torch.nn.functional.linear(x, w), steps, 3, 3)))
 
     def kernel_times(self, reps):
         """(front kernel ms, GEMM kernel ms), each from a pass of its own (decode: the weights still
@@ -319,7 +401,7 @@ class LinearWorkload:
         return g, f
 
     def describe(self):
-        tail = {"had": " with online Hadamard", "rmsnorm": " behind RMSNorm", "heads": f" behind the Hadamard across {self.heads} heads",
+        tail = {"had": " with online Hadamard", "had32": " with online Hadamard in fp32 (force_fp32=True)", "rmsnorm": " behind RMSNorm", "heads": f" behind the Hadamard across {self.heads} heads",
                 "quant": ""}[self.front_kind]
         data = "1% outlier channels x20" if not self.decode else "N(0,1)"
         return f"{self.name}: Linear4bit X[{self.m},{self.k}] fp16 ({data}) . W int4[{self.n},{self.k}]" + tail
@@ -353,6 +435,11 @@ def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, grap
     front_ms, gemm_ms = wl.kernel_times(kernel_reps)
     groof, froof = wl.rooflines(front_ms, gemm_ms)
     staged = timed_loops(wl.staged_step, max(5, steps // 4), 3, min(repeats, 3))
+    if not wl.decode:
+        extra["fp16_linear_ms"] = round(wl.fp16_linear_ms(max(5, steps // 10)), 5)
+    # the whole step against the same roofline as its dominant kernel (algorithmic bytes of the GEMM for decode)
+    extra["step_frac"] = round((wl.gemm_bytes() / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS) if wl.decode
+                               else wl.ops / (ms * 1e-3) / 1e12 / (FP6_MFMA_PEAK_TOPS if wl.fp6 else INT8_MFMA_PEAK_TOPS), 4)
     res = {"ms": ms, "value": round(wl.ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": groof,
            "front": froof, "kernels_ms_sum": round(front_ms + gemm_ms + (wl.convert_ms if wl.fp6 else 0.0), 5),
            "staged_reference_api_ms": round(float(np.median(staged)), 5), "workload": wl.describe(), **extra}
@@ -416,6 +503,7 @@ def run_layer(dev, steps, warmup, repeats, kernel_reps, fp6=False):
     roof["kernel_ms"] = round(gemm_total, 4)
     return {"ms": ms, "value": round(ops / (ms * 1e-3) / 1e12, 2), "unit": "TOPS", "timing": sp, "roofline": roof,
             "per_linear": per, "kernels_ms_sum": round(gemm_total + front_total, 4), "total_TOP": round(ops / 1e12, 2),
+            "step_frac": round(ops / (ms * 1e-3) / 1e12 / peak, 4),
             "workload": "c3: Llama-2-7B decoder-layer linear set at M=32768 (qkv 4096->12288, o 4096->4096, gate_up 4096->22016, "
                         "down 11008->4096 with online Hadamard), W4A4, one step = " + ("12 launches (fronts, conversions to 6-bit operands, GEMMs)" if fp6 else "8 launches")}
 
@@ -459,6 +547,7 @@ def run_kv(dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
     roof["kernel"] = "kv_had128_kernel (K cache: Hadamard on the matrix cores + asymmetric int4)"
     roof["kernel_ms"] = round(k_ms, 5)
     res = {"ms": ms, "value": round(4 * bytes_one / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "timing": sp, "roofline": roof,
+           "step_frac": round(4 * bytes_one / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
            "kernels": {n: {"ms": round(t, 5), "GBs": round(bytes_one / (t * 1e-3) / 1e9, 1), "frac": round(bytes_one / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
                        for n, t in times.items()},
            "workload": "c5: K and V [32,4096,8,128] fp16 (0.5% elements x15) -> asym int4 + fp16 scale/zero per head vector "
@@ -513,6 +602,7 @@ def run_attention(name, dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
     roof["kernel"] = "paged_decode_i4_kernel (single-query attention, in-register dequantisation)"
     roof["kernel_ms"] = round(a_ms, 5)
     res = {"ms": ms, "value": round(cache_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "timing": sp, "roofline": roof,
+           "step_frac": round(cache_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
            "workload": f"{name}: decode step on the paged int4 KV cache, {B} sequences x {S} tokens x {H} heads x 128, pages of {P}: "
                        "quantise-and-append of one token per sequence, query Hadamard, attention over the cache"}
     if cpu_baseline:
@@ -537,7 +627,7 @@ def cpu_baseline(wl, budget_rows):
     rows = min(wl.m, budget_rows)
     wc = cb.unpacked_codes(wl.w_cpu.numpy())
     ws = wl.sw_cpu.view(-1)
-    hadamard, rmsnorm, heads = wl.front_kind == "had", wl.front_kind == "rmsnorm", wl.heads
+    hadamard, rmsnorm, heads = wl.front_kind in ("had", "had32"), wl.front_kind == "rmsnorm", wl.heads
     torch.set_num_threads(os.cpu_count() or 1)
     cb.linear4bit_path(wl.x_cpu[:2].clone(), wc[:64], ws[:64], hadamard, rmsnorm, heads)   # warm-up
     # size the sample for about 4 s per pass (three passes: 10-15 s of CPU work), starting from `budget_rows`
@@ -562,7 +652,8 @@ def cpu_baseline(wl, budget_rows):
 
 def brief(res):
     """The per-config view of a result: step time, value and the dominant kernel's roofline."""
-    keep = ("ms", "value", "unit", "roofline", "front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms", "launch")
+    keep = ("ms", "value", "unit", "roofline", "front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms", "launch",
+            "fp16_linear_ms", "step_frac")
     out = {k: res[k] for k in keep if k in res}
     out["ci95_ms"] = res["timing"]["ci95_ms"]
     return out
@@ -586,6 +677,9 @@ def main():
                          "the step then includes the conversion of the activations' codes to 6-bit operands")
     ap.add_argument("--cpu-rows", type=int, default=64,
                     help="rows of the first CPU-baseline pass; the timed sample is then sized for about 4 s per pass")
+    ap.add_argument("--mfma-ceiling", type=float, default=0.0, metavar="SECONDS",
+                    help="instead of a workload, run the register-only loop of the int8 matrix instruction (qr_calib_mfma_i8) for "
+                         "SECONDS per operand pattern, with the shader clock sampled from rocm-smi beside it")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of a workload, run a plain 256 MiB device copy 20 times (known traffic: 256 MiB read, "
                          "256 MiB written per launch) for scaling the profiler's FETCH_SIZE / WRITE_SIZE counters")
@@ -604,6 +698,9 @@ def main():
         build.build(verbose=False)
     _lib.lib()
     dev = torch.device("cuda:0")
+    if args.mfma_ceiling > 0:
+        print(json.dumps({"mfma_i8_ceiling": mfma_ceiling(args.mfma_ceiling)}))
+        return
     if args.copy_calibration:
         src = torch.randint(0, 255, (256 * 1024 * 1024,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -643,6 +740,12 @@ def main():
         traffic *= 4                                       # the step is four launches; the summary holds their average
     roof["traffic"] = traffic
     roof["traffic_source"] = source
+    if roof.get("bound") == "mfma" and not args.fp6:
+        # what the int8 matrix instruction alone sustains on this box right now (register-only loop, operands with the
+        # GEMM's bit statistics, ~60 ms of launches): the part's own ceiling for ANY int8 kernel; `frac` stays against `peak`
+        roof["attainable"] = round(mfma_i8_rate(1, launches=12), 1)
+        roof["attainable_zero_operands"] = round(mfma_i8_rate(0, launches=12), 1)
+        roof["frac_of_attainable"] = round(roof["achieved"] / roof["attainable"], 4)
     kv_line = args.workload in ("c5", "c6", "c6b")
     out = {
         "metric": ("KV-cache int4 quantise + dequantise GB/s (K with Hadamard, V)" if args.workload == "c5"
@@ -660,7 +763,7 @@ def main():
                              "separate pass of back-to-back launches of that kernel alone between two HIP events on the launch stream"},
         "roofline": roof,
     }
-    for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms"):
+    for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms", "fp16_linear_ms", "step_frac"):
         if key in res:
             out[key] = res[key]
     if wl is not None:
@@ -680,6 +783,10 @@ def main():
             if t is not None:
                 per[name]["roofline"]["traffic"], per[name]["roofline"]["traffic_source"] = (4 * t if name in ("c3", "c3_fp6") else t), s
         out["per_config"] = per
+        # the same table in a few numbers per workload: [step ms, dominant kernel ms, its roofline fraction, the step's]
+        out["roofline"]["per_config"] = {name: [r["ms"], r["roofline"]["kernel_ms"], r["roofline"]["frac"], r.get("step_frac")]
+                                         for name, r in per.items()}
+        out["roofline"]["per_config_front"] = {name: [r["front"]["kernel_ms"], r["front"]["frac"]] for name, r in per.items() if "front" in r}
         out["per_config_note"] = ("same step definition as the headline; operands generated on the GPU, a fifth of the steps per loop "
                                   "(c3, c5: fewer still) and half the repeats")
     print(json.dumps(out))

@@ -185,7 +185,9 @@ int qr_linear_i4_f16_ws(const void* A, const void* sA, const void* W, const void
  *   no scratch run the single-launch kernels.
  *   All calls on one GPU share that GPU's buffer: calls that overlap in time on one GPU (different
  *   streams or host threads) race.  The first call on a device looks the buffer's address up
- *   (hipGetSymbolAddress); make that call outside graph capture.
+ *   (hipGetSymbolAddress); make that call outside graph capture.  The buffer is the CURRENT device's
+ *   (hipGetDevice at the time of the call): `stream` must belong to the current device.  A failure
+ *   of that look-up comes back as the positive hipError_t, like a launch error.
  */
 #define QR_STATIC_SCRATCH_BYTES (32u << 20)
 int qr_linear_i4_f16_static(const void* A, const void* sA, const void* W, const void* sW,
@@ -326,6 +328,22 @@ int qr_batch_decode_qhad_i4(void* o, const void* q, const void* kv_data, const v
                             int64_t num_pages, int num_layers, int layer_idx, int num_heads, int page_size,
                             int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
                             size_t workspace_bytes, void* stream);
+
+/*
+ * Measurement aids.  NO counterpart in the reference and no caller in the product path: kernels whose
+ * work is known exactly, run by bench.py next to the workloads to calibrate the rooflines.
+ *
+ * qr_calib_mfma_i8: `workgroups` workgroups of four waves, each wave `iters` turns of 16
+ *   v_mfma_i32_32x32x32_i8 (four independent accumulator chains, operands and accumulators in
+ *   registers, no memory access): workgroups * 4 * iters * 16 * 65536 integer operations per launch.
+ *   pattern 0: all-zero operands; 1: random int4 codes as the int4 GEMMs feed them (16 * code in every
+ *   byte); 2: random int8 bytes; 3: random int4 codes as sign-extended int8.  `out` (device, >= workgroups * 1024 bytes) is never written (it only
+ *   keeps the loop observable).
+ * qr_calib_copy: dst[0 .. bytes) = src[0 .. bytes) with 16-byte nontemporal loads and stores (bytes a
+ *   multiple of 16, pointers 16-byte aligned): `bytes` read and `bytes` written per launch.
+ */
+int qr_calib_mfma_i8(int pattern, int iters, int workgroups, void* out, void* stream);
+int qr_calib_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

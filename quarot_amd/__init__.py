@@ -219,7 +219,9 @@ def heads_hadamard_quantize(x, num_heads, clip_ratio=1.0, return_transformed=Fal
 
 
 @functools.lru_cache(maxsize=4096)
-def _workspace_bytes(M, N, K):
+def _workspace_bytes(M, N, K, device_index=None):
+    # (the library's split plan depends on the CURRENT device's compute-unit count: callers make the
+    # device current first, and the device index is part of the cache key)
     return _lib.lib().qr_workspace_bytes(M, N, K)
 
 
@@ -239,7 +241,7 @@ def linear_i4(x_q, scales_x, weight, weight_scales, bias=None):
     y = torch.empty((M, N), dtype=torch.float16, device=dev)
     L = _lib.lib()
     with _lib.on_device(dev):
-        ws_bytes = _workspace_bytes(M, N, K)
+        ws_bytes = _workspace_bytes(M, N, K, dev.index)
         if ws_bytes:
             # few output tiles: the library splits K across workgroups and needs int32 scratch for the sums
             ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
@@ -287,8 +289,8 @@ def linear_f6(x6, scales_x, weight6, weight_scales, bias=None):
 
 
 @functools.lru_cache(maxsize=4096)
-def _quantized_linear_workspace_bytes(M, N, K):
-    return _lib.lib().qr_quantized_linear_workspace_bytes(M, N, K)
+def _quantized_linear_workspace_bytes(M, N, K, device_index=None):
+    return _lib.lib().qr_quantized_linear_workspace_bytes(M, N, K)       # (per device, like _workspace_bytes)
 
 
 def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_ratio=1.0, force_fp32=False):
@@ -311,10 +313,10 @@ def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_r
     if hadK is not None and hadK.dtype != want:
         hadK = hadK.to(want)
     y = torch.empty((M, N), dtype=torch.float16, device=dev)
-    ws_bytes = _quantized_linear_workspace_bytes(M, N, n)
-    ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
     mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
     with _lib.on_device(dev):
+        ws_bytes = _quantized_linear_workspace_bytes(M, N, n, dev.index)
+        ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
         _lib.check(_lib.lib().qr_quantized_linear_f16(_ptr(x2), M, n, int(K), _ptr(hadK), mode,
                                                       functional.hadamard.had_scale(n), float(clip_ratio), _ptr(weight),
                                                       _ptr(sw), _ptr(bias), N, _ptr(y), _ptr(ws), ws_bytes,

@@ -1,7 +1,10 @@
 """Build recipe for libquarot_hip.so: plain hipcc, gfx950 only, no torch headers.
 
-    python -m quarot_amd.build          # compile in-tree (quarot_amd/libquarot_hip.so)
+    python -m quarot_amd.build                # compile every source, link in-tree (quarot_amd/libquarot_hip.so)
+    python -m quarot_amd.build --incremental  # recompile only sources newer than their objects
 """
+import concurrent.futures
+import os
 import pathlib
 import subprocess
 import sys
@@ -9,8 +12,9 @@ import sys
 PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libquarot_hip.so"
-SOURCES = ("api.hip", "quant.hip", "gemm.hip", "gemm_f6.hip", "hadamard.hip", "kv.hip", "attn.hip")
-FLAGS = ("--offload-arch=gfx950", "-O3", "-fPIC", "-shared", "-std=c++17", "-fno-gpu-rdc",
+OBJ = PKG.parent / "build" / "obj"
+SOURCES = ("api.hip", "quant.hip", "gemm.hip", "gemm_f6.hip", "hadamard.hip", "kv.hip", "attn.hip", "calib.hip")
+FLAGS = ("--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
          # every fp16/fp32 operation must round on its own (the reference's results are defined that
          # way): no fused multiply-add contraction unless a kernel spells fma out
          "-ffp-contract=off",
@@ -19,9 +23,7 @@ FLAGS = ("--offload-arch=gfx950", "-O3", "-fPIC", "-shared", "-std=c++17", "-fno
          "-Wno-unused-command-line-argument")
 
 
-def build(verbose=True):
-    srcs = [str(CSRC / s) for s in SOURCES if (CSRC / s).exists()]
-    cmd = ["hipcc", *FLAGS, *srcs, "-o", str(LIB)]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -31,8 +33,26 @@ def build(verbose=True):
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose=True, incremental=False):
+    """One object per source (compiled side by side), then one link.  incremental: a source is
+    recompiled only if it, or any header beside it, is newer than its object."""
+    OBJ.mkdir(parents=True, exist_ok=True)
+    headers_mtime = max((h.stat().st_mtime for h in CSRC.glob("*.h")), default=0.0)
+    jobs, objs = [], []
+    for s in SOURCES:
+        src, obj = CSRC / s, OBJ / (s[:-4] + ".o")
+        objs.append(str(obj))
+        fresh = incremental and obj.exists() and obj.stat().st_mtime > max(src.stat().st_mtime, headers_mtime)
+        if not fresh:
+            jobs.append(["hipcc", *FLAGS, "-c", str(src), "-o", str(obj)])
+    workers = max(1, min(len(jobs), (os.cpu_count() or 2)))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=workers) as pool:
+        list(pool.map(lambda c: _run(c, verbose), jobs))
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", str(LIB)], verbose)
     return LIB
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv)

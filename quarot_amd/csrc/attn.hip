@@ -102,6 +102,24 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
     const int b = bh / c.num_heads, h = bh - b * c.num_heads;
     const int p0 = c.indptr[b], npages = c.indptr[b + 1] - p0;
     const int seq_len = npages > 0 ? (npages - 1) * c.page_size + c.last_page_offset[b] : 0;
+    if (npages <= 0) {
+        // A sequence without pages (uniform over the workgroup): nothing may be read -- its slice of kv_indices is
+        // empty, and so may be the whole list and the page pool.  The result is the empty softmax state, i.e. the
+        // 0 / 0 that the loop below would arrive at (and the reference's kernel does).
+        if (threadIdx.x < 128) {
+            if (splits == 1) {
+                o[(int64_t)bh * 128 + threadIdx.x] = (f16)__builtin_nanf("");
+            } else {
+                float* dst = part + (int64_t)blockIdx.x * 132;
+                if (threadIdx.x == 0) {
+                    dst[0] = -5e4f;
+                    dst[1] = 0.f;
+                }
+                dst[4 + threadIdx.x] = 0.f;
+            }
+        }
+        return;
+    }
 
     // this lane's 32 query values as fp16 pairs in the order the codes are consumed: word j of a 16-byte
     // piece holds dimensions 8 j .. 8 j + 7, and (word >> 4 i) & 0x000F000F isolates codes i and i + 4
@@ -410,6 +428,7 @@ int check_cache(const void* kv_data, const void* kv_param, const void* kv_indptr
         return QR_E_SHAPE;
     if (head_dim != 128) return QR_E_UNSUPPORTED;          // as the reference's bindings (CHECK_EQ(head_dim, 128))
     if (batch_size == 0) return QR_OK;
+    if (num_pages == 0) return QR_E_SHAPE;                 // sequences but no page pool: nothing a page number could name
     if (!kv_data || !kv_param || !kv_indptr || !kv_indices || !last_page_offset) return QR_E_NULL;
     if (((uintptr_t)kv_data & 15) || ((uintptr_t)kv_param & 3)) return QR_E_ALIGN;
     return QR_OK;

@@ -1288,8 +1288,7 @@ int launch_spk(const void* A, const void* B, int M, int N, int Kb, void* C, void
     const bool ragged = (Kb & 127) != 0;
     // stage buffers of 48 KB: two behind staging registers, three when loaded straight into LDS
     const size_t LDS = (size_t)(ragged ? 2 : 3) * (128 + 256) * 8 * 16;
-    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
-        return launch_ks<128, 256, 2, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
+    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32)) return QR_E_UNSUPPORTED;   // (the dispatcher routes these away)
     hipError_t e;
     if (Y) {
         auto kern = ragged ? gemm_spk_kernel<true, true> : gemm_spk_kernel<true, false>;
@@ -1322,9 +1321,8 @@ int launch_sp256(const void* A, const void* B, int M, int N, int Kb, void* C, vo
     const int nxcd = qr_device().xcds;                      // the grid is a whole number of rounds over the XCDs
     const unsigned grid = (unsigned)((tiles + nxcd - 1) / nxcd * nxcd);
     const bool ragged = (Kb & 127) != 0;
-    // operands are addressed through 32-bit buffer offsets
-    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32))
-        return launch_cfg<256, 256, 4, 2>(A, B, M, N, Kb, C, Y, sA, sB, bias, st);
+    // operands are addressed through 32-bit buffer offsets (the dispatcher routes larger ones away)
+    if ((int64_t)M * Kb >= (1LL << 32) || (int64_t)N * Kb >= (1LL << 32)) return QR_E_UNSUPPORTED;
     using Kern = void (*)(const uint8_t*, const uint8_t*, int, int, int, int32_t*, f16*, const f16*, const f16*, const f16*,
                           int, int, int);
     static const Kern table[2][2][2] = {
@@ -2181,6 +2179,12 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return QR_E_ALIGN;
     if (Y ? ((uintptr_t)Y & 7) : ((uintptr_t)C & 15)) return QR_E_ALIGN;
     const int m = (int)M, n = (int)N, kb = (int)(K / 2);
+    // An operand of 4 GiB or more: every specialised kernel below addresses its operands through 32-bit offsets;
+    // the plain tiled kernel computes 64-bit row addresses and takes any shape (rows beyond M or N are clamped).
+    if (M * (int64_t)kb >= (1LL << 32) || N * (int64_t)kb >= (1LL << 32)) {
+        if (M <= 128) return launch_cfg<128, 128, 2, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+        return launch_cfg<256, 256, 4, 2>(A, B, m, n, kb, C, Y, sA, sB, bias, st);
+    }
     const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
     // one to four tokens: the dot-product kernel -- except two to four tokens against a weight with enough rows for the
     // shared-token kernel, which is ahead there (57344 x 8192: 40.2 against 42.9 us)

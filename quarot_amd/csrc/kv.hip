@@ -308,15 +308,9 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
             hn[o][e] = neg ? (f16)1.0f : (f16)-1.0f;
         }
 
-    // Identity tiles (PAGED only): a part that is quantised WITHOUT the transform -- the values of an append, or
-    // keys when the caller wants none -- goes through the same matrix instructions with I in place of H_128
-    // (exact: one non-zero product per sum), so that keys and values of an append are ONE launch: blocks
-    // [0, blocks1) take x, blocks [blocks1, 2 blocks1) take x2 into the value slots.
-    f16x8 ib[2];
-#pragma unroll
-    for (int o = 0; o < 2; ++o)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ib[o][e] = (PAGED && v == 16 * o + 8 * h + e) ? (f16)1.0f : (f16)0.0f;
+    // PAGED: a part that is quantised WITHOUT the transform -- the values of an append, or keys when the caller
+    // wants none -- skips the matrix stage (its bit in plain_mask), so that keys and values of an append are ONE
+    // launch: blocks [0, blocks1) take x, blocks [blocks1, 2 blocks1) take x2 into the value slots.
     const int64_t blocks1 = (vectors + 31) >> 5;
     const int64_t blocks = (PAGED && x2) ? 2 * blocks1 : blocks1;
     const int64_t wstride = (int64_t)gridDim.x * KM_WAVES;
@@ -356,24 +350,30 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
         fetch(blk + wstride < blocks ? blk + wstride : blocks - 1);
     }
     for (; blk < blocks; blk += wstride) {
-        u32x4 xf[8];
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) xf[ks] = stage[km_slot(v, 2 * ks + h)];
         const bool second = PAGED && blk >= blocks1;               // wave-uniform
         const bool plain = PAGED && ((plain_mask >> (second ? 1 : 0)) & 1);
-        const float oscale = plain ? 1.0f : hscale;
-        f32x16 acc[4];
-#pragma unroll
-        for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[jt][r] = 0.f;
+        // scaled, rounded outputs: yw[jt][qq] = the four outputs j = 32 jt + 8 qq + 4 h + (0..3), two per word
+        u32 yw[4][4][2];
         if (plain) {
+            // no transform: the lane's outputs are the staged values themselves (half h of piece 4 jt + qq of row v),
+            // taken as they are -- an infinity or NaN stays in its own element, as in the separate quantiser
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
-                for (int o = 0; o < 2; ++o)
-                    acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ib[o], __builtin_bit_cast(f16x8, xf[2 * jt + o]), acc[jt], 0, 0, 0);
+                for (int qq = 0; qq < 4; ++qq) {
+                    const u32x2 t = ((const u32x2*)stage)[km_slot(v, 4 * jt + qq) * 2 + h];
+                    yw[jt][qq][0] = t[0];
+                    yw[jt][qq][1] = t[1];
+                }
         } else {
+            u32x4 xf[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) xf[ks] = stage[km_slot(v, 2 * ks + h)];
+            f32x16 acc[4];
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[jt][r] = 0.f;
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt)
 #pragma unroll
@@ -382,16 +382,14 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                     acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(neg ? hn[ks & 1] : hb[ks & 1],
                                                                      __builtin_bit_cast(f16x8, xf[ks]), acc[jt], 0, 0, 0);
                 }
+#pragma unroll
+            for (int jt = 0; jt < 4; ++jt)
+#pragma unroll
+                for (int qq = 0; qq < 4; ++qq) {
+                    yw[jt][qq][0] = narrow_f16x2(acc[jt][4 * qq] * hscale, acc[jt][4 * qq + 1] * hscale);
+                    yw[jt][qq][1] = narrow_f16x2(acc[jt][4 * qq + 2] * hscale, acc[jt][4 * qq + 3] * hscale);
+                }
         }
-        // scaled, rounded outputs: yq[jt][qq] = the four outputs j = 32 jt + 8 qq + 4 h + (0..3), two per word
-        u32 yw[4][4][2];
-#pragma unroll
-        for (int jt = 0; jt < 4; ++jt)
-#pragma unroll
-            for (int qq = 0; qq < 4; ++qq) {
-                yw[jt][qq][0] = narrow_f16x2(acc[jt][4 * qq] * oscale, acc[jt][4 * qq + 1] * oscale);
-                yw[jt][qq][1] = narrow_f16x2(acc[jt][4 * qq + 2] * oscale, acc[jt][4 * qq + 3] * oscale);
-            }
         const int64_t blk1 = second ? blk - blocks1 : blk;
         const int64_t vec = blk1 * 32 + v;
         if (!QUANT) {
@@ -434,7 +432,7 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
         // Is every value finite?  Behind the transform that needs no pass over the values: an infinity or NaN in
         // a vector reaches EVERY output of that vector (each is a sum of all 128 inputs times +-1), so one output
         // tells; what is left is a finite sum too large for fp16, and that shows in the minimum or maximum.
-        // Parts that pass through the identity (appends) are looked at value by value.
+        // Appends (parts of which skip the transform) are looked at value by value.
         bool bad;
         if (PAGED) {
             u16x2 am2 = {0, 0};                                    // largest magnitude bits: >= 0x7c00 means inf or NaN
@@ -493,7 +491,8 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                         }
                     }
             const float omn = __shfl_xor(mn, 32, 64), omx = __shfl_xor(mx, 32, 64);
-            has_nan = has_nan || (__shfl_xor((int)has_nan, 32, 64) != 0);
+            const int other_nan = __shfl_xor((int)has_nan, 32, 64);    // (every lane takes part: behind a short-circuit
+            has_nan = has_nan || other_nan != 0;                       //  `||` the lanes that hold the NaN would sit the exchange out)
             mn = omn < mn ? omn : mn;
             mx = omx > mx ? omx : mx;
             if (has_nan) mn = mx = __builtin_nanf("");
@@ -643,7 +642,7 @@ extern "C" int qr_kv_dequant_i4_f16(const void* q, const void* scale, const void
 
 // Quantise new K and V vectors and write them straight into their pages: what
 // MultiLayerPagedKVCache4Bit.update does with matmul_had_cuda, asym_quantize_and_pack_i4 (twice), two
-// torch.cat and init_kv_i4 / append_kv_i4 (quarot/transformers/kv_cache.py:174-251), as two launches.
+// torch.cat and init_kv_i4 / append_kv_i4 (quarot/transformers/kv_cache.py:174-251), as one launch.
 extern "C" int qr_kv_quant_append_f16_i4(const void* k, const void* v, int64_t tokens, const void* append_indptr_or_null,
                                          int k_had_mode, void* kv_data, void* kv_param, const void* kv_indptr,
                                          const void* kv_indices, const void* last_page_offset, int64_t num_pages,
@@ -665,7 +664,7 @@ extern "C" int qr_kv_quant_append_f16_i4(const void* k, const void* v, int64_t t
     const int64_t vectors = tokens * num_heads;
     const float hs = (float)(1.0 / __builtin_sqrt(128.0));
     hipStream_t st = (hipStream_t)stream;
-    // keys (through H_128, or through the identity when the caller wants them untransformed) and values (identity) in
+    // keys (through H_128, or as they are when the caller wants them untransformed) and values (as they are) in
     // ONE launch of the matrix-core kernel: bit for bit the codes, scales and zeros of the separate quantisers
     pd.kv = 0;
     return launch_had128<true, true>(k, vectors, hs, nullptr, nullptr, nullptr, nullptr, st, pd, v, k_had_mode ? 2 : 3);

@@ -59,8 +59,9 @@ class Linear4bit(torch.nn.Module):
         rows = q.numel() // max(q.shape[-1], 1)
         if (self.prefill_fp6 and q.is_cuda and rows >= self.fp6_min_rows and self.in_features % 64 == 0
                 and max(rows, self.out_features) * self.in_features * 3 // 4 < 4290000000):     # (32-bit offsets inside the kernel)
-            return quarot_amd.linear_f6(quarot_amd.convert_i4_f6(q), x.scales_x, self._weight_f6(), self.weight_scales,
-                                        self.bias)
+            y = quarot_amd.linear_f6(quarot_amd.convert_i4_f6(q), x.scales_x, self._weight_f6(), self.weight_scales,
+                                     self.bias)
+            return y.view(*q.shape[:-1], self.out_features)     # the converter flattens the leading dimensions
         return quarot_amd.linear_i4(q, x.scales_x, self.weight, self.weight_scales, self.bias)
 
     @staticmethod

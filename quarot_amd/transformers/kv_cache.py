@@ -164,7 +164,9 @@ def quantize_append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_of
 
 
 @functools.lru_cache(maxsize=1024)
-def _decode_workspace_bytes(batch, heads, max_seq_len):
+def _decode_workspace_bytes(batch, heads, max_seq_len, device_index=None):
+    # (the split plan depends on the current device's compute-unit count: called with the device current, and
+    # the device index is part of the cache key)
     return _lib.lib().qr_batch_decode_workspace_bytes(batch, heads, max_seq_len)
 
 
@@ -188,9 +190,9 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
     _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
     _check(last_page_offset.shape[0] == batch, f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
     dev = kv_data.device
-    ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len)) if max_seq_len else 0
-    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
     with _lib.on_device(dev):
+        ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len), dev.index) if max_seq_len else 0
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
         entry = _lib.lib().qr_batch_decode_qhad_i4 if q_hadamard else _lib.lib().qr_batch_decode_i4
         _lib.check(entry(
             o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),

@@ -109,6 +109,35 @@ def test_quantise_and_append_places_the_oracle_quantisers_codes(page_size, lens,
     assert torch.equal(gd2, gd3) and torch.equal(gp2, gp3)
 
 
+@pytest.mark.parametrize("hadamard", [True, False])
+def test_quantise_and_append_with_infinities_and_nans_equals_the_separate_quantisers(hadamard):
+    """A vector that holds an infinity or a NaN: the one-launch quantise-and-append must store what the separate
+    quantiser (itself pinned against the oracle on such vectors) followed by the append stores -- in particular an
+    untransformed vector keeps the non-finite value in its own element (scale inf, zero = -min for an infinity)."""
+    rng = np.random.default_rng(77)
+    heads, layer, page_size, lens = 4, 1, 16, [40, 9, 23]
+    data, param, indptr, indices, last = paged_case(rng, heads, page_size, lens)
+    app = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    T = int(app[-1])
+    k, v = synth_kv(rng, T, heads), synth_kv(rng, T, heads)
+    for t, (a, b) in enumerate([(np.inf, None), (-np.inf, None), (np.nan, None), (np.inf, -np.inf), (np.inf, np.nan), (65504, -65504)]):
+        for x in (k, v):
+            x[3 + 5 * t, t % heads, 7 * t] = a
+            if b is not None:
+                x[3 + 5 * t, t % heads, 127 - t] = b
+    gd2, gp2 = gpu(data), gpu(param)
+    gd3, gp3 = gd2.clone(), gp2.clone()
+    q1, s1, z1 = kv.asym_quantize_and_pack_i4(gpu(k), hadamard=hadamard)
+    q2, s2, z2 = kv.asym_quantize_and_pack_i4(gpu(v))
+    vq, vs, vz = o.kv_asym_quant(v)                         # the untransformed side against the oracle as well
+    assert np.array_equal(q2.cpu().numpy(), vq)
+    assert np.array_equal(bits(s2.cpu().numpy()), bits(vs)) and np.array_equal(bits(z2.cpu().numpy()), bits(vz))
+    kv.init_kv_i4(gd2, gp2, gpu(indptr), gpu(indices), gpu(last), q1, q2, torch.cat([s1, z1], -1), torch.cat([s2, z2], -1), gpu(app), layer)
+    kv.quantize_append_kv_i4(gd3, gp3, gpu(indptr), gpu(indices), gpu(last), gpu(k), gpu(v), gpu(app), layer, hadamard=hadamard)
+    assert torch.equal(gd2, gd3)
+    assert torch.equal(gp2.view(torch.int16), gp3.view(torch.int16))          # (bit patterns: NaN parameters compare unequal as floats)
+
+
 @pytest.mark.parametrize("page_size,lens", [(16, [1, 16, 17, 100, 700]), (64, [64, 1000, 129]), (5, [11, 1, 64]), (100, [250, 99, 1]),
                                             (2048, [2048, 2047])])
 def test_decode_attention_against_the_oracle(page_size, lens):
@@ -130,6 +159,32 @@ def test_decode_attention_against_the_oracle(page_size, lens):
         b = lens.index(1)
         _, _, vc, vp = o.paged_gather(data, param, indptr, indices, last, layer, b)
         assert close(out[b].cpu().numpy(), o.paged_dequant(vc, vp)[0])
+
+
+def test_decode_attention_of_a_sequence_without_pages_reads_nothing():
+    """A sequence whose page list is empty (it is the LAST one, so its slice of kv_indices starts at the list's end)
+    gets the empty softmax, 0 / 0 = NaN, as in the reference's kernel; the other sequences are unaffected.  With the
+    split along the sequence as well.  A cache without any page is refused before the launch."""
+    rng = np.random.default_rng(3)
+    heads, layer, page_size, lens = 3, 0, 16, [40, 7]
+    data, param, indptr, indices, last = paged_case(rng, heads, page_size, lens, layers=1)
+    q = rng.standard_normal((3, heads, 128)).astype(F16)
+    want = o.paged_batch_decode(q[:2], data, param, indptr, indices, last, layer)
+    indptr3 = np.concatenate([indptr, indptr[-1:]]).astype(np.int32)        # third sequence: no pages
+    last3 = np.concatenate([last, [0]]).astype(np.int32)
+    used = gpu(indices[: indptr[-1]])                                       # the list ends where the empty slice starts
+    for hint in (None, 40):
+        out = torch.zeros((3, heads, 128), dtype=torch.float16, device="cuda:0")
+        kw = {} if hint is None else {"max_seq_len": hint}
+        kv.batch_decode_i4(out, gpu(q), gpu(data), gpu(param), gpu(indptr3), used, gpu(last3), layer, **kw)
+        got = out.cpu().numpy()
+        assert close(got[:2], want) and np.isnan(got[2]).all()
+    L, st = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    out = torch.zeros((3, heads, 128), dtype=torch.float16, device="cuda:0")
+    gq, gd, gp, gi, gl = gpu(q), gpu(data), gpu(param), gpu(indptr3), gpu(last3)
+    rc = L.qr_batch_decode_i4(out.data_ptr(), gq.data_ptr(), gd.data_ptr(), gp.data_ptr(), gi.data_ptr(), used.data_ptr(),
+                              gl.data_ptr(), 0, 1, 0, heads, page_size, 128, 3, 0, None, 0, st)
+    assert rc == -2, rc                                                     # QR_E_SHAPE: sequences but no page pool
 
 
 @pytest.mark.parametrize("page_size,lens", [(16, [1, 33, 700, 4100]), (5, [11, 64])])

@@ -361,6 +361,33 @@ def test_enable_fp6_prefill_on_a_module_tree_changes_no_result():
         assert torch.equal(model[k](xs[k][:100]), want[k][:100])        # short input: the usual route
 
 
+def test_fp6_prefill_keeps_the_leading_dimensions_of_a_batched_input():
+    """[batch, seq, hidden] inputs: the FP6 route returns [batch, seq, out] like the default route and the reference's
+    matmul (quarot/__init__.py:37-41 views the result as (*A.shape[:-1], -1)), directly and through the chains."""
+    nn_ = quarot_amd.nn
+    rng = np.random.default_rng(17)
+    def lin(k, n):
+        m = nn_.Linear4bit(k, n, bias=True).half().cuda()
+        m.weight.copy_(gpu(o.pack_i4(rng.integers(-8, 8, (n, k)))))
+        m.weight_scales.copy_(gpu((np.abs(rng.standard_normal((n, 1))) * 0.01 + 0.001).astype(F16)))
+        m.bias.copy_(gpu(rng.standard_normal(n).astype(F16)))
+        return m
+    chains = {"plain": nn_.Linear4bitSequential(nn_.Quantizer(), lin(512, 384)),
+              "had": nn_.Linear4bitSequential(nn_.OnlineHadamard(2304), nn_.Quantizer(), lin(2304, 320))}
+    for name, chain in chains.items():
+        chain = chain.cuda()
+        k = chain[-1].in_features
+        x = gpu(synth_x(600, k, seed=21).reshape(2, 300, k))
+        want = chain(x)
+        packed = chain[-2](x if name == "plain" else chain[0](x))
+        want_direct = chain[-1](packed)
+        assert want.shape == want_direct.shape == (2, 300, chain[-1].out_features)
+        assert nn_.enable_fp6_prefill(chain, min_rows=256) == 1
+        got, got_direct = chain(x), chain[-1](packed)
+        assert got.shape == want.shape and torch.equal(got, want)
+        assert got_direct.shape == want_direct.shape and torch.equal(got_direct, want_direct)
+
+
 def test_matmul_known_answers_and_leading_dims():
     k = 28672                                      # the largest K of the configs: |acc| = 64 K = 1 835 008
     a = np.full((3, k // 2), 0x88, np.uint8)       # all -8
