@@ -1334,6 +1334,287 @@ __global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard
     }
 }
 
+// ---- K >= 64, m = 64, fp16 staging, quantiser fused: the lean form with the fewest vector instructions ----
+// Same decomposition and the same arithmetic as hadamard_m64q_kernel (four waves per row, hadK fragments in
+// registers, only T through LDS; identical fragments and accumulation order, so codes and scales are those of
+// hadamard_m64_kernel followed by the quantiser, bit for bit).  What the counters and a set of timing-only
+// ablations showed about that kernel: its time is the SUM of its vector and matrix instructions' issue cycles on a
+// SIMD -- removing the loads, the LDS reads or doubling the waves per SIMD changed little or nothing, removing
+// instructions did.  So this form issues fewer of them per row:
+//   * the row maximum is taken on the fp32 accumulators (v_max3_f32 with |.| modifiers: one instruction per two
+//     values, where the packed 16-bit form took an AND and a maximum per two) and rounded to fp16 once -- rounding is
+//     monotone, so that is the maximum of the rounded values.  v_max3 drops NaNs; a NaN or infinity anywhere in a
+//     row reaches every output, so one output per lane is tested, and a wave that sees anything non-finite takes
+//     the exact bit-pattern maximum of the lean kernel above instead (NaN wins, as in torch.max);
+//   * the codes are formed right after the row maximum is known, from the registers the matrix stage left them
+//     in: no copies to a "previous row" set, no second set of code registers;
+//   * the quotient goes from the packed fp16 pair to the packed fp16 quotient in one mixed-precision instruction
+//     per value (sym_pair_fast) and, where the clamp cannot act (clip >= 1, normal scale), without a clamp: three
+//     instructions per pair of values where there were six;
+//   * zero fragments for rows beyond hadK's order are formed only in the one tile that is partial, and a tile that
+//     lies entirely beyond it is skipped.
+// TPW: how many of this wave's tiles (rows (wave + 4 i) 16 .. + 15 of hadK) lie inside hadK, at least in part;
+// only the last of them can be partial.  (A function of the wave so that every loop below is free of branches.)
+template <int KS2, int TPW, int CHUNKS>
+__device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, int64_t rows, int n, int K,
+                                                   const f16* __restrict__ hadK, float scale, float clip,
+                                                   u32* __restrict__ q, f16* __restrict__ scales, f32x4* smem_raw, u32* red) {
+    constexpr int CT = 4, NT = 2 * KS2;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, g = lane >> 4;
+    const int nchunks = n >> 3;
+    u32x2* Tl = (u32x2*)smem_raw;                                      // [CT][NT][64 lanes]
+
+    // Sylvester fragments of hadamard_m64_kernel: one base per parity of the column tile; where that kernel takes a
+    // negated fragment (second contraction step, column tiles 2 and 3) the OTHER operand is negated here instead
+    // (sign bits of its fp16 pairs flipped: the products are the same numbers), which saves eight registers
+    f16x8 sb[2];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bool neg = ((__builtin_popcount(((g & 1) * 8 + j) & l16) + ((g >> 1) & o)) & 1) != 0;
+            sb[o][j] = neg ? (f16)-1.0f : (f16)1.0f;
+        }
+    // dval: this lane's row of tile i exists
+    bool dval[TPW];
+    int goff[TPW];
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+        const int t16 = (wave + 4 * i) * 16;
+        dval[i] = t16 + l16 < K;
+        goff[i] = (dval[i] ? t16 + l16 : 0) * 8 + g;         // 16-byte pieces g and 4 + g of that row of X[K][64]
+    }
+    u32x4 xr[TPW][2];
+    auto load_row = [&](const f16* src) {
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) xr[i][c] = *((const u32x4*)src + goff[i] + 4 * c);
+    };
+    int64_t row = blockIdx.x;
+    if (row < rows) load_row(x + row * (int64_t)n);
+    // hadK's fragments (contraction index in the order k = 32 ks + 16 hh + 4 g + e, as in the kernels above), fetched
+    // through LDS: the tiles with the same i of the four waves are 64 consecutive rows of hadK, which the workgroup
+    // copies as one run of 16-byte pieces (coalesced, every line requested once) into the region that will hold T;
+    // each lane then picks its 8-byte pieces from there.  Loading them straight from memory -- a lane's pieces lie 32
+    // bytes apart, every workgroup of the grid asks at the same moment -- cost 3 of the 23 us of a 2048-row launch.
+    f16x8 hf[TPW][KS2];
+    {
+        u32x4* stage = (u32x4*)smem_raw;
+        const u32x4* src = (const u32x4*)hadK;
+        const int total = (K * K) >> 3;                                // 16-byte pieces of hadK (orders are multiples of 4)
+        const int count = (64 * K) >> 3;                               // ... of 64 rows: at most KS2 per thread
+        // every load of every run is issued before the first is used (one memory latency in all)
+        u32x4 hk[CHUNKS][KS2];
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i)
+#pragma unroll
+            for (int j = 0; j < KS2; ++j) {
+                const int pc = tid + j * HT, at = i * count + pc;
+                hk[i][j] = src[pc < count && at < total ? at : 0];
+            }
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+#pragma unroll
+            for (int j = 0; j < KS2; ++j) {
+                const int pc = tid + j * HT;
+                if (pc < count) stage[pc] = hk[i][j];
+            }
+            __syncthreads();
+            if (i < TPW) {
+                const int hr = (wave + 4 * i) * 16 + l16;
+#pragma unroll
+                for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh) {
+                        const int hc = ks * 32 + hh * 16 + g * 4;
+                        const bool ok = hr < K && hc < K;
+                        f16x4 v = *(const f16x4*)((const f16*)stage + (ok ? (wave * 16 + l16) * K + hc : 0));
+                        if (!ok) v = f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) hf[i][ks][hh * 4 + e] = v[e];
+                    }
+            }
+            __syncthreads();
+        }
+        // T slots of tiles beyond K are never written afterwards: clear once
+        for (int i = tid; i < CT * NT * 32; i += HT) stage[i] = u32x4{0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS2; ++ks) asm volatile("" : "+v"(hf[t][ks]));
+    __syncthreads();
+
+    for (; row < rows; row += gridDim.x) {
+        const int64_t nrow = row + gridDim.x;
+        // ---- stage 1: T = X . H_64 for this wave's tiles
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            {
+                const int t = wave + 4 * i;
+                u32x4 a0 = xr[i][0], a1 = xr[i][1];
+                if (i == TPW - 1) {                          // the tile that may be partial: rows beyond K are zero fragments
+                    a0 = dval[i] ? a0 : u32x4{0, 0, 0, 0};
+                    a1 = dval[i] ? a1 : u32x4{0, 0, 0, 0};
+                }
+                const u32x4 a1n = a1 ^ 0x80008000u;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a0), sb[ct & 1], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, (ct >> 1) ? a1n : a1), sb[ct & 1], acc, 0, 0, 0);
+                    u32x2 hi;
+                    hi[0] = narrow_f16x2(acc[0] * scale, acc[1] * scale);
+                    hi[1] = narrow_f16x2(acc[2] * scale, acc[3] * scale);
+                    Tl[(ct * NT + t) * 64 + lane] = hi;
+                }
+            }
+        }
+        // the next row's loads, a whole turn ahead (unconditional, like every store below: with a fixed number of
+        // memory operations per turn the wait for these loads, a turn later, need not include the stores issued
+        // after them; the last turn re-reads its own row)
+        load_row(x + (nrow < rows ? nrow : row) * (int64_t)n);
+        __syncthreads();
+        // ---- stage 2: Y^T = T^T . hadK^T; results stay in registers
+        float mxf = 0.f;
+        u32x2 yv[TPW][CT];
+        float probe = 0.f;                                   // one output of a row that always exists (K >= 64)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            // fragments of T one contraction step ahead of their use (8 registers; a whole column tile's set ahead
+            // was no faster, and three workgroups per CU, which these registers would allow, spilled and lost 15 %)
+            auto frag = [&](int ks) {
+                const u32x2 p0 = Tl[(ct * NT + 2 * ks) * 64 + lane], p1 = Tl[(ct * NT + 2 * ks + 1) * 64 + lane];
+                return u32x4{p0[0], p0[1], p1[0], p1[1]};
+            };
+            f32x4 acc[TPW];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+            u32x4 th = frag(0);
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                __builtin_amdgcn_sched_barrier(0);           // (keeps the scheduler from hoisting every read to the top)
+                const u32x4 cur = th;
+                if (ks + 1 < KS2) th = frag(ks + 1);
+#pragma unroll
+                for (int i = 0; i < TPW; ++i)
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, cur), hf[i][ks], acc[i], 0, 0, 0);
+            }
+            if (ct == 0) probe = acc[0][0];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+#ifdef QR_OLDCVT
+                yv[i][ct][0] = narrow_f16x2(acc[i][0], acc[i][1]);
+                yv[i][ct][1] = narrow_f16x2(acc[i][2], acc[i][3]);
+#else
+                yv[i][ct][0] = cvt_f16x2(acc[i][0], acc[i][1]);
+                yv[i][ct][1] = cvt_f16x2(acc[i][2], acc[i][3]);
+#endif
+                // (rows of hadK beyond its order are zero fragments: their outputs are 0, or NaN from 0 . inf, which
+                // the maximum instruction drops)
+                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[i][0])), __builtin_fabsf(acc[i][1]));
+                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[i][2])), __builtin_fabsf(acc[i][3]));
+            }
+        }
+        // ---- this row's maximum: rounded once; a wave that sees anything non-finite takes the exact form
+        u32 mx = f16_bits((f16)mxf);
+        if (__builtin_amdgcn_ballot_w64(mx >= 0x7c00u || probe != probe) != 0) {
+            u16x2 mx2 = {0, 0};
+#pragma unroll
+            for (int i = 0; i < TPW; ++i)
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    // (magnitude bits; rows beyond hadK's order do not count: 0 . inf leaves NaNs there)
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, dval[i] ? yv[i][ct][0] & 0x7fff7fffu : 0u));
+                    mx2 = __builtin_elementwise_max(mx2, __builtin_bit_cast(u16x2, dval[i] ? yv[i][ct][1] & 0x7fff7fffu : 0u));
+                }
+            mx = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
+        }
+        mx = wave_max_u32_dpp(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < HT / QR_WAVE; ++w) mx = mx > red[w] ? mx : red[w];
+        const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+        scales[row] = sh;                                     // every lane, the same value: no branch around the store
+        const float sp = (float)sh;
+        // ---- codes: lanes l16 + 16 g hold, for output row k' = 16 t + l16, the columns 16 ct + 4 g .. + 3
+        u32 c01[TPW], c23[TPW];
+        if (fast_quant_ok(mx, sp)) {
+            const FastRecip fq = make_fast_recip(sp);
+            // no clamp where it cannot act: |x| <= amax and a normal scale >= (amax / 7) (1 - 2^-11)^2 keep |x / s| below 7.5
+            if (clip >= 1.0f && sp >= 6.103515625e-05f) {
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    u32 b0[4], b1[4];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        b0[w] = sym_pair_fast<false>(yv[i][w >> 1][w & 1], fq);
+                        b1[w] = sym_pair_fast<false>(yv[i][2 + (w >> 1)][w & 1], fq);
+                    }
+                    c01[i] = pack_nibbles8(b0);
+                    c23[i] = pack_nibbles8(b1);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    u32 b0[4], b1[4];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        b0[w] = sym_pair_fast<true>(yv[i][w >> 1][w & 1], fq);
+                        b1[w] = sym_pair_fast<true>(yv[i][2 + (w >> 1)][w & 1], fq);
+                    }
+                    c01[i] = pack_nibbles8(b0);
+                    c23[i] = pack_nibbles8(b1);
+                }
+            }
+        } else {
+            const bool fs = scale_fast_ok(sp);
+            const float rs = fs ? 1.0f / sp : 0.0f;
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                c01[i] = sym_codes8(u32x4{yv[i][0][0], yv[i][0][1], yv[i][1][0], yv[i][1][1]}, sp, rs, fs);
+                c23[i] = sym_codes8(u32x4{yv[i][2][0], yv[i][2][1], yv[i][3][0], yv[i][3][1]}, sp, rs, fs);
+            }
+        }
+        // piece (g, ct) -> lane ct: first the halves of the wave (g and g ^ 2), then neighbouring rows of 16 lanes
+        u32x2* qrow = (u32x2*)(q + row * (int64_t)nchunks);
+        u32x2 outv[TPW];
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const auto s1 = __builtin_amdgcn_permlane32_swap(c01[i], c23[i], false, false);
+            const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);
+            const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);
+            const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
+            outv[i] = u32x2{__builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u), __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u)};
+        }
+        // lanes on rows beyond K store their first tile's piece once more (K >= 64: that row exists)
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int kp = (wave + 4 * i) * 16 + l16;
+            qrow[(dval[i] ? kp : wave * 16 + l16) * CT + g] = dval[i] ? outv[i] : outv[0];
+        }
+        // Tl is next written after the second barrier of this turn, which every wave reaches only after its stage-2
+        // reads; red[] is next written after the next row's first barrier.  (A form with T double-buffered and ONE
+        // barrier per row -- the next row's stage 1 ahead of it -- was measured no faster.)
+    }
+}
+
+template <int KS2>
+__global__ __launch_bounds__(HT, 2) void hadamard_m64r_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
+                                                            const f16* __restrict__ hadK, float scale, float clip,
+                                                            u32* __restrict__ q, f16* __restrict__ scales) {
+    constexpr int NT = 2 * KS2, TPW = (NT + 3) / 4;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[HT / QR_WAVE];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // (both forms pass the same barriers: two per 64 rows of hadK and one more before the loop, two per row)
+    if ((wave + 4 * (TPW - 1)) * 16 < K) hadamard_m64r_rows<KS2, TPW, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
+    else hadamard_m64r_rows<KS2, TPW - 1, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
+}
+
 // A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
 // kernel applies with a generated outer factor, in its fp32-precision mode so that the result is
 // rounded to fp16 once, like a plain fp32 transform.  Returns the outer order (0: not applicable).
@@ -1380,12 +1661,12 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
         const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
-        if (!MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
+        if (!MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0 && ((uintptr_t)hadK & 15) == 0) {
             // fused, fp16 staging, no copy of the transformed rows wanted: the lean kernel (T alone in LDS)
             const size_t ldsq = (size_t)4096 * KS2;
 #define QR_M64Q(KS)                                                                                                    \
     do {                                                                                                               \
-        auto kern = hadamard_m64q_kernel<KS>;                                                                          \
+        auto kern = hadamard_m64r_kernel<KS>;                                                                          \
         const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                                     \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
         kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \

@@ -126,6 +126,14 @@ __device__ __forceinline__ u32 narrow_f16x2(float a, float b) {
     return __builtin_bit_cast(u32, h);
 }
 
+// Two floats -> two fp16 (round to nearest even) where nothing can be folded into the conversion (the
+// operands are matrix-instruction results, not products): no empty asm, so no copies of the operands.
+__device__ __forceinline__ u32 cvt_f16x2(float a, float b) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2));
+}
+
 // Reinterpret one 32-bit word as two halves.  Always go through this by-value helper: applying
 // __builtin_bit_cast directly to an element of an ext-vector (v[i]) was seen to read element 0
 // whatever the index.
@@ -261,6 +269,26 @@ __device__ __forceinline__ u32 pack_nibbles8(const u32 (&w)[4]) {
     const u32 even = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
     const u32 odd = __builtin_amdgcn_perm(p23, p01, 0x07060302u);
     return (even & 0x0F0F0F0Fu) | ((odd << 4) & 0xF0F0F0F0u);
+}
+// Two codes from one packed word, as the fp16 pair (1536 + code, 1536 + code).  The quotient is formed as
+// fp16(fma(x, r, 0)) -- the halves go into the mixed-precision multiply as they are, and where the compiler
+// takes the form that rounds the exact product once (v_fma_mixlo/hi_f16) the result is still the correctly
+// rounded fp16 quotient: x r lies within 2^-24 (relative) of x / s and a quotient of two fp16 numbers keeps more
+// than 2^-23 from every rounding boundary it is not exactly on.  The clamp acts on the bit patterns AFTER the
+// addition: 1536 + code in [1528, 1543] is 0x65f8 .. 0x6607, patterns of positive halves order like signed
+// 16-bit integers, every negative sum (quotients below -1536) is a negative integer and an overflow to +inf
+// (0x7c00) lies above: two packed integer instructions instead of two fp32 clamps and a conversion.
+template <bool CLAMP>
+__device__ __forceinline__ u32 sym_pair_fast(u32 w, FastRecip f) {
+    const f16x2 h2 = as_f16x2(w);
+    f16x2 qh = {(f16)__builtin_fmaf((float)h2[0], f.r, 0.0f), (f16)__builtin_fmaf((float)h2[1], f.r, 0.0f)};
+    qh = qh + f16x2{(f16)1536.0f, (f16)1536.0f};
+    if (!CLAMP) return __builtin_bit_cast(u32, qh);
+    typedef short i16x2 __attribute__((ext_vector_type(2)));
+    i16x2 b = __builtin_bit_cast(i16x2, qh);
+    b = __builtin_elementwise_max(b, i16x2{0x65f8, 0x65f8});
+    b = __builtin_elementwise_min(b, i16x2{0x6607, 0x6607});
+    return __builtin_bit_cast(u32, b);
 }
 __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
     u32 b[4];
