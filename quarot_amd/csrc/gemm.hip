@@ -1536,11 +1536,16 @@ __global__ __launch_bounds__(512) void decode_i4_kernel(const uint8_t* __restric
 //   on the order): with a row pitch that is a power of two, workgroups marching through K in step
 //   would all be reading the same few memory channels at any one time (measured 49 -> 41 us at
 //   57344 x 8192).
+// * ksplit > 1 (int32 output only; weights with few rows, 32..64 tokens): `ksplit` workgroups share a block of R
+//   groups and each walks its own slice of K, writing its partial sums to its own [M, N] slab of C -- a workgroup then
+//   pulls 1 / ksplit of the tokens' codes through its CU's vector memory path, which is what bounds this shape (every
+//   CU reading ALL the tokens' codes next to its share of the weights: 0.92 MB beside 0.46 MB at 64 tokens).
 template <int MT, int R, int RD, bool DEQ>
 __global__ __launch_bounds__(768) void decode_xs_kernel(const uint8_t* __restrict__ A, const uint8_t* __restrict__ B,
                                                         int M, int N, int Kb, int32_t* __restrict__ C,
                                                         f16* __restrict__ Y, const f16* __restrict__ sA,
-                                                        const f16* __restrict__ sB, const f16* __restrict__ bias) {
+                                                        const f16* __restrict__ sB, const f16* __restrict__ bias,
+                                                        int ksplit) {
     constexpr int XR = MT * 32;                             // staged rows of X
     constexpr int NL = MT + R;                              // 16-byte chunks per loader thread and stage: 32 rows each
     constexpr int XPLANES = XR * 16;                        // slots of the tokens' planes (32 bytes per packed chunk)
@@ -1550,8 +1555,12 @@ __global__ __launch_bounds__(768) void decode_xs_kernel(const uint8_t* __restric
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 31, h = lane >> 5;
     const bool loader = wave >= 8;                          // waves 8..11 fetch, waves 0..R-1 multiply
-    const int n0 = blockIdx.x * (R * 32);
-    const int stages = (Kb + 127) / 128;
+    const int rblock = blockIdx.x / ksplit, slice = blockIdx.x - rblock * ksplit;
+    const int n0 = rblock * (R * 32);
+    const int all_stages = (Kb + 127) / 128;
+    const int sfirst = (int)((int64_t)all_stages * slice / ksplit);
+    const int stages = (int)((int64_t)all_stages * (slice + 1) / ksplit) - sfirst;      // >= 1: ksplit <= all_stages
+    if (ksplit > 1) C += (int64_t)slice * M * N;
     const bool ragged = (Kb & 127) != 0;
     auto slot8 = [](int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); };
     auto slot16 = [](int row, int chunk, int plane) {
@@ -1573,10 +1582,10 @@ __global__ __launch_bounds__(768) void decode_xs_kernel(const uint8_t* __restric
     }
     const int wdst0 = XPLANES + slot8(srow, piece);         // rows differ by multiples of 32: same swizzle
     const int xdst0 = slot16(srow, piece, 0);
-    const int s0 = blockIdx.x % stages;
-    auto stage_of = [&](int st) {
+    const int s0 = rblock % stages;
+    auto stage_of = [&](int st) {                           // absolute stage of this workgroup's st-th step
         int a = (st < stages ? st : stages - 1) + s0;
-        return a >= stages ? a - stages : a;
+        return sfirst + (a >= stages ? a - stages : a);
     };
     auto fetch = [&](int st, u32x4(&v)[NL]) {
         const int kb = stage_of(st) * 128;
@@ -2046,8 +2055,9 @@ int decode_xs_groups(int N) {
 }
 
 int launch_decode_xs(const void* A, const void* B, int M, int N, int Kb, void* C, void* Y, const void* sA,
-                     const void* sB, const void* bias, hipStream_t st, int rg) {
-    const unsigned grid = (unsigned)(((N + 31) / 32 + rg - 1) / rg);
+                     const void* sB, const void* bias, hipStream_t st, int rg, int ksplit = 1) {
+    if (ksplit > 1 && Y) return QR_E_UNSUPPORTED;           // partial sums exist only as int32
+    const unsigned grid = (unsigned)((((N + 31) / 32 + rg - 1) / rg) * ksplit);
 #define QR_XS(MT, R)                                                                                                  \
     do {                                                                                                              \
         constexpr int RD = 3;   /* deeper rings were measured slower (4: +3 %, 5: +6 %) */                            \
@@ -2058,13 +2068,13 @@ int launch_decode_xs(const void* A, const void* B, int M, int N, int Kb, void* C
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(768), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, nullptr, (f16*)Y, \
-                                                     (const f16*)sA, (const f16*)sB, (const f16*)bias);               \
+                                                     (const f16*)sA, (const f16*)sB, (const f16*)bias, 1);            \
         } else {                                                                                                      \
             auto kern = decode_xs_kernel<MT, R, RD, false>;                                                           \
             e = qr_allow_dynamic_lds((const void*)kern, LDS);                                                         \
             if (e != hipSuccess) return (int)e;                                                                       \
             kern<<<dim3(grid), dim3(768), LDS, st>>>((const uint8_t*)A, (const uint8_t*)B, M, N, Kb, (int32_t*)C,     \
-                                                     nullptr, nullptr, nullptr, nullptr);                             \
+                                                     nullptr, nullptr, nullptr, nullptr, ksplit);                     \
         }                                                                                                             \
     } while (0)
 #define QR_XS_R(MT)                                                                                                   \
@@ -2149,8 +2159,24 @@ __global__ __launch_bounds__(256) void dequant_slabs_kernel(const int32_t* __res
 // M = 96..768, N = 4096..12288, K = 4096..28672 the model is within 10 % and picks the measured
 // optimum or its neighbour (e.g. 256 x 4096 x 11008: 48 -> 26 us with four slices, 256 x 8192 x
 // 28672: 119 -> 78 us with two; 512 x 4096 x 4096 and 256 x 11008 x 4096 stay unsplit).
+// Decode against a weight with too few rows for the shared-token kernel to fill the CUs (70B down_proj: 8192 rows =
+// 64 blocks of four groups): at 40 and more tokens each CU's intake of the tokens' codes bounds the barrier-free
+// kernel.  With scratch from the caller the shared-token kernel runs with four groups per workgroup and as many K
+// slices per block as fill the CUs, and dequant_slabs_kernel adds the slabs.  Measured (8192 x 28672, both launches):
+// 64 tokens 35.5 -> 30.6 us, 48 tokens 31.3 -> 29.8; level at 32 and behind below that, and behind at every token count
+// when K is 8192 (the slices get too short for their fixed costs): those shapes keep the barrier-free kernel.
+int decode_split(int64_t M, int64_t N, int64_t Kb) {
+    if (M < 40 || M > 64 || Kb < 8192 || decode_xs_groups((int)N) != 0) return 1;
+    const int64_t blocks = ((N + 31) / 32 + 3) / 4, cus = qr_device().cus, all_stages = (Kb + 127) / 128;
+    int64_t s = cus / blocks;
+    if (s > all_stages / 16) s = all_stages / 16;
+    if (s > 8) s = 8;
+    return s >= 2 ? (int)s : 1;
+}
+
 int ks_split(int64_t M, int64_t N, int64_t Kb) {
-    if (M <= 64 || N <= 128) return 1;
+    if (M <= 64) return decode_split(M, N, Kb);
+    if (N <= 128) return 1;
     const int64_t tn = (N + 255) / 256;
     const int64_t cus = qr_device().cus;
     if (((M + 127) / 128) * tn >= cus / 2) return 1;
@@ -2193,7 +2219,8 @@ int gemm_dispatch(const void* A, const void* B, int64_t M, int64_t N, int64_t K,
     // slices' partial sums
     const int split = ks_split(M, N, kb);
     if (split > 1 && Y && ws && ws_bytes >= (size_t)split * (size_t)M * (size_t)N * 4 && ((uintptr_t)ws & 15) == 0) {
-        int rc = launch_ks<64, 256, 1, 4>(A, B, m, n, kb, ws, nullptr, nullptr, nullptr, nullptr, st, split);
+        int rc = M <= 64 ? launch_decode_xs(A, B, m, n, kb, ws, nullptr, nullptr, nullptr, nullptr, st, 4, split)
+                         : launch_ks<64, 256, 1, 4>(A, B, m, n, kb, ws, nullptr, nullptr, nullptr, nullptr, st, split);
         if (rc != QR_OK) return rc;
         int64_t db = (M * N / 4 + 255) / 256;
         db = db < 1 ? 1 : (db > 4096 ? 4096 : db);

@@ -63,16 +63,21 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const f16x2 sh = as_f16x2(v[i]) + z2;
-        const float x0 = (float)sh[0], x1 = (float)sh[1];
-        float q0 = __builtin_fmaf(x0, f.r, 0.0f);
-        float q1 = __builtin_fmaf(x1, f.r, 0.0f);
-        if (CLAMP) {
-            q0 = __builtin_amdgcn_fmed3f(q0, 0.0f, 15.0f);
-            q1 = __builtin_amdgcn_fmed3f(q1, 0.0f, 15.0f);
-        }
-        f16x2 h = {(f16)q0, (f16)q1};
+        // the quotient straight from the packed pair to the packed fp16 quotient (one mixed-precision instruction per
+        // value; see sym_pair_fast for why its single rounding is still the correctly rounded division), then + 1536
+        f16x2 h = {(f16)__builtin_fmaf((float)sh[0], f.r, 0.0f), (f16)__builtin_fmaf((float)sh[1], f.r, 0.0f)};
         h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
-        b[i] = __builtin_bit_cast(u32, h);
+        if (CLAMP) {
+            // on the bit patterns: 1536 + code in [1536, 1551] is 0x6600 .. 0x660f; patterns of positive halves order
+            // like signed 16-bit integers, negative sums are negative integers, +inf (0x7c00) lies above
+            typedef short i16x2 __attribute__((ext_vector_type(2)));
+            i16x2 c = __builtin_bit_cast(i16x2, h);
+            c = __builtin_elementwise_max(c, i16x2{0x6600, 0x6600});
+            c = __builtin_elementwise_min(c, i16x2{0x660f, 0x660f});
+            b[i] = __builtin_bit_cast(u32, c);
+        } else {
+            b[i] = __builtin_bit_cast(u32, h);
+        }
     }
     return pack_nibbles8(b);
 }

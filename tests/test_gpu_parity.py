@@ -1110,6 +1110,36 @@ def test_decode_shapes_bit_exact(m, k, n):
     assert np.array_equal(bits(y[:, cols].cpu().numpy()), bits(want))
 
 
+@pytest.mark.parametrize("m,k,n", [(40, 28672, 8192), (53, 28672, 8192), (64, 28672, 8192), (48, 16384, 8192), (64, 16384, 8160),
+                                   (40, 28608, 8192), (64, 8192, 8192), (39, 28672, 8192)])
+def test_decode_many_tokens_against_a_narrow_weight_with_and_without_scratch(m, k, n):
+    """40..64 tokens against a weight with few rows and a long K (70B down_proj): with scratch from the caller the
+    shared-token kernel runs with K sliced across workgroups and a second kernel adds the slices' int32 slabs; without
+    it the barrier-free kernel runs.  Both bit-exact against the oracle and each other -- whole and ragged K stages,
+    a last block of rows that is partial, and shapes just outside the rule (a shorter K, one token fewer), with and
+    without bias."""
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(0, 256, (m, k // 2), dtype=np.uint8)
+    w = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    a[0, :], w[0, :] = 0x88, 0x88                                  # the largest possible sum: 64 k
+    sa = (np.abs(rng.standard_normal(m)) * 0.2 + 0.01).astype(F16)
+    sw = (np.abs(rng.standard_normal(n)) * 0.01 + 0.001).astype(F16)
+    bias = rng.standard_normal(n).astype(F16)
+    ga, gw, gsa, gsw, gb = gpu(a), gpu(w), gpu(sa), gpu(sw), gpu(bias)
+    L, st = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    ws_bytes = L.qr_workspace_bytes(m, n, k)
+    assert (ws_bytes > 0) == (k >= 16384 and m >= 40)
+    cols = np.concatenate([np.arange(0, n, 7), [n - 1]])
+    for b, nb in ((gb, bias), (None, None)):
+        y = quarot_amd.linear_i4(ga, gsa, gw, gsw, b)              # passes the scratch the library asks for
+        plain = torch.empty_like(y)
+        _lib.check(L.qr_linear_i4_f16(ga.data_ptr(), gsa.data_ptr(), gw.data_ptr(), gsw.data_ptr(),
+                                      0 if b is None else b.data_ptr(), m, n, k, plain.data_ptr(), st))
+        assert torch.equal(y, plain)
+        want = o.linear4bit(a, sa, w[cols], sw[cols], None if nb is None else nb[cols])
+        assert np.array_equal(bits(y[:, cols].cpu().numpy()), bits(want))
+
+
 def test_linear4bit_sequential_is_one_call_with_the_same_results_and_state_dict():
     """Linear4bitSequential against torch.nn.Sequential of the same modules: identical output bits
     (the same two kernels run), identical state-dict keys, and the oracle on a small case; chains
