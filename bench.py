@@ -78,7 +78,7 @@ for _t in (1, 8, 32, 64):
     WORKLOADS[f"c4m{_t}"] = (_t, 28672, 8192, "had")      # decode, 70B down_proj
     WORKLOADS[f"c4g{_t}"] = (_t, 8192, 57344, "quant")    # decode, 70B gate_up
 PER_CONFIG = ["c1", "c2_fp32had", "c3", "c4g1", "c4g8", "c4g32", "c4g64", "c4m1", "c4m8", "c4m32", "c4m64", "c5", "c6", "b13v", "b70v", "b13d", "b70d",
-              "c2_fp6", "c3_fp6", "b13v_fp6", "b70v_fp6", "b13d_fp6", "b70d_fp6"]
+              "c2_fp6", "c3_fp6"]
 INT8_MFMA_PEAK_TOPS = 5000.0     # MI355X dense int8, published
 FP6_MFMA_PEAK_TOPS = 10100.0     # MI355X dense fp6, published (the opt-in exact int4 GEMM on 6-bit operands)
 HBM_PEAK_GBS = 8000.0
@@ -88,12 +88,13 @@ HBM_PEAK_GBS = 8000.0
 # calibration ("traffic_scale: fetch=<factor> write=<factor>").
 PROFILE_OF = {
     "c1": "gemm_spk_c1_q_proj_7b.txt", "c1n": "rmsnorm_quant_rows_c1n_q_proj_7b.txt",
-    "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt", "c2": "gemm_spk_and_hadamard_m64q_c2_down_proj_7b.txt",
+    "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt", "c2": "gemm_spk_and_hadamard_m64r_c2_down_proj_7b.txt",
+    "c2_fp32had": "gemm_spk_and_hadamard_m64_fp32_c2_down_proj_7b.txt",
     "c3": "gemm_sp256_c3_prefill_layer_set_32768_tokens.txt",
     "c4g8": "decode_xs_c4g8_decode_8_tokens_70b_gate_up.txt", "c4g32": "decode_xs_c4g32_decode_32_tokens_70b_gate_up.txt",
     "c4g64": "decode_xs_c4g64_decode_64_tokens_70b_gate_up.txt", "c4m1": "gemv_i4_c4m1_decode_70b_down_proj.txt",
     "c4m8": "decode_i4_c4m8_decode_8_tokens_70b_down_proj.txt", "c4m32": "decode_i4_c4m32_decode_32_tokens_70b_down_proj.txt",
-    "c4m64": "decode_i4_c4m64_decode_64_tokens_70b_down_proj.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
+    "c4m64": "decode_xs_sliced_c4m64_decode_64_tokens_70b_down_proj.txt", "c5": "kv_quant_c5_kv_cache_32x4096x8x128.txt",
     "c6": "paged_decode_i4_c6_decode_attention_32x4096x8x128.txt",
     "b13v": "gemm_sp256_b13v_2048x5120x5120.txt", "b70v": "gemm_sp256_b70v_2048x8192x8192.txt",
     "b13d": "gemm_sp256_b13d_2048x13824x5120.txt", "b70d": "gemm_sp256_b70d_2048x28672x8192.txt",
@@ -257,7 +258,7 @@ def mfma_ceiling(seconds):
     return res
 
 
-def gemm_kernel_name(m, n):
+def gemm_kernel_name(m, n, k=0):
     t256 = ((m + 255) // 256) * ((n + 255) // 256)
     t128 = ((m + 127) // 128) * ((n + 255) // 256)
     groups = (n + 31) // 32                # the library's choice: enough groups of 32 rows to give every CU a workgroup
@@ -265,6 +266,8 @@ def gemm_kernel_name(m, n):
     if m == 1 or (m <= 4 and not xs):
         return "gemv_i4_kernel"
     if m <= 64:
+        if not xs and m >= 40 and k >= 16384:   # narrow weight, many tokens, long K: K sliced across workgroups + slab sum
+            return "decode_xs_kernel (K sliced) + dequant_slabs_kernel"
         return "decode_xs_kernel" if xs else "decode_i4_kernel"
     if t128 >= 128:         # the library's choice between its pipelined kernels, by rounds of tiles (256-, 192- or 128-row)
         t192 = ((m + 191) // 192) * ((n + 255) // 256)
@@ -384,7 +387,7 @@ class LinearWorkload:
         return n * k / 2 + m * k / 2 + 2 * m + 2 * n + 2 * m * n
 
     def rooflines(self, front_ms, gemm_ms):
-        kern = "gemm_f6_kernel" if self.fp6 else gemm_kernel_name(self.m, self.n)
+        kern = "gemm_f6_kernel" if self.fp6 else gemm_kernel_name(self.m, self.n, self.k)
         if self.fp6:
             g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": FP6_MFMA_PEAK_TOPS, "unit": "TOP/s",
                  "convert_kernel_ms": round(self.convert_ms, 5)}
