@@ -116,10 +116,13 @@ def traffic_from_profile(workload, kernel):
     sc = re.search(r"traffic_scale:\s*fetch=([\d.]+)\s+write=([\d.]+)", cal)
     if not sc:
         return None, None
+    kib, seen = 0.0, set()                       # a dominant "kernel" of two launches (K-sliced decode) sums both
     for m in re.finditer(r"traffic_kib:\s*kernel=(\S+)\s+fetch=([\d.]+)\s+write=([\d.]+)", text):
-        if m.group(1) in kernel:
-            kib = float(m.group(2)) * float(sc.group(1)) + float(m.group(3)) * float(sc.group(2))
-            return round(kib * 1024), f"profiles/{name}"
+        if m.group(1) in kernel and m.group(1) not in seen:
+            seen.add(m.group(1))
+            kib += float(m.group(2)) * float(sc.group(1)) + float(m.group(3)) * float(sc.group(2))
+    if seen:
+        return round(kib * 1024), f"profiles/{name}"
     return None, None
 
 
