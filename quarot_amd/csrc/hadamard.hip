@@ -1355,15 +1355,20 @@ __global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard
 //     lies entirely beyond it is skipped.
 // TPW: how many of this wave's tiles (rows (wave + 4 i) 16 .. + 15 of hadK) lie inside hadK, at least in part;
 // only the last of them can be partial.  (A function of the wave so that every loop below is free of branches.)
-template <int KS2, int TPW, int CHUNKS>
+// MODE32: the fp32-precision staging of hadamard_m64_kernel<true, ..> -- T = X . H_64 * scale is kept as an fp16 hi and an
+// fp16 lo plane (hi = fp16(T), lo = fp16(T - hi)), every product of the hadK stage is a hi and a lo matrix instruction
+// in that order, and the result is rounded to fp16 once; hadK is then an fp32 table, or null for a power-of-two row,
+// whose outer factor is the Sylvester matrix of order K (generated).
+template <bool MODE32, int KS2, int TPW, int CHUNKS>
 __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, int64_t rows, int n, int K,
-                                                   const f16* __restrict__ hadK, float scale, float clip,
+                                                   const void* __restrict__ hadK, float scale, float clip,
                                                    u32* __restrict__ q, f16* __restrict__ scales, f32x4* smem_raw, u32* red) {
     constexpr int CT = 4, NT = 2 * KS2;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4;
     const int nchunks = n >> 3;
     u32x2* Tl = (u32x2*)smem_raw;                                      // [CT][NT][64 lanes]
+    u32x2* Tlo = Tl + CT * NT * 64;                                    // lo plane (fp32-precision mode)
 
     // Sylvester fragments of hadamard_m64_kernel: one base per parity of the column tile; where that kernel takes a
     // negated fragment (second contraction step, column tiles 2 and 3) the OTHER operand is negated here instead
@@ -1400,7 +1405,69 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
     // each lane then picks its 8-byte pieces from there.  Loading them straight from memory -- a lane's pieces lie 32
     // bytes apart, every workgroup of the grid asks at the same moment -- cost 3 of the 23 us of a 2048-row launch.
     f16x8 hf[TPW][KS2];
-    {
+    if (MODE32 && hadK == nullptr) {
+        // power-of-two row: the outer factor is the Sylvester matrix of order K, generated in place
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int hr = (wave + 4 * i) * 16 + l16;
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const int hc = ks * 32 + hh * 16 + g * 4;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        hf[i][ks][hh * 4 + e] = (hr < K && hc < K) ? ((__builtin_popcount(hr & (hc + e)) & 1) ? (f16)-1.0f : (f16)1.0f) : (f16)0.0f;
+                }
+        }
+        u32x4* stage = (u32x4*)smem_raw;
+        for (int i = tid; i < 2 * CT * NT * 32; i += HT) stage[i] = u32x4{0, 0, 0, 0};
+    } else if constexpr (MODE32) {
+        // fp32 table: the same staging as below with the pieces converted on their way into LDS (+-1: exact), 64 rows
+        // of the table at a time, the next run's loads in flight while the current one is converted and picked up
+        u32x2* stage = (u32x2*)smem_raw;                               // fp16 [64][K] as 8-byte pieces
+        const f32x4* src = (const f32x4*)hadK;
+        const int total = (K * K) >> 2;                                // 16-byte pieces (four coefficients) of hadK
+        const int count = (64 * K) >> 2;                               // ... of 64 rows: at most 2 KS2 per thread
+        constexpr int P = 2 * KS2;
+        f32x4 hk[2][P];
+        auto fetch = [&](int i, int b) {
+#pragma unroll
+            for (int j = 0; j < P; ++j) {
+                const int pc = tid + j * HT, at = i * count + pc;
+                hk[b][j] = src[pc < count && at < total ? at : 0];
+            }
+        };
+        fetch(0, 0);
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            if (i + 1 < CHUNKS) fetch(i + 1, (i + 1) & 1);
+#pragma unroll
+            for (int j = 0; j < P; ++j) {
+                const int pc = tid + j * HT;
+                const f32x4 w = hk[i & 1][j];
+                if (pc < count) stage[pc] = u32x2{cvt_f16x2(w[0], w[1]), cvt_f16x2(w[2], w[3])};
+            }
+            __syncthreads();
+            if (i < TPW) {
+                const int hr = (wave + 4 * i) * 16 + l16;
+#pragma unroll
+                for (int ks = 0; ks < KS2; ++ks)
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh) {
+                        const int hc = ks * 32 + hh * 16 + g * 4;
+                        const bool ok = hr < K && hc < K;
+                        f16x4 v = *(const f16x4*)((const f16*)stage + (ok ? (wave * 16 + l16) * K + hc : 0));
+                        if (!ok) v = f16x4{(f16)0, (f16)0, (f16)0, (f16)0};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) hf[i][ks][hh * 4 + e] = v[e];
+                    }
+            }
+            __syncthreads();
+        }
+        u32x4* clr = (u32x4*)smem_raw;
+        for (int i = tid; i < 2 * CT * NT * 32; i += HT) clr[i] = u32x4{0, 0, 0, 0};
+    } else {
         u32x4* stage = (u32x4*)smem_raw;
         const u32x4* src = (const u32x4*)hadK;
         const int total = (K * K) >> 3;                                // 16-byte pieces of hadK (orders are multiples of 4)
@@ -1466,8 +1533,22 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a0), sb[ct & 1], acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, (ct >> 1) ? a1n : a1), sb[ct & 1], acc, 0, 0, 0);
                     u32x2 hi;
-                    hi[0] = narrow_f16x2(acc[0] * scale, acc[1] * scale);
-                    hi[1] = narrow_f16x2(acc[2] * scale, acc[3] * scale);
+                    if constexpr (MODE32) {
+                        float tv[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) tv[e] = acc[e] * scale;
+                        u32x2 lo;
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            hi[e] = narrow_f16x2(tv[2 * e], tv[2 * e + 1]);
+                            const f16x2 h = as_f16x2(hi[e]);
+                            lo[e] = narrow_f16x2(tv[2 * e] - (float)h[0], tv[2 * e + 1] - (float)h[1]);
+                        }
+                        Tlo[(ct * NT + t) * 64 + lane] = lo;
+                    } else {
+                        hi[0] = narrow_f16x2(acc[0] * scale, acc[1] * scale);
+                        hi[1] = narrow_f16x2(acc[2] * scale, acc[3] * scale);
+                    }
                     Tl[(ct * NT + t) * 64 + lane] = hi;
                 }
             }
@@ -1485,33 +1566,34 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
         for (int ct = 0; ct < CT; ++ct) {
             // fragments of T one contraction step ahead of their use (8 registers; a whole column tile's set ahead
             // was no faster, and three workgroups per CU, which these registers would allow, spilled and lost 15 %)
-            auto frag = [&](int ks) {
-                const u32x2 p0 = Tl[(ct * NT + 2 * ks) * 64 + lane], p1 = Tl[(ct * NT + 2 * ks + 1) * 64 + lane];
+            auto frag = [&](const u32x2* plane, int ks) {
+                const u32x2 p0 = plane[(ct * NT + 2 * ks) * 64 + lane], p1 = plane[(ct * NT + 2 * ks + 1) * 64 + lane];
                 return u32x4{p0[0], p0[1], p1[0], p1[1]};
             };
             f32x4 acc[TPW];
 #pragma unroll
             for (int i = 0; i < TPW; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-            u32x4 th = frag(0);
+            u32x4 th = frag(Tl, 0), tl = MODE32 ? frag(Tlo, 0) : u32x4{0, 0, 0, 0};
 #pragma unroll
             for (int ks = 0; ks < KS2; ++ks) {
                 __builtin_amdgcn_sched_barrier(0);           // (keeps the scheduler from hoisting every read to the top)
-                const u32x4 cur = th;
-                if (ks + 1 < KS2) th = frag(ks + 1);
+                const u32x4 cur = th, curl = tl;
+                if (ks + 1 < KS2) {
+                    th = frag(Tl, ks + 1);
+                    if constexpr (MODE32) tl = frag(Tlo, ks + 1);
+                }
 #pragma unroll
-                for (int i = 0; i < TPW; ++i)
+                for (int i = 0; i < TPW; ++i) {
                     acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, cur), hf[i][ks], acc[i], 0, 0, 0);
+                    if constexpr (MODE32)
+                        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, curl), hf[i][ks], acc[i], 0, 0, 0);
+                }
             }
             if (ct == 0) probe = acc[0][0];
 #pragma unroll
             for (int i = 0; i < TPW; ++i) {
-#ifdef QR_OLDCVT
-                yv[i][ct][0] = narrow_f16x2(acc[i][0], acc[i][1]);
-                yv[i][ct][1] = narrow_f16x2(acc[i][2], acc[i][3]);
-#else
                 yv[i][ct][0] = cvt_f16x2(acc[i][0], acc[i][1]);
                 yv[i][ct][1] = cvt_f16x2(acc[i][2], acc[i][3]);
-#endif
                 // (rows of hadK beyond its order are zero fragments: their outputs are 0, or NaN from 0 . inf, which
                 // the maximum instruction drops)
                 mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[i][0])), __builtin_fabsf(acc[i][1]));
@@ -1602,17 +1684,17 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
     }
 }
 
-template <int KS2>
+template <bool MODE32, int KS2>
 __global__ __launch_bounds__(HT, 2) void hadamard_m64r_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
-                                                            const f16* __restrict__ hadK, float scale, float clip,
+                                                            const void* __restrict__ hadK, float scale, float clip,
                                                             u32* __restrict__ q, f16* __restrict__ scales) {
     constexpr int NT = 2 * KS2, TPW = (NT + 3) / 4;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[HT / QR_WAVE];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // (both forms pass the same barriers: two per 64 rows of hadK and one more before the loop, two per row)
-    if ((wave + 4 * (TPW - 1)) * 16 < K) hadamard_m64r_rows<KS2, TPW, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
-    else hadamard_m64r_rows<KS2, TPW - 1, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
+    if ((wave + 4 * (TPW - 1)) * 16 < K) hadamard_m64r_rows<MODE32, KS2, TPW, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
+    else hadamard_m64r_rows<MODE32, KS2, TPW - 1, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
 }
 
 // A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
@@ -1661,16 +1743,20 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
         const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
-        if (!MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0 && ((uintptr_t)hadK & 15) == 0) {
-            // fused, fp16 staging, no copy of the transformed rows wanted: the lean kernel (T alone in LDS)
-            const size_t ldsq = (size_t)4096 * KS2;
+        if (QUANT && y == nullptr && (MODE32 || hadK != nullptr) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)hadK & 15) == 0) {
+            // fused, no copy of the transformed rows wanted: the lean kernel (T alone in LDS; two planes of it in the
+            // fp32-precision mode)
+            const size_t ldsq = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2;
 #define QR_M64Q(KS)                                                                                                    \
     do {                                                                                                               \
-        auto kern = hadamard_m64r_kernel<KS>;                                                                          \
-        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                                     \
+        auto kern = hadamard_m64r_kernel<MODE32, KS>;                                                                  \
+        if (ldsq > 48 * 1024) {                                                                                        \
+            hipError_t e = qr_allow_dynamic_lds((const void*)kern, ldsq);                                              \
+            if (e != hipSuccess) return (int)e;                                                                        \
+        }                                                                                                              \
+        const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                  \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
-        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, (const f16*)hadK, scale, clip, (u32*)q,    \
-                                                 (f16*)scales);                                                        \
+        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, hadK, scale, clip, (u32*)q, (f16*)scales); \
     } while (0)
             // (orders of 64 and more among the reference's tables: 108, 140, 156, 172)
             if (KS2 >= 4) {

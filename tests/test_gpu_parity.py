@@ -677,6 +677,43 @@ def test_fused_hadamard_quantize_lean_kernel_rows_of_every_kind(n):
     assert torch.equal(one.quantized_x, p.quantized_x[5:6])
 
 
+@pytest.mark.parametrize("n", [11008, 8960, 6912, 8192])
+@pytest.mark.parametrize("clip", [1.0, 0.9])
+def test_fused_hadamard_quantize_lean_kernel_in_fp32_precision(n, clip):
+    """force_fp32=True without the copy of the transformed rows: the lean m = 64 kernel with T kept as fp16 hi + lo planes
+    (tables of order 108 .. 172 staged through LDS from their fp32 form; 8192 = 128 x 64 with the generated Sylvester
+    outer factor).  Same rows of every kind as above; codes and scales must equal those of the kernels that also
+    return the rows (same arithmetic in the same order), whose codes are checked against the oracle on those rows,
+    and the rows against the oracle's fp32 transform."""
+    rows = 1100
+    x = synth_x(rows, n, seed=n + 11)
+    x[3, 17] = np.inf
+    x[700, 5] = np.nan
+    x[701] = 0
+    x[1099] = 0
+    x[900, 9] = 60000.0
+    x[44] *= F16(1e-4)
+    x[0, :] = 0
+    xg = gpu(x)
+    mod = quarot_amd.nn.OnlineHadamardQuantizer(n, force_fp32=True, input_clip_ratio=clip).cuda()
+    p = mod(xg)
+    p2, y = quarot_amd.hadamard_quantize(xg, mod.had_rem_dim, mod.rem_dim, clip, force_fp32=True, return_transformed=True)
+    assert torch.equal(p.quantized_x, p2.quantized_x)
+    assert np.array_equal(bits(p.scales_x.cpu().numpy()), bits(p2.scales_x.cpu().numpy()))
+    with np.errstate(all="ignore"):
+        wq, ws = o.quantizer(y.cpu().numpy(), clip)
+    assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
+    got_s = p.scales_x.cpu().numpy().reshape(-1)
+    nan = np.isnan(ws)
+    assert np.array_equal(np.isnan(got_s), nan) and np.array_equal(bits(got_s[~nan]), bits(ws[~nan]))
+    fin = np.isfinite(x.astype(np.float32)).all(axis=1)
+    sample = np.flatnonzero(fin)[::97]
+    with np.errstate(all="ignore"):
+        assert close(y.cpu().numpy()[sample], o.online_hadamard(x[sample], force_fp32=True))
+    one = mod(xg[5:6])
+    assert torch.equal(one.quantized_x, p.quantized_x[5:6])
+
+
 @pytest.mark.parametrize("shape", [(5, 64), (9, 4096), (7, 5120), (3, 8192), (4, 11008), (2, 32768), (6, 24), (3, 100)])
 @pytest.mark.parametrize("clip", [1.0, 0.9])
 def test_fused_rmsnorm_quantize(shape, clip):
