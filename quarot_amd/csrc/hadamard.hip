@@ -2045,12 +2045,22 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
             const float s = (float)sh;
             const bool lean = fast_quant_ok(mx, s);
             const FastRecip fq = make_fast_recip(lean ? s : 1.0f);
-            const bool fast = scale_fast_ok(s);
-            const float rs = fast ? 1.0f / s : 0.0f;
-            for (int c = tid; c < nchunks; c += BT) {
-                const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
-                q[row * (int64_t)nchunks + c] = lean ? sym_codes8_fast(h, fq) : sym_codes8(h, s, rs, fast);
-                if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+            // (three loops rather than a choice per chunk: the forms differ in length, the choice is the row's)
+            auto codes_of_row = [&](auto form) {
+                for (int c = tid; c < nchunks; c += BT) {
+                    const u32x4 h = *(const u32x4*)(Yl + ((c * 8) >> LOG2M) * YS + ((c * 8) & (M_ - 1)));
+                    q[row * (int64_t)nchunks + c] = form(h);
+                    if (y) __builtin_nontemporal_store(h, (u32x4*)(y + row * (int64_t)n) + c);
+                }
+            };
+            if (lean && clamp_cannot_act(clip, s)) {
+                codes_of_row([&](u32x4 h) { return sym_codes8_fast<false>(h, fq); });
+            } else if (lean) {
+                codes_of_row([&](u32x4 h) { return sym_codes8_fast<true>(h, fq); });
+            } else {
+                const bool fast = scale_fast_ok(s);
+                const float rs = fast ? 1.0f / s : 0.0f;
+                codes_of_row([&](u32x4 h) { return sym_codes8(h, s, rs, fast); });
             }
         } else {
             for (int c = tid; c < nchunks; c += BT) {

@@ -241,9 +241,9 @@ __device__ __forceinline__ u32 sym_codes8(u32x4 v, float s, float rs, bool fast_
 // reciprocal must be the correctly rounded one).  Why it works: a quotient of two fp16 numbers keeps
 // a relative distance above 2^-23 from every fp16 rounding boundary (see sym_code), and the two
 // roundings here (r, then the product) stay within 2^-23.
-// Clamping to [-8, 7] before the conversion commutes with it (rounding is monotone and -8, 7 are
-// representable).  Adding 1536 (ulp 1 in [1024, 2048)) in fp16 then rounds to the nearest integer,
-// ties to even, and leaves the two's-complement code in the low four mantissa bits.
+// Adding 1536 (ulp 1 in [1024, 2048)) in fp16 rounds to the nearest integer, ties to even, and leaves the
+// two's-complement code in the low four mantissa bits; the clamp to [-8, 7] follows on the bit patterns
+// (sym_pair_fast), which commutes with the rounding (monotone, and -8, 7 are representable).
 struct FastRecip {
     float r;
 };
@@ -290,24 +290,19 @@ __device__ __forceinline__ u32 sym_pair_fast(u32 w, FastRecip f) {
     b = __builtin_elementwise_min(b, i16x2{0x6607, 0x6607});
     return __builtin_bit_cast(u32, b);
 }
+// 8 fp16 (one 16-byte chunk) -> 8 nibbles, element 0 lowest: four sym_pair_fast and the gather.  CLAMP = false only
+// where clamp_cannot_act() holds for the row.
+template <bool CLAMP = true>
 __device__ __forceinline__ u32 sym_codes8_fast(u32x4 v, FastRecip f) {
     u32 b[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float x0 = (float)f16_from_bits((unsigned short)(v[i] & 0xffffu));
-        const float x1 = (float)f16_from_bits((unsigned short)(v[i] >> 16));
-        // x * r written as fma(x, r, 0): the same value (a zero of either sign ends as code 0), and the
-        // instruction takes the half straight from the packed word (v_fma_mix_f32) instead of converting first
-        float q0 = __builtin_fmaf(x0, f.r, 0.0f);
-        float q1 = __builtin_fmaf(x1, f.r, 0.0f);
-        q0 = __builtin_amdgcn_fmed3f(q0, -8.0f, 7.0f);
-        q1 = __builtin_amdgcn_fmed3f(q1, -8.0f, 7.0f);
-        f16x2 h = {(f16)q0, (f16)q1};
-        h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
-        b[i] = __builtin_bit_cast(u32, h);
-    }
+    for (int i = 0; i < 4; ++i) b[i] = sym_pair_fast<CLAMP>(v[i], f);
     return pack_nibbles8(b);
 }
+// A scale that the quantiser itself derived from the row's largest magnitude with clip >= 1 keeps every quotient
+// inside the code range when it is a normal fp16 number: |x| <= amax and s >= (amax / 7) (1 - 2^-11)^2 give
+// |x / s| < 7.5, which rounds to at most 7 (a subnormal scale can be several per cent off: it keeps the clamp).
+__device__ __forceinline__ bool clamp_cannot_act(float clip, float s) { return clip >= 1.0f && s >= 6.103515625e-05f; }
 // amax bits below 0x7c00 <=> every element of the row is finite
 __device__ __forceinline__ bool fast_quant_ok(u32 amax_bits, float s) {
     const float a = __builtin_fabsf(s);

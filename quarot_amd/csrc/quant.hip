@@ -21,22 +21,23 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
         int c = threadIdx.x + i * QT;
         v[i] = c < cols8 ? __builtin_nontemporal_load(xr + c) : u32x4{0, 0, 0, 0};
     }
+    // the row's largest magnitude: it gives the scale, and (also with a given scale) tells whether the row is all
+    // finite, i.e. whether the lean codes apply
     float s;
-    u32 m = 0x7c00u;                 // "not known to be finite" unless the abs-max says otherwise
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        u32 mi = absmax_bits8(v[i]);
+        m = m > mi ? m : mi;
+    }
+    m = wave_max_u32(m);
+    if ((threadIdx.x & (QR_WAVE - 1)) == 0) red[threadIdx.x / QR_WAVE] = m;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
     if (GIVEN_SCALE) {
         s = (float)scale_in[row];
     } else {
-        m = 0;
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            u32 mi = absmax_bits8(v[i]);
-            m = m > mi ? m : mi;
-        }
-        m = wave_max_u32(m);
-        if ((threadIdx.x & (QR_WAVE - 1)) == 0) red[threadIdx.x / QR_WAVE] = m;
-        __syncthreads();
-#pragma unroll
-        for (int w = 0; w < QT / QR_WAVE; ++w) m = m > red[w] ? m : red[w];
         f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
         if (threadIdx.x == 0) scale_out[row] = sh;
         s = (float)sh;
@@ -44,10 +45,18 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
     u32* qr = q + row * (int64_t)cols8;
     if (fast_quant_ok(m, s)) {       // workgroup-uniform
         const FastRecip fr = make_fast_recip(s);
+        if (!GIVEN_SCALE && clamp_cannot_act(clip, s)) {
 #pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            int c = threadIdx.x + i * QT;
-            if (c < cols8) qr[c] = sym_codes8_fast(v[i], fr);
+            for (int i = 0; i < NV; ++i) {
+                int c = threadIdx.x + i * QT;
+                if (c < cols8) qr[c] = sym_codes8_fast<false>(v[i], fr);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                int c = threadIdx.x + i * QT;
+                if (c < cols8) qr[c] = sym_codes8_fast<true>(v[i], fr);
+            }
         }
         return;
     }
