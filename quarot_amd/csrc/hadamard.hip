@@ -1842,8 +1842,8 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
 //              second operand (no exchange between lanes); T is split into fp16 hi + lo (two MFMAs), so
 //              the result has fp32 accuracy and is rounded to fp16 once, after the scale, as in the
 //              butterfly form;
-//     a wave takes four k and one half of c', and packs its four results per position into one 8-byte
-//     LDS write in the fragment order of the hadK stage;
+//     a wave takes two k and both halves of c' (every byte of the row is loaded once), and packs its two results
+//     per position into one 4-byte LDS write in the fragment order of the hadK stage;
 //   m = 512 with butterflies in registers (8 values per chunk, 64 lanes: 3 + 6 levels, no LDS), scattered
 //     into the same order as 2-byte writes.
 // The hadK factor then runs on the matrix cores as in hadamard_mm_kernel (T^T as first operand, hadK
@@ -1869,18 +1869,20 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
     const int l16 = lane & 15, g = lane >> 4;
     const int nchunks = n >> 3;
 
-    // m = 1024: unit (wave / 2) = four k, wave % 2 = the half of c'; Sylvester fragments of both stages
-    constexpr int XL = CPL == 2 ? 8 : SPW * CPL;
-    const int unit = wave >> 1, cth = wave & 1;
-    const bool works = CPL == 2 && unit * 4 < K;
+    // m = 1024: a wave takes the two segments k = 2 wave, 2 wave + 1 and both halves of c', so that every byte of the
+    // row is requested once (a CU's vector memory path takes a row in at ~60 GB/s: with the halves of c' on different
+    // waves, each loading the unit's segments, a one-row launch waited 4.3 us for 130 KB); Sylvester fragments of
+    // both stages
+    constexpr int XL = CPL == 2 ? 4 : SPW * CPL;
+    const bool works = CPL == 2 && wave * 2 < K;
     u32x4 raw[XL];
     auto request = [&](int64_t row) {
         if (CPL == 2) {
 #pragma unroll
-            for (int ai = 0; ai < 4; ++ai)          // (waves beyond the last unit repeat unit 0's loads and drop them: no branch)
+            for (int sg = 0; sg < 2; ++sg)          // (waves beyond the last pair repeat wave 0's loads and drop them: no branch)
 #pragma unroll
                 for (int bt = 0; bt < 2; ++bt)
-                    raw[ai * 2 + bt] = *((const u32x4*)(x + row * (int64_t)n) + ((works ? unit : 0) * 4 + ai) * 128 + bt * 64 + l16 * 4 + g);
+                    raw[sg * 2 + bt] = *((const u32x4*)(x + row * (int64_t)n) + ((works ? wave : 0) * 2 + sg) * 128 + bt * 64 + l16 * 4 + g);
             return;
         }
 #pragma unroll
@@ -1894,11 +1896,12 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
     };
     int64_t row = blockIdx.x;
     if (row < rows) request(row);           // in flight while the fragments are made and T is cleared
-    f16x8 ha, hb[2];
+    f16x8 ha[2], hb[2];
     if (CPL == 2) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) {
-            ha[t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+#pragma unroll
+            for (int cth = 0; cth < 2; ++cth) ha[cth][t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
             const int b = 16 * (t >> 2) + 4 * g + (t & 3);
 #pragma unroll
             for (int bt = 0; bt < 2; ++bt) hb[bt][t] = (__builtin_popcount(b & (bt * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
@@ -1926,45 +1929,46 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
         // ---- phase 1: the power-of-two factor of every segment, results in fragment order in LDS
         if (CPL == 2) {
             if (works) {
-                u32 o[4][2][2];                          // [k of the unit][b' tile][pair of e]: fp16 pairs
 #pragma unroll
-                for (int ai = 0; ai < 4; ++ai) {
-                    // T = hi + lo, both fp16, as packed pairs (the difference is exact in fp32, so one rounding each)
-                    typedef float f32x2_t __attribute__((ext_vector_type(2)));
-                    u32x4 whi, wlo;
+                for (int cth = 0; cth < 2; ++cth) {
+                    u32 o[2][2][2];                      // [segment of the pair][b' tile][pair of e]: fp16 pairs
 #pragma unroll
-                    for (int bt = 0; bt < 2; ++bt) {
-                        const f32x4 da = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, raw[ai * 2 + bt]), ha,
-                                                                              f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    for (int sg = 0; sg < 2; ++sg) {
+                        // T = hi + lo, both fp16, as packed pairs (the difference is exact in fp32, so one rounding each)
+                        typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                        u32x4 whi, wlo;
 #pragma unroll
-                        for (int pr = 0; pr < 2; ++pr) {
-                            const f16x2 hi = __builtin_convertvector(f32x2_t{da[2 * pr], da[2 * pr + 1]}, f16x2);
-                            const f16x2 lo = __builtin_convertvector(f32x2_t{da[2 * pr] - (float)hi[0], da[2 * pr + 1] - (float)hi[1]}, f16x2);
-                            whi[bt * 2 + pr] = __builtin_bit_cast(u32, hi);
-                            wlo[bt * 2 + pr] = __builtin_bit_cast(u32, lo);
+                        for (int bt = 0; bt < 2; ++bt) {
+                            const f32x4 da = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, raw[sg * 2 + bt]), ha[cth],
+                                                                                  f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                            for (int pr = 0; pr < 2; ++pr) {
+                                const f16x2 hi = __builtin_convertvector(f32x2_t{da[2 * pr], da[2 * pr + 1]}, f16x2);
+                                const f16x2 lo = __builtin_convertvector(f32x2_t{da[2 * pr] - (float)hi[0], da[2 * pr + 1] - (float)hi[1]}, f16x2);
+                                whi[bt * 2 + pr] = __builtin_bit_cast(u32, hi);
+                                wlo[bt * 2 + pr] = __builtin_bit_cast(u32, lo);
+                            }
+                        }
+                        const f16x8 thi = __builtin_bit_cast(f16x8, whi), tlo = __builtin_bit_cast(f16x8, wlo);
+#pragma unroll
+                        for (int bt = 0; bt < 2; ++bt) {
+                            f32x4 db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], thi, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                            db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], tlo, db, 0, 0, 0);
+                            o[sg][bt][0] = narrow_f16x2(db[0] * scale, db[1] * scale);
+                            o[sg][bt][1] = narrow_f16x2(db[2] * scale, db[3] * scale);
                         }
                     }
-                    const f16x8 thi = __builtin_bit_cast(f16x8, whi), tlo = __builtin_bit_cast(f16x8, wlo);
+                    // position (b' = 16 bt + 4 g + e, c' = 16 cth + l16) = column tile 2 b' + cth, column l16; the pair's
+                    // two k are one 32-bit word of that position's fragment (k = 2 wave, 2 wave + 1: k-group wave / 4)
+                    u32* const dst = (u32*)(Tl + ((wave >> 2) * CT + cth) * TS + l16) + (wave & 3);
 #pragma unroll
-                    for (int bt = 0; bt < 2; ++bt) {
-                        f32x4 db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], thi, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                        db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], tlo, db, 0, 0, 0);
-                        o[ai][bt][0] = narrow_f16x2(db[0] * scale, db[1] * scale);
-                        o[ai][bt][1] = narrow_f16x2(db[2] * scale, db[3] * scale);
-                    }
+                    for (int bt = 0; bt < 2; ++bt)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const u32 sel = (e & 1) ? 0x07060302u : 0x05040100u;      // high or low halves of two dwords
+                            dst[(2 * (16 * bt + 4 * g + e)) * TS * 4] = __builtin_amdgcn_perm(o[1][bt][e >> 1], o[0][bt][e >> 1], sel);
+                        }
                 }
-                // position (b' = 16 bt + 4 g + e, c' = 16 cth + l16) = column tile 2 b' + cth, column l16
-                u32x2* const dst = (u32x2*)(Tl + ((unit >> 1) * CT + cth) * TS + l16) + (unit & 1);
-#pragma unroll
-                for (int bt = 0; bt < 2; ++bt)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const u32 sel = (e & 1) ? 0x07060302u : 0x05040100u;      // high or low halves of two dwords
-                        u32x2 v;
-                        v[0] = __builtin_amdgcn_perm(o[1][bt][e >> 1], o[0][bt][e >> 1], sel);
-                        v[1] = __builtin_amdgcn_perm(o[3][bt][e >> 1], o[2][bt][e >> 1], sel);
-                        dst[(2 * (16 * bt + 4 * g + e)) * TS * 2] = v;
-                    }
             }
         } else {
 #pragma unroll
@@ -2001,6 +2005,100 @@ __global__ __launch_bounds__(1024) void hadamard_bm_kernel(const f16* __restrict
         const int64_t nrow = row + gridDim.x;
         if (nrow < rows) request(nrow);
         __syncthreads();
+        if constexpr (QUANT && CPL == 2) {
+            if (y == nullptr) {
+                // ---- no copy of the transformed row wanted (the decode step, prefill): the results of the hadK stage
+                // stay in registers and become codes there, as in hadamard_m64r_kernel -- same layout: lanes l16 + 16 g
+                // hold, for output row k' = 16 rt + l16, the columns 16 c + 4 g .. + 3 of this wave's four column tiles
+                // (64 consecutive columns of the segment) -- so the row's trip through LDS and the second pass over it
+                // are gone: one barrier (for the row maximum) instead of a barrier, 16-byte reads and a 120-instruction loop
+                bool dval[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) dval[rt] = rt * 16 + l16 < K;
+                f16x8 th4[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) th4[c] = __builtin_bit_cast(f16x8, Tl[(g * CT + wave * 4 + c) * TS + l16]);
+                u32x2 yv[RT][4];
+                float mxf = 0.f, probe = 0.f;
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        const f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(th4[c], hf[rt][0], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        if (c == 0 && rt == 0) probe = acc[0];
+                        yv[rt][c][0] = cvt_f16x2(acc[0], acc[1]);
+                        yv[rt][c][1] = cvt_f16x2(acc[2], acc[3]);
+                        // (rows of hadK beyond its order are zero fragments: their outputs are 0, or NaN from 0 . inf,
+                        // which the maximum instruction drops)
+                        mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[0])), __builtin_fabsf(acc[1]));
+                        mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[2])), __builtin_fabsf(acc[3]));
+                    }
+                // the row's maximum: rounded once (rounding is monotone); an infinity or NaN anywhere in the row reaches
+                // every output, so one output per lane tells, and a wave that sees one takes the exact form (NaN wins)
+                u32 mx = f16_bits((f16)mxf);
+                if (__builtin_amdgcn_ballot_w64(mx >= 0x7c00u || probe != probe) != 0) {
+                    u16x2 m2 = {0, 0};
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(u16x2, dval[rt] ? yv[rt][c][0] & 0x7fff7fffu : 0u));
+                            m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(u16x2, dval[rt] ? yv[rt][c][1] & 0x7fff7fffu : 0u));
+                        }
+                    mx = m2[0] > m2[1] ? m2[0] : m2[1];
+                }
+                mx = wave_max_u32_dpp(mx);
+                if (lane == 0) red[wave] = mx;          // (last read before the barrier that follows the previous row's phase 1)
+                __syncthreads();
+#pragma unroll
+                for (int w = 0; w < NW; ++w) mx = mx > red[w] ? mx : red[w];
+                const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+                if (tid == 0) scales[row] = sh;
+                const float sp = (float)sh;
+                u32 c01[RT], c23[RT];
+                auto codes_from = [&](auto pair) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        u32 b0[4], b1[4];
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            b0[w] = pair(yv[rt][w >> 1][w & 1]);
+                            b1[w] = pair(yv[rt][2 + (w >> 1)][w & 1]);
+                        }
+                        c01[rt] = pack_nibbles8(b0);
+                        c23[rt] = pack_nibbles8(b1);
+                    }
+                };
+                if (fast_quant_ok(mx, sp)) {
+                    const FastRecip fq = make_fast_recip(sp);
+                    if (clamp_cannot_act(clip, sp)) codes_from([&](u32 w) { return sym_pair_fast<false>(w, fq); });
+                    else codes_from([&](u32 w) { return sym_pair_fast<true>(w, fq); });
+                } else {
+                    const bool fs = scale_fast_ok(sp);
+                    const float rs = fs ? 1.0f / sp : 0.0f;
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        c01[rt] = sym_codes8(u32x4{yv[rt][0][0], yv[rt][0][1], yv[rt][1][0], yv[rt][1][1]}, sp, rs, fs);
+                        c23[rt] = sym_codes8(u32x4{yv[rt][2][0], yv[rt][2][1], yv[rt][3][0], yv[rt][3][1]}, sp, rs, fs);
+                    }
+                }
+                // piece (g, c) -> lane c: first the halves of the wave (g and g ^ 2), then neighbouring rows of 16 lanes;
+                // a lane ends with 16 consecutive codes of row k' = 16 rt + l16: columns 64 wave + 16 g ..
+                u32x2* qrow = (u32x2*)(q + row * (int64_t)nchunks);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    const auto s1 = __builtin_amdgcn_permlane32_swap(c01[rt], c23[rt], false, false);
+                    const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);
+                    const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);
+                    const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
+                    const u32x2 outv = {__builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u), __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u)};
+                    if (dval[rt]) qrow[(rt * 16 + l16) * (M_ / 16) + wave * 4 + g] = outv;
+                }
+                // Tl is next written after the next barrier (the one behind the next row's phase 1 comes after these
+                // reads); red[] is next written after that barrier too
+                continue;
+            }
+        }
         // ---- stage 2: Y^T = T^T . hadK^T (the row's largest magnitude is taken on the way: packed unsigned maxima
         // of the fp16 bit patterns without their signs, so that a NaN still wins)
         u16x2 mx2 = {0, 0};
