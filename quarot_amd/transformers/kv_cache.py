@@ -171,13 +171,14 @@ def _decode_workspace_bytes(batch, heads, max_seq_len, device_index=None):
 
 
 def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, max_seq_len=0,
-                    q_hadamard=False):
+                    q_hadamard=False, workspace=None):
     """o[b, h] = softmax(q[b, h] . K^T / sqrt(128)) . V over the int4 cache of sequence b, dequantised in
     registers as float(code) * scale - zero (kv_cache.py:60-67 -> bindings.cpp:118-153).  Writes into `o`
     and returns None, like the reference's binding.  max_seq_len (optional, an upper bound of the
     sequence lengths) lets a small batch be split along the sequence.  q_hadamard: `q` is the
     untransformed query and the kernel applies matmul_had_cuda(q, torch.float16) itself (one launch
-    instead of two)."""
+    instead of two).  workspace: a uint8 tensor on the cache's device to hold the partial states of a split along
+    the sequence; one is allocated per call when it is missing or too small."""
     fn = "batch_decode_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     for name, t in (("o", o), ("q", q)):
@@ -192,7 +193,11 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
     dev = kv_data.device
     with _lib.on_device(dev):
         ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len), dev.index) if max_seq_len else 0
-        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
+        ws = None
+        if ws_bytes:
+            fits = (workspace is not None and workspace.device == dev and workspace.dtype == torch.uint8
+                    and workspace.is_contiguous() and workspace.numel() >= ws_bytes)
+            ws = workspace if fits else torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
         entry = _lib.lib().qr_batch_decode_qhad_i4 if q_hadamard else _lib.lib().qr_batch_decode_i4
         _lib.check(entry(
             o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
@@ -210,7 +215,7 @@ class _AttentionStub(object):
         self.disable_quant = disable_quant
         self.hadamard_dtype = hadamard_dtype
 
-    def forward(self, q, num_kv_heads, attention_kwargs, layer_idx, max_seq_len=0):
+    def forward(self, q, num_kv_heads, attention_kwargs, layer_idx, max_seq_len=0, workspace=None):
         batch_size, q_len, num_qo_heads, head_dim = q.shape
         assert q_len == 1
         q = q.view(batch_size, num_qo_heads, head_dim)
@@ -218,7 +223,8 @@ class _AttentionStub(object):
         if self.hadamard_dtype is not None and not fused:
             q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
         attn_output = torch.empty_like(q)
-        batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len, q_hadamard=fused)
+        batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len, q_hadamard=fused,
+                        workspace=workspace)
         return attn_output.unsqueeze(1)
 
 
@@ -254,6 +260,18 @@ class MultiLayerPagedKVCache4Bit:
 
     def page_cnt_from_length(self, length):
         return (length + self.page_size - 1) // self.page_size
+
+    def _decode_workspace(self, num_heads):
+        """Scratch for decode attention split along the sequence, kept with the cache (every layer of every decode
+        step would otherwise allocate its own): sized for the longer of the current and the maximum length."""
+        dev = self.pages.device
+        with _lib.on_device(dev):
+            need = max((_decode_workspace_bytes(self.batch_size, num_heads, int(n), dev.index)
+                        for n in (self.length, self.max_seq_len) if n), default=0)
+        ws = getattr(self, "_decode_ws", None)
+        if need and (ws is None or ws.numel() < need):
+            ws = self._decode_ws = torch.empty((need,), dtype=torch.uint8, device=dev)
+        return ws
 
     def _ensure_page_cnt_per_batch(self, expected_page_cnt_per_batch):
         if expected_page_cnt_per_batch * self.batch_size <= self.pages.shape[0]:
@@ -303,7 +321,7 @@ class MultiLayerPagedKVCache4Bit:
                               v=value_states.reshape(self.batch_size, num_heads, head_dim).contiguous(), seqlen_indptr=None,
                               layer_idx=layer_idx, hadamard=fused_had)
         return functools.partial(self._stub.forward, num_kv_heads=num_heads, attention_kwargs=specs, layer_idx=layer_idx,
-                                 max_seq_len=self.length)
+                                 max_seq_len=self.length, workspace=self._decode_workspace(num_heads))
 
     def get_cache_specs_for_flash_infer(self, attention_mask):
         """Page tables of the current state (kv_cache.py:253-275): page i of sequence b is page number
