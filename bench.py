@@ -145,27 +145,42 @@ def synth_w(n, k, seed=1, device="cpu"):
     return pack_i4(codes), s
 
 
-def timed_loops(step, steps, warmup, repeats):
-    """warm-up, then `repeats` loops of `steps` steps, each between two synchronisations and holding
-    nothing but the step's own launches.  Returns per-step milliseconds of every loop."""
+MIN_SPAN_MS = 150.0      # timed loops keep coming until they span this much GPU time (see timed_loops)
+MAX_LOOPS = 600
+_RAMP = {}
+
+
+def timed_loops(step, steps, warmup, repeats, min_span_ms=MIN_SPAN_MS):
+    """warm-up, then loops of exactly `steps` steps, each between two synchronisations and holding nothing but
+    the step's own launches.  Returns per-step milliseconds of the LAST `repeats` loops.
+    After an idle period this GPU needs about 30 ms of continuous work before its clocks settle (20-step loops
+    of the default workload from a cold start: 92, 104, 98, 94, 91, 89, 87, 86, 84 ... 81 us per step, level from
+    the twentieth loop on), so with short loops the first ones measure the ramp, not the kernels: loops are run
+    until they span `min_span_ms` in all (at least `repeats`, at most MAX_LOOPS), and the last `repeats` are the
+    measurement.  The first loop's time and the number of loops are reported next to it.  (The context columns,
+    measured right behind the main loops on a GPU that is already at its clocks, pass min_span_ms = 0.)"""
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    out = []
-    for _ in range(repeats):
+    out, span = [], 0.0
+    while len(out) < repeats or (span < min_span_ms and len(out) < MAX_LOOPS):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        out.append((time.perf_counter() - t0) * 1e3 / steps)
-    return out
+        dt = (time.perf_counter() - t0) * 1e3
+        out.append(dt / steps)
+        span += dt
+    _RAMP.update(first_loop_ms=round(out[0], 5), loops_run=len(out))
+    return out[-repeats:]
 
 
 def spread(ms_list):
     a = np.asarray(ms_list, dtype=np.float64)
     return {"median_ms": round(float(np.median(a)), 5), "mean_ms": round(float(a.mean()), 5),
-            "ci95_ms": round(float(1.96 * a.std()), 5), "min_ms": round(float(a.min()), 5), "repeats": int(a.size)}
+            "ci95_ms": round(float(1.96 * a.std()), 5), "min_ms": round(float(a.min()), 5), "repeats": int(a.size),
+            "loops_run": _RAMP.get("loops_run", int(a.size)), "first_loop_ms": _RAMP.get("first_loop_ms")}
 
 
 _BLOCKER = {}
@@ -371,7 +386,7 @@ class LinearWorkload:
         prints its int4 chains beside it, benchmarks/qlinear_benchmark.py:60-66,102-106); random weights."""
         w = torch.randn(self.n, self.k, device=self.x.device, dtype=torch.float16) * 0.02
         x = self.x.reshape(self.m, self.k)
-        return float(np.median(timed_loops(lambda: torch.nn.functional.linear(x, w), steps, 3, 3)))
+        return float(np.median(timed_loops(lambda: torch.nn.functional.linear(x, w), steps, 3, 3, min_span_ms=0)))
 
     def kernel_times(self, reps):
         """(front kernel ms, GEMM kernel ms), each from a pass of its own (decode: the weights still
@@ -440,7 +455,7 @@ def run_linear(name, dev, steps, warmup, repeats, kernel_reps, on_gpu_data, grap
     ms = sp["median_ms"]
     front_ms, gemm_ms = wl.kernel_times(kernel_reps)
     groof, froof = wl.rooflines(front_ms, gemm_ms)
-    staged = timed_loops(wl.staged_step, max(5, steps // 4), 3, min(repeats, 3))
+    staged = timed_loops(wl.staged_step, max(5, steps // 4), 3, min(repeats, 3), min_span_ms=0)
     if not wl.decode:
         extra["fp16_linear_ms"] = round(wl.fp16_linear_ms(max(5, steps // 10)), 5)
     # the whole step against the same roofline as its dominant kernel (algorithmic bytes of the GEMM for decode)
@@ -724,6 +739,8 @@ def main():
         spec = WORKLOADS[name]
         big = name.startswith("c3") or name in ("c5", "c6")
         steps = args.steps if headline else max(20, args.steps // 5)
+        if not headline and (name in ("c6", "c6b") or (spec is not None and spec[0] <= 64)):
+            steps = max(steps, 100)                        # decode steps of 25-50 us: a loop's ~30 us of start and wake-up spread over 100
         if big:
             steps = max(5, steps // (25 if name == "c3" else 10))
         repeats = args.repeats if headline else max(3, args.repeats // 2)
@@ -765,8 +782,11 @@ def main():
                   else "int4 x int4 -> int32 (int8 MFMA), fp16 scales"),
         "data": "synthetic",
         "config": {"workload": res["workload"], "launch": res.get("launch", "eager"),
-                   "timing": "median of `repeats` loops of `steps` steps, each loop between two synchronisations; kernel times from a "
-                             "separate pass of back-to-back launches of that kernel alone between two HIP events on the launch stream"},
+                   "timing": "median of the last `repeats` loops of `steps` steps, each loop between two synchronisations; loops run until "
+                             f"they span {MIN_SPAN_MS:.0f} ms (`loops_run`), because the GPU's clocks take ~30 ms of work to settle after idling "
+                             "(`first_loop_ms`: the first loop); kernel times from a separate pass of back-to-back launches of that kernel "
+                             "alone between two HIP events on the launch stream",
+                   "loops_run": res["timing"].get("loops_run"), "first_loop_ms": res["timing"].get("first_loop_ms")},
         "roofline": roof,
     }
     for key in ("front", "kernels", "per_linear", "kernels_ms_sum", "staged_reference_api_ms", "fp16_linear_ms", "step_frac"):
@@ -794,7 +814,7 @@ def main():
                                          for name, r in per.items()}
         out["roofline"]["per_config_front"] = {name: [r["front"]["kernel_ms"], r["front"]["frac"]] for name, r in per.items() if "front" in r}
         out["per_config_note"] = ("same step definition as the headline; operands generated on the GPU, a fifth of the steps per loop "
-                                  "(c3, c5: fewer still) and half the repeats")
+                                  "(c3, c5: fewer still; decode and attention steps: at least 100) and half the repeats")
     print(json.dumps(out))
 
 
