@@ -405,6 +405,34 @@ def test_cache_class_padded_prompt_and_the_reference_benchmarks_fake_prefill():
     assert close(attn_out.cpu().numpy().reshape(B, H, 128), want)
 
 
+def test_cache_class_long_sequence_small_batch_keeps_one_scratch_buffer():
+    """One sequence of 1500+ tokens, 8 heads: decode attention is split along the sequence, and the partial states go
+    through the scratch buffer that the cache keeps (one allocation, reused by every step and layer).  Three decode
+    steps of two layers each against the oracle on the cache's own pages."""
+    B, H, P, S0, L = 1, 8, 16, 1500, 2
+    g = torch.Generator().manual_seed(12)
+    cache = kv.MultiLayerPagedKVCache4Bit(B, P, S0 + 8, "cuda:0", L, H, 128)
+    assert kv._decode_workspace_bytes(B, H, S0 + 8, 0) > 0                 # this shape does split
+    for layer in range(L):
+        k = torch.randn(B, S0, H, 128, generator=g).half().cuda()
+        v = torch.randn(B, S0, H, 128, generator=g).half().cuda()
+        cache.update(k, v, layer, {})
+    seen = set()
+    for step in range(3):
+        for layer in range(L):
+            k1 = torch.randn(B, 1, H, 128, generator=g).half().cuda()
+            v1 = torch.randn(B, 1, H, 128, generator=g).half().cuda()
+            q1 = torch.randn(B, 1, H, 128, generator=g).half().cuda()
+            out = cache.update(k1, v1, layer, {})(q1)
+            seen.add(cache._decode_ws.data_ptr())
+            specs = cache.get_cache_specs_for_flash_infer(None)
+            qh = kv.matmul_had_cuda(q1.view(B, H, 128), torch.float16).cpu().numpy()
+            want = o.paged_batch_decode(qh, cache.pages.cpu().numpy(), cache.scales.cpu().numpy(),
+                                        *[specs[n].cpu().numpy() for n in ("kv_indptr", "kv_indices", "last_page_offset")], layer)
+            assert out.shape == (B, 1, H, 128) and close(out.cpu().numpy().reshape(B, H, 128), want)
+    assert len(seen) == 1 and cache.length == S0 + 3
+
+
 def test_decode_attention_at_config5_size():
     """The cache of config 5 (32 sequences x 4096 tokens x 8 KV heads x 128) in pages of 16: filled by the
     fused quantise-and-append, read by decode attention; sampled (sequence, head) pairs against the oracle,
