@@ -157,8 +157,8 @@ int qr_linear_i4_f16(const void* A, const void* sA, const void* W, const void* s
 
 /*
  * The same with a caller-provided scratch buffer, for shapes whose output tiles would occupy only a
- * fraction of the CUs (decode batches of 5..64 tokens against a narrow weight, prompts of a few
- * hundred tokens): K is then split across workgroups, each slice leaves its int32 partial sums in
+ * fraction of the CUs (decode batches of 40..64 tokens against a narrow weight with K >= 16384,
+ * prompts of a few hundred tokens): K is then split across workgroups, each slice leaves its int32 partial sums in
  * `workspace` and a second kernel adds and dequantises them (two launches on `stream`).  The library never
  * allocates (the reference's bindings allocate their outputs with torch::empty,
  * quarot/kernels/bindings.cpp:20,39,74; here the caller does).
