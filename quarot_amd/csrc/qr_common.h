@@ -134,6 +134,16 @@ __device__ __forceinline__ u32 cvt_f16x2(float a, float b) {
     return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2));
 }
 
+// An 8-byte store that is written through the L2 to memory at once (device scope) instead of staying dirty in the
+// L2 until the kernel ends; the line remains in the L2 for readers on the same XCD.
+__device__ __forceinline__ void store_through(u32x2* dst, u32x2 v) {
+    __hip_atomic_store((unsigned long long*)dst, ((unsigned long long)v[1] << 32) | v[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ void store_through(u32* dst, u32 v) {
+    __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Reinterpret one 32-bit word as two halves.  Always go through this by-value helper: applying
 // __builtin_bit_cast directly to an element of an ext-vector (v[i]) was seen to read element 0
 // whatever the index.

@@ -45,17 +45,19 @@ __global__ __launch_bounds__(QT) void quant_rows_kernel(const u32x4* __restrict_
     u32* qr = q + row * (int64_t)cols8;
     if (fast_quant_ok(m, s)) {       // workgroup-uniform
         const FastRecip fr = make_fast_recip(s);
+        // (codes are written through the L2: the GEMM that follows still finds them there, and they are not left to
+        // be written back in a burst when the kernel ends -- 2048 x 4096: 4.5 -> 4.35 us, the step 33.8 -> 33.5 us)
         if (!GIVEN_SCALE && clamp_cannot_act(clip, s)) {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 int c = threadIdx.x + i * QT;
-                if (c < cols8) qr[c] = sym_codes8_fast<false>(v[i], fr);
+                if (c < cols8) store_through(&qr[c], sym_codes8_fast<false>(v[i], fr));
             }
         } else {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 int c = threadIdx.x + i * QT;
-                if (c < cols8) qr[c] = sym_codes8_fast<true>(v[i], fr);
+                if (c < cols8) store_through(&qr[c], sym_codes8_fast<true>(v[i], fr));
             }
         }
         return;
