@@ -189,16 +189,24 @@ _BLOCKER = {}
 def kernel_ms(fn, reps):
     """Average duration of one launch of fn(): `reps` back-to-back launches between one pair of HIP events
     on the launch stream.  The host needs longer to issue a launch than a short kernel runs, and an idle
-    GPU would then time the host: a few milliseconds of device copies are queued first, so that the events
-    and every launch are already waiting in the stream when the GPU reaches them."""
+    GPU would then time the host: a device copy is queued first, so that the events and every launch are
+    already waiting in the stream when the GPU reaches them.  The copy is kept as short as that allows
+    (~16 us of host time per launch to cover: 0.8 ms for 50 launches) and follows 20 ms of the function itself:
+    the GPU's clocks follow what it has been doing for the last milliseconds, and behind 6-13 ms of copying --
+    the blocker this pass used to queue -- the prefill GEMMs ran 8-11 % slower than in the loop of the step
+    (68.8 against 63.3 us for the default workload's, whose step loop -- 83.1 us -- is the sum of 18.4, 63.3
+    and two launch boundaries; behind a sleeping kernel likewise: 71 us)."""
     if "src" not in _BLOCKER:
         _BLOCKER["src"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
         _BLOCKER["dst"] = torch.empty(1 << 32, dtype=torch.uint8, device="cuda")
     fn()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
-    for _ in range(max(2, reps // 12)):                      # ~1.6 ms each
-        _BLOCKER["dst"].copy_(_BLOCKER["src"])
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.02:
+        fn()
+    nbytes = min(1 << 32, max(1 << 30, reps * (42 << 20)))      # the copy moves ~2.6 GB per millisecond
+    _BLOCKER["dst"][:nbytes].copy_(_BLOCKER["src"][:nbytes])
     e0.record()
     for _ in range(reps):
         fn()
