@@ -203,8 +203,10 @@ def kernel_ms(fn, reps):
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    while time.perf_counter() - t0 < 0.02:
-        fn()
+    while time.perf_counter() - t0 < 0.02:                   # (20 ms of GPU time: the host would queue far more unsynchronised)
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     nbytes = min(1 << 32, max(1 << 30, reps * (42 << 20)))      # the copy moves ~2.6 GB per millisecond
     _BLOCKER["dst"][:nbytes].copy_(_BLOCKER["src"][:nbytes])
     e0.record()
