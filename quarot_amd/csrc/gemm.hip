@@ -1183,28 +1183,31 @@ __global__ __launch_bounds__(256) void gemm_spk_kernel(
     // tile, group 1: 64..127) and sends tiles j = 2, 3 across through LDS, two 32-row tiles (i) per
     // round, four 16-byte pieces per lane and tile.
     {
+        // (all four 32-row tiles in one round: 32 KB per wave, 128 KB of the stage buffers' 144 KB in the direct form;
+        // the register-staged form has 96 KB of LDS and takes two rounds)
         u32x4* xbuf = spk_lds;
+        constexpr int IR = DIRECT ? IM : 2;                   // 32-row tiles per round
 #pragma unroll
-        for (int ip = 0; ip < IM; ip += 2) {
+        for (int ip = 0; ip < IM; ip += IR) {
             __syncthreads();
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
+            for (int ii = 0; ii < IR; ++ii)
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                     for (int qv = 0; qv < 4; ++qv) {
                         const i32x16& t = acc[ip + ii][2 + jj];
-                        xbuf[((((wn * 2 + (1 - kg)) * 2 + ii) * 2 + jj) * 4 + qv) * 64 + lane] =
+                        xbuf[((((wn * 2 + (1 - kg)) * IR + ii) * 2 + jj) * 4 + qv) * 64 + lane] =
                             u32x4{(u32)t[qv * 4], (u32)t[qv * 4 + 1], (u32)t[qv * 4 + 2], (u32)t[qv * 4 + 3]};
                     }
             __syncthreads();
 #pragma unroll
-            for (int ii = 0; ii < 2; ++ii)
+            for (int ii = 0; ii < IR; ++ii)
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
                     for (int qv = 0; qv < 4; ++qv) {
-                        const u32x4 piece = xbuf[((((wn * 2 + kg) * 2 + ii) * 2 + jj) * 4 + qv) * 64 + lane];
+                        const u32x4 piece = xbuf[((((wn * 2 + kg) * IR + ii) * 2 + jj) * 4 + qv) * 64 + lane];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) acc[ip + ii][jj][qv * 4 + e] += (int)piece[e];
                     }
