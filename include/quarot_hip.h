@@ -36,6 +36,13 @@ extern "C" {
 
 #define QR_DTYPE_F16 0
 #define QR_DTYPE_F32 1
+/* or-ed into the `mode` of qr_hadamard_quantize_f16_i4 / qr_quantized_linear_f16: hadK points to SIGN WORDS instead of
+ * the table -- uint32 [K][ceil(K / 32)] row-major, 4-byte aligned, bit j of word w of row r set where hadK[r][32 w + j]
+ * is -1 and clear where it is +1 (bits past column K clear).  A prepared operand like a packed weight: built once per
+ * table by the caller, 4 KB where the fp16 table of order 172 is 59 KB that every workgroup would fetch.  Only for
+ * tables of +-1 (all of the reference's are); taken where the lean kernel applies (n / K = 64, K = 97 .. 192, no copy
+ * of the transformed rows), QR_E_UNSUPPORTED with nothing launched otherwise: pass the table then. */
+#define QR_HADK_SIGNS 0x100
 
 /* Library version (major*10000 + minor*100 + patch). */
 int qr_version(void);
@@ -86,7 +93,8 @@ int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, int64_t col
  * the transformed row is rounded to fp16 exactly as qr_hadamard(QR_DTYPE_F16 input) would store it
  * and quantised from there, without the fp16 tensor making a round trip through HBM.
  *   x fp16 [rows, n]; mode QR_DTYPE_F16 (fp16 staging) or QR_DTYPE_F32 (OnlineHadamard force_fp32:
- *   hadK is then fp32 [K,K]); y_or_null: optional fp16 [rows, n] copy of the transformed rows.
+ *   hadK is then fp32 [K,K]), optionally | QR_HADK_SIGNS (hadK is then the table's sign words, see above);
+ *   y_or_null: optional fp16 [rows, n] copy of the transformed rows.
  *   x and y 16-byte aligned, q 8-byte aligned.
  */
 int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, int K, const void* hadK,

@@ -9,6 +9,8 @@ its C ABI.  Extras that fuse adjacent steps are listed after the reference's nam
 """
 import functools
 
+import weakref
+
 import torch
 
 from . import _lib
@@ -145,6 +147,37 @@ def quantize_rows(x, clip_ratio=1.0):
     return q.view(*lead, q.shape[-1]), s.view(s_shape)
 
 
+_SIGNS = {}                 # id(table) -> (weak reference to the table, its version, sign words or None)
+_SIGNS_REFUSED = set()      # (n, K) for which the library takes the table itself
+
+
+def _hadamard_sign_words(hadK, n, K):
+    """The table's sign words -- uint32 [K][ceil(K / 32)] as bytes, bit j of word w of row r set where
+    hadK[r][32 w + j] = -1 -- for the widths whose fused kernel takes them (n / K = 64 behind a table of order
+    97 .. 192: the down_proj width 11008 = 172 x 64), or None.  A prepared operand: packed once per table
+    (4 KB for order 172, where the fp16 table is 59 KB that every workgroup of the kernel would fetch) and
+    kept while the table object lives and is not written to; tables with entries other than +-1 are never
+    packed."""
+    if hadK is None or K <= 96 or K > 192 or n != 64 * K or (n, K) in _SIGNS_REFUSED:
+        return None
+    key = id(hadK)
+    hit = _SIGNS.get(key)
+    if hit is not None and hit[0]() is hadK and hit[1] == hadK._version:
+        return hit[2]
+    words = None
+    if tuple(hadK.shape) == (K, K) and bool((hadK.abs() == 1).all()):
+        import numpy as np
+        neg = (hadK < 0).cpu().numpy()
+        padded = np.zeros((K, (K + 31) // 32 * 32), dtype=bool)
+        padded[:, :K] = neg
+        words = torch.from_numpy(np.packbits(padded, axis=1, bitorder="little")).to(hadK.device)
+    if len(_SIGNS) > 64:
+        for k in [k for k, v in _SIGNS.items() if v[0]() is None]:
+            del _SIGNS[k]
+    _SIGNS[key] = (weakref.ref(hadK), hadK._version, words)
+    return words
+
+
 def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_transformed=False):
     """OnlineHadamard.forward followed by Quantizer.forward in one kernel
     (quarot/nn/hadamard.py:17-23 + quarot/nn/quantization.py:9-13)."""
@@ -153,6 +186,7 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
     dev = _require_gpu_contiguous("hadamard_quantize", x=x2, hadK=hadK)
     rows, n = x2.shape
     want = torch.float32 if force_fp32 else torch.float16
+    table = hadK                                   # (the caller's object: what the sign words are remembered for)
     if hadK is not None and hadK.dtype != want:
         hadK = hadK.to(want)
     q = torch.empty((rows, n // 2), dtype=torch.uint8, device=dev)
@@ -160,10 +194,18 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
     y = torch.empty_like(x2) if return_transformed else None
     scale = functional.hadamard.had_scale(n)
     mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
+    signs = None if return_transformed else _hadamard_sign_words(table, n, int(K))
     with _lib.on_device(dev):
-        _lib.check(_lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
-                                                          float(clip_ratio), _ptr(q), _ptr(s), _ptr(y),
-                                                          _lib.stream_ptr(dev)))
+        rc = _lib.QR_E_UNSUPPORTED
+        if signs is not None:
+            rc = _lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(signs), mode | _lib.QR_HADK_SIGNS, scale,
+                                                        float(clip_ratio), _ptr(q), _ptr(s), None, _lib.stream_ptr(dev))
+            if rc == _lib.QR_E_UNSUPPORTED:
+                _SIGNS_REFUSED.add((n, int(K)))
+        if rc == _lib.QR_E_UNSUPPORTED:
+            rc = _lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
+                                                        float(clip_ratio), _ptr(q), _ptr(s), _ptr(y), _lib.stream_ptr(dev))
+        _lib.check(rc)
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))
     return (packed, y.view(x.shape)) if return_transformed else packed
@@ -310,15 +352,24 @@ def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_r
     if bias is not None and (bias.dtype != torch.float16 or bias.numel() != N):
         raise RuntimeError("quantized_linear: bias must be fp16 of size out_features")
     want = torch.float32 if force_fp32 else torch.float16
+    table = hadK
     if hadK is not None and hadK.dtype != want:
         hadK = hadK.to(want)
     y = torch.empty((M, N), dtype=torch.float16, device=dev)
     mode = _lib.QR_DTYPE_F32 if force_fp32 else _lib.QR_DTYPE_F16
+    signs = _hadamard_sign_words(table, n, int(K)) if K else None
     with _lib.on_device(dev):
         ws_bytes = _quantized_linear_workspace_bytes(M, N, n, dev.index)
         ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
-        _lib.check(_lib.lib().qr_quantized_linear_f16(_ptr(x2), M, n, int(K), _ptr(hadK), mode,
-                                                      functional.hadamard.had_scale(n), float(clip_ratio), _ptr(weight),
-                                                      _ptr(sw), _ptr(bias), N, _ptr(y), _ptr(ws), ws_bytes,
-                                                      _lib.stream_ptr(dev)))
+        call = lambda table, md: _lib.lib().qr_quantized_linear_f16(
+            _ptr(x2), M, n, int(K), _ptr(table), md, functional.hadamard.had_scale(n), float(clip_ratio), _ptr(weight),
+            _ptr(sw), _ptr(bias), N, _ptr(y), _ptr(ws), ws_bytes, _lib.stream_ptr(dev))
+        rc = _lib.QR_E_UNSUPPORTED
+        if signs is not None:
+            rc = call(signs, mode | _lib.QR_HADK_SIGNS)                  # (refused before anything is launched)
+            if rc == _lib.QR_E_UNSUPPORTED:
+                _SIGNS_REFUSED.add((n, int(K)))
+        if rc == _lib.QR_E_UNSUPPORTED:
+            rc = call(hadK, mode)
+        _lib.check(rc)
     return y.view(*lead, N)

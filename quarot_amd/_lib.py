@@ -49,6 +49,8 @@ SIGNATURES = {
 }
 
 QR_DTYPE_F16, QR_DTYPE_F32 = 0, 1
+QR_HADK_SIGNS = 0x100          # or-ed into a `mode`: hadK is passed as sign words (include/quarot_hip.h)
+QR_E_UNSUPPORTED = -3
 
 _lib = None
 

@@ -1362,7 +1362,8 @@ __global__ __launch_bounds__(HT, (LOG2M == 7 && KS2 >= 5 ? 1 : 2)) void hadamard
 template <bool MODE32, int KS2, int TPW, int CHUNKS>
 __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, int64_t rows, int n, int K,
                                                    const void* __restrict__ hadK, float scale, float clip,
-                                                   u32* __restrict__ q, f16* __restrict__ scales, f32x4* smem_raw, u32* red) {
+                                                   u32* __restrict__ q, f16* __restrict__ scales, f32x4* smem_raw, u32* red,
+                                                   int signs) {
     constexpr int CT = 4, NT = 2 * KS2;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4;
@@ -1405,7 +1406,35 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
     // each lane then picks its 8-byte pieces from there.  Loading them straight from memory -- a lane's pieces lie 32
     // bytes apart, every workgroup of the grid asks at the same moment -- cost 3 of the 23 us of a 2048-row launch.
     f16x8 hf[TPW][KS2];
-    if (MODE32 && hadK == nullptr) {
+    if (signs) {
+        // hadK as sign words (uint32 [K][ceil(K / 32)], bit j of word w of row r set where hadK[r][32 w + j] = -1; the
+        // table is +-1 by construction): a lane reads the KS2 words of each of its rows -- 4 KB in all where the fp16
+        // table is 59 KB per workgroup, two workgroups per CU, through a memory path of 35-60 GB/s per CU: 3 us of a
+        // 2048-row launch -- and expands the four bits of every fragment half into four halves of +-1
+        const u32* sw = (const u32*)hadK;
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) {
+            const int hr = (wave + 4 * i) * 16 + l16;
+            const bool rok = hr < K;
+#pragma unroll
+            for (int ks = 0; ks < KS2; ++ks) {
+                const u32 w = sw[rok ? hr * KS2 + ks : 0];
+                u32x4 fr;
+#pragma unroll
+                for (int hh = 0; hh < 2; ++hh) {
+                    const u32 nib = (w >> (hh * 16 + g * 4)) & 15u;
+                    const bool ok = rok && ks * 32 + hh * 16 + g * 4 < K;
+                    const u32 p0 = 0x3C003C00u | ((nib & 1u) << 15) | ((nib & 2u) << 30);
+                    const u32 p1 = 0x3C003C00u | ((nib & 4u) << 13) | ((nib & 8u) << 28);
+                    fr[hh * 2] = ok ? p0 : 0u;
+                    fr[hh * 2 + 1] = ok ? p1 : 0u;
+                }
+                hf[i][ks] = __builtin_bit_cast(f16x8, fr);
+            }
+        }
+        u32x4* stage = (u32x4*)smem_raw;
+        for (int i = tid; i < (MODE32 ? 2 : 1) * CT * NT * 32; i += HT) stage[i] = u32x4{0, 0, 0, 0};
+    } else if (MODE32 && hadK == nullptr) {
         // power-of-two row: the outer factor is the Sylvester matrix of order K, generated in place
 #pragma unroll
         for (int i = 0; i < TPW; ++i) {
@@ -1689,14 +1718,14 @@ __device__ __forceinline__ void hadamard_m64r_rows(const f16* __restrict__ x, in
 template <bool MODE32, int KS2>
 __global__ __launch_bounds__(HT, 2) void hadamard_m64r_kernel(const f16* __restrict__ x, int64_t rows, int n, int K,
                                                             const void* __restrict__ hadK, float scale, float clip,
-                                                            u32* __restrict__ q, f16* __restrict__ scales) {
+                                                            u32* __restrict__ q, f16* __restrict__ scales, int signs) {
     constexpr int NT = 2 * KS2, TPW = (NT + 3) / 4;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[HT / QR_WAVE];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // (both forms pass the same barriers: two per 64 rows of hadK and one more before the loop, two per row)
-    if ((wave + 4 * (TPW - 1)) * 16 < K) hadamard_m64r_rows<MODE32, KS2, TPW, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
-    else hadamard_m64r_rows<MODE32, KS2, TPW - 1, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red);
+    if ((wave + 4 * (TPW - 1)) * 16 < K) hadamard_m64r_rows<MODE32, KS2, TPW, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red, signs);
+    else hadamard_m64r_rows<MODE32, KS2, TPW - 1, TPW>(x, rows, n, K, hadK, scale, clip, q, scales, smem_raw, red, signs);
 }
 
 // A power-of-two row of 1024..16384 elements is H_K (x) H_m with both factors Sylvester: the same
@@ -1715,7 +1744,7 @@ bool mm_applies(int n, int K) {
 
 template <bool MODE32, bool QUANT>
 int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const void* hadK, float scale, float clip,
-                       void* q, void* scales, hipStream_t st, int ident = 0) {
+                       void* q, void* scales, hipStream_t st, int ident = 0, int signs = 0) {
     const int m = n / K;
     const int KS2 = ((K + 31) & ~31) >> 5;
     if (m == 128 && KS2 >= 2 && KS2 != 3 && !ident && !MODE32 && QUANT && y == nullptr && hadK != nullptr && ((uintptr_t)x & 15) == 0) {
@@ -1745,7 +1774,8 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         // two workgroups still fit on a CU
         const int tpw = (2 * KS2 + 3) / 4;
         const size_t lds64 = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2 + (size_t)tpw * (64 * 72 * 2 + 4 * 2048);
-        if (QUANT && y == nullptr && (MODE32 || hadK != nullptr) && ((uintptr_t)x & 15) == 0 && ((uintptr_t)hadK & 15) == 0) {
+        if (QUANT && y == nullptr && (MODE32 || hadK != nullptr) && ((uintptr_t)x & 15) == 0 &&
+            ((uintptr_t)hadK & (signs ? 3 : 15)) == 0) {
             // fused, no copy of the transformed rows wanted: the lean kernel (T alone in LDS; two planes of it in the
             // fp32-precision mode)
             const size_t ldsq = (size_t)(MODE32 ? 2 : 1) * 4096 * KS2;
@@ -1758,7 +1788,8 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
         }                                                                                                              \
         const int64_t cap = (int64_t)qr_device().cus * qr_blocks_per_cu((const void*)kern, HT, ldsq);                  \
         const unsigned grid = (unsigned)(rows < cap ? rows : cap);                                                     \
-        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, hadK, scale, clip, (u32*)q, (f16*)scales); \
+        kern<<<dim3(grid), dim3(HT), ldsq, st>>>((const f16*)x, rows, n, K, hadK, scale, clip, (u32*)q, (f16*)scales,  \
+                                                 signs);                                                               \
     } while (0)
             // (orders of 64 and more among the reference's tables: 108, 140, 156, 172)
             if (KS2 >= 4) {
@@ -1771,6 +1802,7 @@ int launch_hadamard_mm(const void* x, void* y, int64_t rows, int n, int K, const
             }
 #undef QR_M64Q
         }
+        if (signs) return QR_E_UNSUPPORTED;
         if (lds64 <= 80 * 1024) {
 #define QR_M64(KS)                                                                                                     \
     do {                                                                                                               \
@@ -2437,7 +2469,16 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
     if (!x || !q || !scales || (K > 1 && !hadK)) return QR_E_NULL;
     if (((uintptr_t)x & 15) || ((uintptr_t)y_or_null & 15) || ((uintptr_t)q & 7)) return QR_E_ALIGN;
     hipStream_t st = (hipStream_t)stream;
+    const int signs = (mode & QR_HADK_SIGNS) ? 1 : 0;
+    mode &= ~QR_HADK_SIGNS;
     if (mode != QR_DTYPE_F16 && mode != QR_DTYPE_F32) return QR_E_DTYPE;
+    if (signs) {
+        // hadK as sign words: the lean kernel of the m = 64 widths behind a table of order 97 .. 192 only (nothing is
+        // launched otherwise: the caller passes the table itself)
+        if (K <= 96 || y_or_null || !mm_applies(n, K) || n / K != 64 || ((uintptr_t)hadK & 3)) return QR_E_UNSUPPORTED;
+        if (mode == QR_DTYPE_F16) return launch_hadamard_mm<false, true>(x, nullptr, rows, n, K, hadK, scale, clip, q, scales, st, 0, 1);
+        return launch_hadamard_mm<true, true>(x, nullptr, rows, n, K, hadK, scale, clip, q, scales, st, 0, 1);
+    }
     if (tiny_applies(n, K)) return QR_E_UNSUPPORTED;       // rows this short: qr_hadamard, then qr_quantize_rows_f16_i4
     if (K == 1 && pow2_split(n))
         return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, pow2_split(n), nullptr, scale, clip, q, scales, st);

@@ -714,6 +714,85 @@ def test_fused_hadamard_quantize_lean_kernel_in_fp32_precision(n, clip):
     assert torch.equal(one.quantized_x, p.quantized_x[5:6])
 
 
+def sign_words(table):
+    """uint32 [K][ceil(K / 32)]: bit j of word w of row r set where table[r][32 w + j] is -1 (include/quarot_hip.h)."""
+    k = table.shape[0]
+    padded = np.zeros((k, (k + 31) // 32 * 32), dtype=bool)
+    padded[:, :k] = np.asarray(table) < 0
+    return np.packbits(padded, axis=1, bitorder="little").view(np.uint32)
+
+
+@pytest.mark.parametrize("n", [6912, 8960, 9984, 11008])
+@pytest.mark.parametrize("fp32", [False, True])
+def test_fused_hadamard_quantize_with_the_table_as_sign_words(n, fp32):
+    """QR_HADK_SIGNS through the C entry points: hadK passed as packed sign bits gives the codes and scales of the call
+    that passes the table, bit for bit (orders 108, 140, 156, 172 behind FWHT-64; both precisions; rows of every
+    kind), also through the one-call chain; shapes outside the lean kernel and calls that want the transformed rows
+    are refused with QR_E_UNSUPPORTED before anything is written."""
+    from quarot_amd.functional import hadamard as fh
+    table, K = fh.get_hadK(n)
+    rows = 700
+    x = synth_x(rows, n, seed=n + 31)
+    x[3, 17] = np.inf
+    x[5, 5] = np.nan
+    x[7] = 0
+    xg = gpu(x)
+    L, st = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    mode = _lib.QR_DTYPE_F32 if fp32 else _lib.QR_DTYPE_F16
+    tab = gpu(np.asarray(table, dtype=np.float32 if fp32 else F16))
+    sw = gpu(sign_words(np.asarray(table)).view(np.uint8))
+    scale = fh.had_scale(n)
+    out = {}
+    for name, ptr, md in (("table", tab, mode), ("signs", sw, mode | _lib.QR_HADK_SIGNS)):
+        q = torch.full((rows, n // 2), 0x5A, dtype=torch.uint8, device="cuda:0")
+        s = torch.zeros(rows, dtype=torch.float16, device="cuda:0")
+        rc = L.qr_hadamard_quantize_f16_i4(xg.data_ptr(), rows, n, K, ptr.data_ptr(), md, scale, 0.9, q.data_ptr(), s.data_ptr(), None, st)
+        assert rc == 0, (name, rc)
+        out[name] = (q, s)
+    assert torch.equal(out["signs"][0], out["table"][0])
+    assert np.array_equal(bits(out["signs"][1].cpu().numpy()), bits(out["table"][1].cpu().numpy()))
+    # refused, nothing written: the transformed rows wanted; a width of another kernel family
+    q = torch.full((rows, n // 2), 0x5A, dtype=torch.uint8, device="cuda:0")
+    s = torch.zeros(rows, dtype=torch.float16, device="cuda:0")
+    y = torch.zeros(rows, n, dtype=torch.float16, device="cuda:0")
+    rc = L.qr_hadamard_quantize_f16_i4(xg.data_ptr(), rows, n, K, sw.data_ptr(), mode | _lib.QR_HADK_SIGNS, scale, 0.9, q.data_ptr(),
+                                       s.data_ptr(), y.data_ptr(), st)
+    assert rc == _lib.QR_E_UNSUPPORTED and bool((q == 0x5A).all()) and not bool(y.any())
+    t28, k28 = fh.get_hadK(28672)
+    x28 = gpu(synth_x(4, 28672, seed=1))
+    q28 = torch.full((4, 14336), 0x5A, dtype=torch.uint8, device="cuda:0")
+    sw28 = gpu(sign_words(np.asarray(t28)).view(np.uint8))
+    rc = L.qr_hadamard_quantize_f16_i4(x28.data_ptr(), 4, 28672, k28, sw28.data_ptr(), mode | _lib.QR_HADK_SIGNS, fh.had_scale(28672), 1.0,
+                                       q28.data_ptr(), s.data_ptr(), None, st)
+    assert rc == _lib.QR_E_UNSUPPORTED and bool((q28 == 0x5A).all())
+
+
+def test_sign_words_follow_the_table_object():
+    """The Python layer packs a table's sign words once and reuses them while that table object is unchanged: a table
+    written to in place is packed again (the results follow it), a table with entries other than +-1 is never packed
+    (the call passes the table), and either way the results equal those of the call that returns the transformed rows,
+    which always passes the table."""
+    n = 11008
+    x = gpu(synth_x(300, n, seed=5))
+    mod = quarot_amd.nn.OnlineHadamardQuantizer(n, input_clip_ratio=1.0).cuda()
+    def both():
+        p = quarot_amd.hadamard_quantize(x, mod.had_rem_dim, mod.rem_dim, 1.0)
+        p2, _ = quarot_amd.hadamard_quantize(x, mod.had_rem_dim, mod.rem_dim, 1.0, return_transformed=True)
+        assert torch.equal(p.quantized_x, p2.quantized_x) and torch.equal(p.scales_x, p2.scales_x)
+        return p.quantized_x.clone()
+    first = both()
+    assert quarot_amd._SIGNS[id(mod.had_rem_dim)][2] is not None              # packed
+    assert torch.equal(both(), first)
+    mod.had_rem_dim[5].neg_()                                                 # in place: another +-1 table
+    second = both()
+    assert not torch.equal(second, first)
+    mod.had_rem_dim[5].neg_()
+    assert torch.equal(both(), first)
+    mod.had_rem_dim[0, 0] = 0.5                                               # no longer +-1: never packed
+    third = both()
+    assert quarot_amd._SIGNS[id(mod.had_rem_dim)][2] is None and not torch.equal(third, first)
+
+
 @pytest.mark.parametrize("shape", [(5, 64), (9, 4096), (7, 5120), (3, 8192), (4, 11008), (2, 32768), (6, 24), (3, 100)])
 @pytest.mark.parametrize("clip", [1.0, 0.9])
 def test_fused_rmsnorm_quantize(shape, clip):
