@@ -152,7 +152,7 @@ __global__ __launch_bounds__(QT) void rmsnorm_quant_rows_kernel(const u32x4* __r
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int c = threadIdx.x + i * QT;
-            if (c < cols8) qr[c] = sym_codes8_fast(v[i], fr);
+            if (c < cols8) store_through(&qr[c], sym_codes8_fast(v[i], fr));      // (through the L2, as in quant_rows_kernel)
         }
         return;
     }
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(QT) void heads_hadamard_quant_rows_kernel(const u32
     if (fast_quant_ok(m, s)) {       // wave-uniform
         const FastRecip fr = make_fast_recip(s);
 #pragma unroll
-        for (int i = 0; i < NC; ++i) qr[lane + i * QR_WAVE] = sym_codes8_fast(v[i], fr);
+        for (int i = 0; i < NC; ++i) store_through(&qr[lane + i * QR_WAVE], sym_codes8_fast(v[i], fr));   // (through the L2, as in quant_rows_kernel)
         return;
     }
     const bool fast = scale_fast_ok(s);
