@@ -1,0 +1,304 @@
+// One token through OnlineHadamard -> Quantizer -> Linear4bit in ONE launch (quarot/nn/hadamard.py:17-23,
+// quarot/nn/quantization.py:10, quarot/nn/linear.py:42-56 on a single row).
+// A decode step at one token is latency: the transform of a 57 KB row keeps one CU busy for a few microseconds
+// while the others wait, and only then does the weight stream start.  Here EVERY workgroup transforms and
+// quantises the row itself (the row comes out of L2; the arithmetic is that of hadamard_bm_kernel's register
+// path, operation for operation, so codes and scale are the same bits) with its first weight segments already
+// requested, keeps the codes in LDS and goes on as the dot-product kernel does (v_dot8_i32_i4 over 1 KB segments of
+// the weight rows, gemv_i4_kernel's arithmetic and epilogue).  Nothing is exchanged between workgroups.
+#include "qr_common.h"
+namespace {
+
+// Weight segments a wave requests at each point of the front (after the first barrier, after its part of the power-of-two
+// factor, after the table stage, after the codes); their sum is the depth of the ring.  A CU's memory pipeline takes
+// requests only as fast as it drains (the stream runs at the HBM rate from the first request on), so a wave that asks for
+// its whole ring at once stands at the load instructions for microseconds while the row's transform waits; spread out,
+// the front finishes earlier and the ring is still full when the dot products start.  Alternating runs, one token,
+// 8192 x 28672: {5,0,0,0} 22.0 us, {3,1,1,0} 21.4, {2,1,1,1} 20.9, {2,1,2,0} 20.7, {1,2,2,0} 20.6, {0,3,2,0} 21.3; deeper
+// rings are slower ({1,2,2,1} 21.0, {1,2,2,2} 22.2: more requests queue ahead of what the front waits for).
+constexpr int F0 = 1, F1 = 2, F2 = 2, F3 = 0, RING = F0 + F1 + F2 + F3;
+
+// n = 1024 K (K = order of the table, a multiple of 4, at most 32).  A wave takes `ng` consecutive pairs of weight
+// rows as one flattened sequence of 1 KB segments, RD segments in flight (first requested while the row is transformed).
+template <int RD>
+__global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x, int K, const f16* __restrict__ hadK,
+                                                       float scale, float clip, const uint8_t* __restrict__ B,
+                                                       const f16* __restrict__ sB, const f16* __restrict__ bias, int N,
+                                                       int ng, f16* __restrict__ Y) {
+    constexpr int NW = 16, M_ = 1024, CT = M_ / 16, RT = 2, TS = 17, R = 2;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[NW];
+    u32x4* Tl = (u32x4*)smem_raw;                // [4][CT][TS]
+    u32x2* xq = (u32x2*)(Tl + 4 * CT * TS);      // codes of the transformed row, K * 512 bytes
+    u32x4* hk = (u32x4*)(xq + K * 64);           // the table, K * K halves
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l16 = lane & 15, g = lane >> 4;
+    const int Kb = K * (M_ / 2);
+
+    // the table as it lies in memory, one piece per thread (eight copies over the workgroup, no branch: it is the
+    // oldest request, so waiting for it leaves everything else in flight); fragments are read from LDS later
+    const u32x4 hpiece = *((const u32x4*)hadK + ((tid & 127) < K * K / 8 ? (tid & 127) : 0));
+
+    // ---- the row (requested first: it is what the workgroup waits for) --------------------------------------
+    const bool works = wave * 2 < K;
+    const int pair = works ? wave : 0;
+    u32x4 raw[4];
+#pragma unroll
+    for (int sg = 0; sg < 2; ++sg)
+#pragma unroll
+        for (int bt = 0; bt < 2; ++bt)
+            raw[sg * 2 + bt] = *((const u32x4*)x + (pair * 2 + sg) * 128 + bt * 64 + l16 * 4 + g);
+    // (Lanes take the pieces in the order the matrix instruction wants them, neighbouring lanes 64 bytes apart; loading
+    // them as they lie and swapping lanes through LDS was measured 0.1 us slower.)
+
+    // ---- the weight stream of this wave ----------------------------------------------------------------------
+    const int groups = (N + R - 1) / R;
+    const int g0 = (blockIdx.x * NW + wave) * ng;
+    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
+    const int nseg = Kb / 1024;
+    const int total = gcount * nseg;
+    const int my_r = lane >> 5;                  // which of a pair's two sums this lane ends up with
+    struct Seg {
+        u32x4 w[R];
+        f16 sb, bi;
+    };
+    int fg = 0, fs = 0;
+    auto fetch = [&](Seg& s) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int nr = (g0 + fg) * R + r;
+            nr = nr < N ? nr : N - 1;
+            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + fs * 1024 + lane * 16));
+        }
+        int col = (g0 + fg) * R + my_r;
+        col = col < N ? col : N - 1;
+        s.sb = sB[col];
+        s.bi = (bias ? bias : sB)[col];
+        if (fs + 1 < nseg) ++fs;
+        else if (fg + 1 < gcount) { ++fg; fs = 0; }
+    };
+
+    // ---- fragments: Sylvester factors of both stages -----------------------------------------------------------
+    f16x8 ha[2], hb[2];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+#pragma unroll
+        for (int cth = 0; cth < 2; ++cth) ha[cth][t] = (__builtin_popcount((g * 8 + t) & (cth * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+        const int b = 16 * (t >> 2) + 4 * g + (t & 3);
+#pragma unroll
+        for (int bt = 0; bt < 2; ++bt) hb[bt][t] = (__builtin_popcount(b & (bt * 16 + l16)) & 1) ? (f16)-1.0f : (f16)1.0f;
+    }
+    for (int i = tid; i < 4 * CT * TS; i += 1024) Tl[i] = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    // every wave's requests for the row now stand before every weight request in the CU's memory queue
+    Seg ring[RD];
+#pragma unroll
+    for (int r = 0; r < F0; ++r) fetch(ring[r]);
+    if (tid < 128) hk[tid] = hpiece;        // (read after the next barrier)
+
+    // ---- H_1024 of the wave's two segments as H_32 (x) H_32, into the fragment order of the table stage ------
+    if (works) {
+#pragma unroll
+        for (int cth = 0; cth < 2; ++cth) {
+            u32 o[2][2][2];
+#pragma unroll
+            for (int sg = 0; sg < 2; ++sg) {
+                typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                u32x4 whi, wlo;
+#pragma unroll
+                for (int bt = 0; bt < 2; ++bt) {
+                    const f32x4 da = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, raw[sg * 2 + bt]), ha[cth],
+                                                                          f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int pr = 0; pr < 2; ++pr) {
+                        const f16x2 hi = __builtin_convertvector(f32x2_t{da[2 * pr], da[2 * pr + 1]}, f16x2);
+                        const f16x2 lo = __builtin_convertvector(f32x2_t{da[2 * pr] - (float)hi[0], da[2 * pr + 1] - (float)hi[1]}, f16x2);
+                        whi[bt * 2 + pr] = __builtin_bit_cast(u32, hi);
+                        wlo[bt * 2 + pr] = __builtin_bit_cast(u32, lo);
+                    }
+                }
+                const f16x8 thi = __builtin_bit_cast(f16x8, whi), tlo = __builtin_bit_cast(f16x8, wlo);
+#pragma unroll
+                for (int bt = 0; bt < 2; ++bt) {
+                    f32x4 db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], thi, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    db = __builtin_amdgcn_mfma_f32_16x16x32_f16(hb[bt], tlo, db, 0, 0, 0);
+                    o[sg][bt][0] = narrow_f16x2(db[0] * scale, db[1] * scale);
+                    o[sg][bt][1] = narrow_f16x2(db[2] * scale, db[3] * scale);
+                }
+            }
+            u32* const dst = (u32*)(Tl + ((pair >> 2) * CT + cth) * TS + l16) + (pair & 3);
+#pragma unroll
+            for (int bt = 0; bt < 2; ++bt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const u32 sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                    dst[(2 * (16 * bt + 4 * g + e)) * TS * 4] = __builtin_amdgcn_perm(o[1][bt][e >> 1], o[0][bt][e >> 1], sel);
+                }
+        }
+    }
+#pragma unroll
+    for (int r = F0; r < F0 + F1; ++r) fetch(ring[r]);
+    __syncthreads();
+
+    // ---- the table stage, the row's maximum, the codes (into LDS) -------------------------------------------
+    // the table's fragments (second operand of the table stage): column k' = 16 rt + l16, contraction k = 8 g + j
+    f16x8 hf[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        u32x4 v;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const int hr = rt * 16 + l16, hc = g * 8 + hh * 4;
+            const bool in = hr < K && hc < K;
+            const u32x2 w = *((const u32x2*)hk + (in ? (hr * K + hc) >> 2 : 0));
+            v[hh * 2] = in ? w[0] : 0u;
+            v[hh * 2 + 1] = in ? w[1] : 0u;
+        }
+        hf[rt] = __builtin_bit_cast(f16x8, v);
+    }
+    bool dval[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) dval[rt] = rt * 16 + l16 < K;
+    f16x8 th4[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) th4[c] = __builtin_bit_cast(f16x8, Tl[(g * CT + wave * 4 + c) * TS + l16]);
+    u32x2 yv[RT][4];
+    float mxf = 0.f, probe = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(th4[c], hf[rt], f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            if (c == 0 && rt == 0) probe = acc[0];
+            yv[rt][c][0] = cvt_f16x2(acc[0], acc[1]);
+            yv[rt][c][1] = cvt_f16x2(acc[2], acc[3]);
+            mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[0])), __builtin_fabsf(acc[1]));
+            mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fabsf(acc[2])), __builtin_fabsf(acc[3]));
+        }
+    u32 mx = f16_bits((f16)mxf);
+    if (__builtin_amdgcn_ballot_w64(mx >= 0x7c00u || probe != probe) != 0) {
+        u16x2 m2 = {0, 0};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(u16x2, dval[rt] ? yv[rt][c][0] & 0x7fff7fffu : 0u));
+                m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(u16x2, dval[rt] ? yv[rt][c][1] & 0x7fff7fffu : 0u));
+            }
+        mx = m2[0] > m2[1] ? m2[0] : m2[1];
+    }
+    mx = wave_max_u32_dpp(mx);
+    if (lane == 0) red[wave] = mx;
+#pragma unroll
+    for (int r = F0 + F1; r < F0 + F1 + F2; ++r) fetch(ring[r]);
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < NW; ++w) mx = mx > red[w] ? mx : red[w];
+    const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
+    const float sp = (float)sh;
+    u32 c01[RT], c23[RT];
+    auto codes_from = [&](auto pair) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            u32 b0[4], b1[4];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                b0[w] = pair(yv[rt][w >> 1][w & 1]);
+                b1[w] = pair(yv[rt][2 + (w >> 1)][w & 1]);
+            }
+            c01[rt] = pack_nibbles8(b0);
+            c23[rt] = pack_nibbles8(b1);
+        }
+    };
+    if (fast_quant_ok(mx, sp)) {
+        const FastRecip fq = make_fast_recip(sp);
+        if (clamp_cannot_act(clip, sp)) codes_from([&](u32 w) { return sym_pair_fast<false>(w, fq); });
+        else codes_from([&](u32 w) { return sym_pair_fast<true>(w, fq); });
+    } else {
+        const bool fs_ok = scale_fast_ok(sp);
+        const float rs = fs_ok ? 1.0f / sp : 0.0f;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            c01[rt] = sym_codes8(u32x4{yv[rt][0][0], yv[rt][0][1], yv[rt][1][0], yv[rt][1][1]}, sp, rs, fs_ok);
+            c23[rt] = sym_codes8(u32x4{yv[rt][2][0], yv[rt][2][1], yv[rt][3][0], yv[rt][3][1]}, sp, rs, fs_ok);
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const auto s1 = __builtin_amdgcn_permlane32_swap(c01[rt], c23[rt], false, false);
+        const u32 ev = __builtin_amdgcn_perm(s1[1], s1[0], 0x05040100u);
+        const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);
+        const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
+        const u32x2 outv = {__builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u), __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u)};
+        if (dval[rt]) xq[(rt * 16 + l16) * (M_ / 16) + wave * 4 + g] = outv;
+    }
+#pragma unroll
+    for (int r = F0 + F1 + F2; r < RD; ++r) fetch(ring[r]);
+    __syncthreads();
+
+    // ---- the dot products -----------------------------------------------------------------------------------
+    if (gcount == 0) return;
+    const u32x4* xs = (const u32x4*)xq + lane;
+    int acc[R] = {0, 0};
+    int cg = 0, cs = 0;
+    auto consume = [&](const Seg& s) {
+        const u32x4 xv = xs[cs * 64];
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_sdot8((int)s.w[r][d], (int)xv[d], acc[r], false);
+        if (++cs < nseg) return;
+        // end of a pair of rows: lanes 0..31 end with the first row's sum, lanes 32..63 with the second's
+        const bool upper = (lane & 32) != 0;
+        const int give = upper ? acc[0] : acc[1];
+        const int keep = upper ? acc[1] : acc[0];
+        int sum = keep + __shfl_xor(give, 32, QR_WAVE);
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
+        if ((lane & 31) == 0) {
+            const int col = (g0 + cg) * R + my_r;
+            if (col < N) {
+                f16 yo = (f16)(sh * s.sb) * (f16)(float)sum;
+                if (bias) yo = yo + s.bi;
+                Y[col] = yo;
+            }
+        }
+        acc[0] = acc[1] = 0;
+        cs = 0;
+        ++cg;
+    };
+    int it = 0;
+    for (; it + RD <= total; it += RD) {                    // whole turns of the ring: no branch around the loads
+#pragma unroll
+        for (int r = 0; r < RD; ++r) {
+            consume(ring[r]);
+            fetch(ring[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RD - 1; ++r)
+        if (it + r < total) consume(ring[r]);
+}
+
+}  // namespace
+
+// api.hip: the whole layer for one token where the row is 1024 K halves behind a table of order K <= 32.
+// QR_E_UNSUPPORTED (nothing launched) for every other shape: the caller then chains the two kernels.
+__attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(const void* x, int n, int K, const void* hadK,
+                                                                            float scale, float clip, const void* W,
+                                                                            const void* sW, const void* bias, int64_t N,
+                                                                            void* y, hipStream_t st) {
+    if (K < 4 || K > 32 || (K & 3) != 0 || n != 1024 * K || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
+    if (((uintptr_t)x & 15) || ((uintptr_t)W & 15) || ((uintptr_t)hadK & 15)) return QR_E_UNSUPPORTED;
+    const int cus = qr_device().cus;
+    const int64_t groups = (N + 1) / 2;
+    const int ng = (int)((groups + (int64_t)cus * 16 - 1) / ((int64_t)cus * 16));
+    const unsigned grid = (unsigned)(((groups + ng - 1) / ng + 15) / 16);
+    const size_t lds = (size_t)4 * 64 * 17 * 16 + (size_t)K * 512 + 128 * 16;
+    auto kern = bm_gemv_kernel<RING>;
+    hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);
+    if (e != hipSuccess) return (int)e;
+    kern<<<dim3(grid), dim3(1024), lds, st>>>((const f16*)x, K, (const f16*)hadK, scale, clip, (const uint8_t*)W,
+                                                        (const f16*)sW, (const f16*)bias, (int)N, ng, (f16*)y);
+    return qr_launch_status();
+}

@@ -1307,3 +1307,55 @@ def test_runs_on_the_current_stream():
     s.synchronize()
     wq, ws = o.quantizer(x.cpu().numpy())
     assert np.array_equal(q.cpu().numpy(), wq)
+
+
+@pytest.mark.parametrize("n", [12288, 20480, 28672])
+def test_one_token_hadamard_linear_in_one_launch(n):
+    """One token behind a 1024-point factor and a table of order 12, 20 or 28: qr_quantized_linear_f16 runs the front
+    and the dot products in ONE kernel in which every workgroup transforms the row itself.  Its output must carry the
+    bits of the two-launch chain (same codes, same scale, same sums, same epilogue) for any number of weight rows
+    (odd, one, more than one pass per wave), with and without bias, with a clip that lets the clamp act, and on rows
+    holding zeros only, an infinity, a NaN or values that overflow the transform; the oracle's Quantizer + Linear4bit on
+    the kernel's own transformed row (itself within rtol / atol 1e-3 of the oracle's transform) closes the chain."""
+    rng = np.random.default_rng(n)
+    hadK, K = quarot_amd.functional.hadamard.get_hadK(n)
+    hadK = hadK.to(dev()).half()
+    had = quarot_amd.nn.OnlineHadamard(n).to(dev())
+    for N, bias, clip in [(1, False, 1.0), (2, True, 1.0), (130, False, 0.9), (4097, True, 1.0), (8192, False, 1.0),
+                          (9001, True, 0.8), (20000, False, 1.0)]:
+        w = gpu(rng.integers(0, 256, (N, n // 2), dtype=np.uint8))
+        sw = gpu((np.abs(rng.standard_normal((N, 1))) * 0.01 + 0.001).astype(F16))
+        b = gpu(rng.standard_normal(N).astype(F16)) if bias else None
+        x = gpu(synth_x(1, n, seed=N + n, outliers=N % 2 == 1))
+        got = quarot_amd.quantized_linear(x, w, sw, b, hadK, K, clip_ratio=clip)
+        p = quarot_amd.hadamard_quantize(x, hadK, K, clip_ratio=clip)
+        want = quarot_amd.linear_i4(p.quantized_x, p.scales_x, w, sw, b)
+        assert got.shape == (1, N) and torch.equal(got, want), (n, N)
+        if N <= 4097:
+            xh = had(x).cpu().numpy()
+            ref = o.online_hadamard(x.cpu().numpy()).astype(np.float64)
+            assert np.all(np.abs(xh.astype(np.float64) - ref) <= ATOL + RTOL * np.abs(ref))
+            xq, xs = o.quantizer(xh, clip)
+            ref_y = o.linear4bit(xq, xs, w.cpu().numpy(), sw.cpu().numpy(), None if b is None else b.cpu().numpy())
+            assert np.array_equal(bits(got.cpu().numpy()), bits(ref_y)), (n, N)
+    N = 777
+    w = gpu(rng.integers(0, 256, (N, n // 2), dtype=np.uint8))
+    sw = gpu((np.abs(rng.standard_normal((N, 1))) * 0.01 + 0.001).astype(F16))
+    for case in ("zeros", "inf", "nan", "overflow", "tiny"):
+        x = synth_x(1, n, seed=5)
+        if case == "zeros":
+            x[:] = 0
+        elif case == "inf":
+            x[0, 5] = np.inf
+        elif case == "nan":
+            x[0, n - 3] = np.nan
+        elif case == "overflow":
+            with np.errstate(over="ignore"):
+                x = (x.astype(F32) * F32(900)).astype(F16)          # infinities where the product leaves the fp16 range
+        else:
+            x *= F16(1e-4)
+        xg = gpu(x)
+        got = quarot_amd.quantized_linear(xg, w, sw, None, hadK, K)
+        p = quarot_amd.hadamard_quantize(xg, hadK, K)
+        want = quarot_amd.linear_i4(p.quantized_x, p.scales_x, w, sw, None)
+        assert np.array_equal(bits(got.cpu().numpy()), bits(want.cpu().numpy())), (n, case)
