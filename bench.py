@@ -91,6 +91,7 @@ PROFILE_OF = {
     "c1o": "heads_hadamard_quant_c1o_o_proj_7b.txt", "c2": "gemm_spk_and_hadamard_m64r_c2_down_proj_7b.txt",
     "c2_fp32had": "gemm_spk_and_hadamard_m64_fp32_c2_down_proj_7b.txt",
     "c3": "gemm_sp256_c3_prefill_layer_set_32768_tokens.txt",
+    "c4g1": "quant_gemv_c4g1_decode_70b_gate_up.txt",
     "c4g8": "decode_xs_c4g8_decode_8_tokens_70b_gate_up.txt", "c4g32": "decode_xs_c4g32_decode_32_tokens_70b_gate_up.txt",
     "c4g64": "decode_xs_c4g64_decode_64_tokens_70b_gate_up.txt", "c4m1": "bm_gemv_c4m1_decode_70b_down_proj.txt",
     "c4m8": "decode_i4_c4m8_decode_8_tokens_70b_down_proj.txt", "c4m32": "decode_i4_c4m32_decode_32_tokens_70b_down_proj.txt",
@@ -354,7 +355,8 @@ class LinearWorkload:
             self.lin.prefill_fp6, self.lin.fp6_min_rows = True, 0
         self.had_args = (self.front.had_rem_dim, self.front.rem_dim) if self.front_kind in ("had", "had32") else (None, 0)
         # one token behind a 1024-point factor: the library runs front and dot products in ONE kernel
-        self.single_launch = self.one_call and m == 1 and self.front_kind == "had" and k % 1024 == 0 and k // 1024 in (12, 20, 28)
+        self.single_launch = self.one_call and m == 1 and (
+            (self.front_kind == "had" and k % 1024 == 0 and k // 1024 in (12, 20, 28)) or (self.front_kind == "quant" and k <= 32768))
         self.fp32_had = self.front_kind == "had32"
         self.ops = 2.0 * m * n * k
 
@@ -419,9 +421,9 @@ class LinearWorkload:
         return n * k / 2 + m * k / 2 + 2 * m + 2 * n + 2 * m * n
 
     def fused_bytes(self):
-        """Algorithmic bytes of the one-kernel step: the weights, the fp16 row, the table, scales and outputs."""
+        """Algorithmic bytes of the one-kernel step: the weights, the fp16 row, the table (if any), scales and outputs."""
         m, k, n = self.m, self.k, self.n
-        return n * k / 2 + 2 * m * k + 2 * (k // 1024) ** 2 + 2 * n + 2 * m * n
+        return n * k / 2 + 2 * m * k + (2 * (k // 1024) ** 2 if self.front_kind == "had" else 0) + 2 * n + 2 * m * n
 
     def rooflines(self, front_ms, gemm_ms):
         kern = "gemm_f6_kernel" if self.fp6 else gemm_kernel_name(self.m, self.n, self.k)
@@ -429,7 +431,7 @@ class LinearWorkload:
             g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": FP6_MFMA_PEAK_TOPS, "unit": "TOP/s",
                  "convert_kernel_ms": round(self.convert_ms, 5)}
         elif self.single_launch:
-            kern = "bm_gemv_kernel"
+            kern = "bm_gemv_kernel" if self.front_kind == "had" else "quant_gemv_kernel"
             g = {"bound": "hbm", "achieved": round(self.fused_bytes() / (gemm_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
         elif self.decode:
             g = {"bound": "hbm", "achieved": round(self.gemm_bytes() / (gemm_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
@@ -437,7 +439,8 @@ class LinearWorkload:
             g = {"bound": "mfma", "achieved": round(self.ops / (gemm_ms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s"}
         g["frac"] = round(g["achieved"] / g["peak"], 4)
         g["kernel"] = kern + (" (exact int4 GEMM on FP6 operands + dequant epilogue)" if self.fp6 else
-                              " (Hadamard + quantiser + int4 dot products + dequant epilogue in one launch)" if self.single_launch else
+                              (" (Hadamard + quantiser" if self.front_kind == "had" else " (quantiser")
+                              + " + int4 dot products + dequant epilogue in one launch)" if self.single_launch else
                               " (int4 GEMM + dequant epilogue)")
         g["kernel_ms"] = round(gemm_ms, 5)
         f = {"bound": "hbm", "achieved": round(self.front_bytes() / (front_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -280,6 +280,131 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
         if (it + r < total) consume(ring[r]);
 }
 
+// ---- Quantizer -> Linear4bit for one token (no Hadamard in front) ---------------------------------------------
+// The same construction with quant_rows_kernel's arithmetic as the front: every workgroup takes the row's largest
+// magnitude, the scale and the codes itself (element-wise work on the row out of L2: the scale and every code are the
+// bits of the separate quantiser), keeps the codes in LDS and takes its dot products.  NV: 16-byte pieces of the row
+// per thread (rows of up to 8192 NV halves).  The last segment of a row may be short: its missing codes are zeros in
+// LDS and the lanes past the row's end re-read the row's start.
+template <int NV>
+__global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restrict__ x, int cols8, float clip,
+                                                          const uint8_t* __restrict__ B, const f16* __restrict__ sB,
+                                                          const f16* __restrict__ bias, int N, int ng, f16* __restrict__ Y) {
+    constexpr int NW = 16, R = 2, RD = 5;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[NW];
+    u32* xq = (u32*)smem_raw;                    // codes of the row, a word per piece, zero-filled to whole segments
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int Kb = cols8 * 4, nseg = (Kb + 1023) >> 10;
+    u32x4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = tid + i * 1024;
+        v[i] = x[c < cols8 ? c : 0];
+    }
+    const int groups = (N + R - 1) / R;
+    const int g0 = (blockIdx.x * NW + wave) * ng;
+    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
+    const int total = gcount * nseg;
+    const int my_r = lane >> 5;
+    struct Seg {
+        u32x4 w[R];
+        f16 sb, bi;
+    };
+    int fg = 0, fs = 0;
+    auto fetch = [&](Seg& s) {
+        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int nr = (g0 + fg) * R + r;
+            nr = nr < N ? nr : N - 1;
+            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
+        }
+        int col = (g0 + fg) * R + my_r;
+        col = col < N ? col : N - 1;
+        s.sb = sB[col];
+        s.bi = (bias ? bias : sB)[col];
+        if (fs + 1 < nseg) ++fs;
+        else if (fg + 1 < gcount) { ++fg; fs = 0; }
+    };
+    Seg ring[RD];
+    fetch(ring[0]);
+    fetch(ring[1]);
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const u32 mi = tid + i * 1024 < cols8 ? absmax_bits8(v[i]) : 0u;
+        m = m > mi ? m : mi;
+    }
+    m = wave_max_u32(m);
+    if (lane == 0) red[wave] = m;
+    fetch(ring[2]);
+    fetch(ring[3]);
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < NW; ++w) m = m > red[w] ? m : red[w];
+    const f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
+    const float s = (float)sh;
+    auto codes_of_row = [&](auto form) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = tid + i * 1024;
+            if (c < nseg * 256) xq[c] = c < cols8 ? form(v[i]) : 0u;
+        }
+    };
+    if (fast_quant_ok(m, s)) {
+        const FastRecip fr = make_fast_recip(s);
+        if (clamp_cannot_act(clip, s)) codes_of_row([&](u32x4 h) { return sym_codes8_fast<false>(h, fr); });
+        else codes_of_row([&](u32x4 h) { return sym_codes8_fast<true>(h, fr); });
+    } else {
+        const bool fast = scale_fast_ok(s);
+        const float rs = fast ? 1.0f / s : 0.0f;
+        codes_of_row([&](u32x4 h) { return sym_codes8(h, s, rs, fast); });
+    }
+    fetch(ring[4]);
+    __syncthreads();
+    if (gcount == 0) return;
+    const u32x4* xs = (const u32x4*)xq + lane;
+    int acc[R] = {0, 0};
+    int cg = 0, cs = 0;
+    auto consume = [&](const Seg& sg) {
+        const u32x4 xv = xs[cs * 64];
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_sdot8((int)sg.w[r][d], (int)xv[d], acc[r], false);
+        if (++cs < nseg) return;
+        const bool upper = (lane & 32) != 0;
+        const int give = upper ? acc[0] : acc[1];
+        const int keep = upper ? acc[1] : acc[0];
+        int sum = keep + __shfl_xor(give, 32, QR_WAVE);
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
+        if ((lane & 31) == 0) {
+            const int col = (g0 + cg) * R + my_r;
+            if (col < N) {
+                f16 yo = (f16)(sh * sg.sb) * (f16)(float)sum;
+                if (bias) yo = yo + sg.bi;
+                Y[col] = yo;
+            }
+        }
+        acc[0] = acc[1] = 0;
+        cs = 0;
+        ++cg;
+    };
+    int it = 0;
+    for (; it + RD <= total; it += RD) {
+#pragma unroll
+        for (int r = 0; r < RD; ++r) {
+            consume(ring[r]);
+            fetch(ring[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RD - 1; ++r)
+        if (it + r < total) consume(ring[r]);
+}
+
 }  // namespace
 
 // api.hip: the whole layer for one token where the row is 1024 K halves behind a table of order K <= 32.
@@ -300,5 +425,27 @@ __attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(cons
     if (e != hipSuccess) return (int)e;
     kern<<<dim3(grid), dim3(1024), lds, st>>>((const f16*)x, K, (const f16*)hadK, scale, clip, (const uint8_t*)W,
                                                         (const f16*)sW, (const f16*)bias, (int)N, ng, (f16*)y);
+    return qr_launch_status();
+}
+
+// api.hip: Quantizer + Linear4bit for one token in one launch (rows of up to 32768 halves, a multiple of 64).
+__attribute__((visibility("hidden"))) int qr_internal_token_quant_linear(const void* x, int64_t K, float clip, const void* W,
+                                                                         const void* sW, const void* bias, int64_t N, void* y,
+                                                                         hipStream_t st) {
+    if (K <= 0 || K % 64 != 0 || K > 32768 || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
+    if (((uintptr_t)x & 15) || ((uintptr_t)W & 15)) return QR_E_UNSUPPORTED;
+    const int cols8 = (int)(K / 8), nseg = (cols8 * 4 + 1023) / 1024;
+    const int cus = qr_device().cus;
+    const int64_t groups = (N + 1) / 2;
+    const int ng = (int)((groups + (int64_t)cus * 16 - 1) / ((int64_t)cus * 16));
+    const unsigned grid = (unsigned)(((groups + ng - 1) / ng + 15) / 16);
+    const size_t lds = (size_t)nseg * 1024;
+#define QR_QG(NV)                                                                                                          \
+    quant_gemv_kernel<NV><<<dim3(grid), dim3(1024), lds, st>>>((const u32x4*)x, cols8, clip, (const uint8_t*)W, (const f16*)sW, \
+                                                               (const f16*)bias, (int)N, ng, (f16*)y)
+    if (cols8 <= 1024) QR_QG(1);
+    else if (cols8 <= 2048) QR_QG(2);
+    else QR_QG(4);
+#undef QR_QG
     return qr_launch_status();
 }

@@ -3,6 +3,7 @@ quantiser and its inverse, the paged int4 cache (append, quantise-and-append, si
 the cache) and the cache class the model code drives.  Pages of fp16 (the reference's disable_quant
 debugging mode) are not built."""
 import functools
+import weakref
 import math
 
 import torch
@@ -69,49 +70,75 @@ def matmul_had_cuda(X, dtype):
 # paged int4 cache: kv_data uint8 [pages, layers, 2, heads, page_size, head_dim / 2],
 # kv_param fp16 [pages, layers, 2, heads, page_size, 2] = {scale, zero}
 
-def _check(cond, msg):
-    if not cond:
-        raise RuntimeError(msg)
+_CHECKED = None     # the five cache tensors validated last (weak references), their element counts, their dimensions
 
 
 def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx):
-    """The checks of quarot/kernels/bindings.cpp:118-245 (CHECK_INPUT / CHECK_DIM / CHECK_EQ) as RuntimeError."""
+    """The checks of quarot/kernels/bindings.cpp:118-245 (CHECK_INPUT / CHECK_DIM / CHECK_EQ) as RuntimeError.
+    A decode step passes the same five tensor objects to the append and to the attention of every layer: the
+    objects validated last (same identity, same element counts) are not walked through again."""
+    global _CHECKED
+    seen = _CHECKED
+    if seen is not None:
+        refs, counts, dims = seen
+        if (refs[0]() is kv_data and refs[1]() is kv_param and refs[2]() is kv_indptr and refs[3]() is kv_indices
+                and refs[4]() is last_page_offset
+                and counts == (kv_data.numel(), kv_param.numel(), kv_indptr.numel(), kv_indices.numel(), last_page_offset.numel())):
+            if not (0 <= int(layer_idx) < dims[1]):
+                raise RuntimeError(f"{fn}: layer_idx out of range")
+            return dims
     for name, t in (("kv_data", kv_data), ("kv_param", kv_param), ("kv_indptr", kv_indptr), ("kv_indicies", kv_indices),
                     ("last_page_offset", last_page_offset)):
-        _check(t.is_cuda, f"{fn}: {name} must be a CUDA tensor")
-        _check(t.is_contiguous(), f"{fn}: {name} must be contiguous")
-    _check(kv_data.dim() == 6, f"{fn}: kv_data must be a 6D tensor")
-    _check(kv_param.dim() == 6, f"{fn}: kv_param must be a 6D tensor")
-    _check(kv_indptr.dim() == 1 and kv_indices.dim() == 1 and last_page_offset.dim() == 1,
-           f"{fn}: kv_indptr, kv_indicies and last_page_offset must be 1D tensors")
-    _check(kv_data.dtype == torch.uint8, f"{fn}: kv_data must be uint8 (fp16 pages are not built)")
-    _check(kv_param.dtype == torch.float16, f"{fn}: kv_param must be fp16")
+        if not (t.is_cuda):
+            raise RuntimeError(f"{fn}: {name} must be a CUDA tensor")
+        if not (t.is_contiguous()):
+            raise RuntimeError(f"{fn}: {name} must be contiguous")
+    if not (kv_data.dim() == 6):
+        raise RuntimeError(f"{fn}: kv_data must be a 6D tensor")
+    if not (kv_param.dim() == 6):
+        raise RuntimeError(f"{fn}: kv_param must be a 6D tensor")
+    if not (kv_indptr.dim() == 1 and kv_indices.dim() == 1 and last_page_offset.dim() == 1):
+        raise RuntimeError(f"{fn}: kv_indptr, kv_indicies and last_page_offset must be 1D tensors")
+    if not (kv_data.dtype == torch.uint8):
+        raise RuntimeError(f"{fn}: kv_data must be uint8 (fp16 pages are not built)")
+    if not (kv_param.dtype == torch.float16):
+        raise RuntimeError(f"{fn}: kv_param must be fp16")
     for name, t in (("kv_indptr", kv_indptr), ("kv_indicies", kv_indices), ("last_page_offset", last_page_offset)):
-        _check(t.dtype == torch.int32, f"{fn}: {name} must be int32")
+        if not (t.dtype == torch.int32):
+            raise RuntimeError(f"{fn}: {name} must be int32")
     pages, layers, two, heads, page_size, half_dim = kv_data.shape
-    _check(two == 2 and tuple(kv_param.shape) == (pages, layers, 2, heads, page_size, 2),
-           f"{fn}: kv_param must be [pages, layers, 2, heads, page_size, 2]")
-    _check(half_dim * 2 == 128, f"{fn}: CHECK_EQ(head_dim, 128) failed. {half_dim * 2} vs 128")
-    _check(0 <= int(layer_idx) < layers, f"{fn}: layer_idx out of range")
-    return pages, layers, heads, page_size, half_dim * 2
+    if not (two == 2 and tuple(kv_param.shape) == (pages, layers, 2, heads, page_size, 2)):
+        raise RuntimeError(f"{fn}: kv_param must be [pages, layers, 2, heads, page_size, 2]")
+    if not (half_dim * 2 == 128):
+        raise RuntimeError(f"{fn}: CHECK_EQ(head_dim, 128) failed. {half_dim * 2} vs 128")
+    if not (0 <= int(layer_idx) < layers):
+        raise RuntimeError(f"{fn}: layer_idx out of range")
+    dims = (pages, layers, heads, page_size, half_dim * 2)
+    five = (kv_data, kv_param, kv_indptr, kv_indices, last_page_offset)
+    _CHECKED = (tuple(weakref.ref(t) for t in five), tuple(t.numel() for t in five), dims)
+    return dims
 
 
 def _append(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     batch = last_page_offset.shape[0]
-    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    if not (kv_indptr.shape[0] == batch + 1):
+        raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
     for name, t in (("k", k), ("v", v), ("k_param", k_param), ("v_param", v_param)):
-        _check(t.is_cuda and t.is_contiguous() and t.dim() == 3, f"{fn}: {name} must be a contiguous 3D CUDA tensor")
-    _check(k.shape == v.shape and k.dtype == v.dtype == torch.uint8 and tuple(k.shape[1:]) == (heads, head_dim // 2),
-           f"{fn}: k and v must be uint8 [tokens, heads, head_dim / 2]")
+        if not (t.is_cuda and t.is_contiguous() and t.dim() == 3):
+            raise RuntimeError(f"{fn}: {name} must be a contiguous 3D CUDA tensor")
+    if not (k.shape == v.shape and k.dtype == v.dtype == torch.uint8 and tuple(k.shape[1:]) == (heads, head_dim // 2)):
+        raise RuntimeError(f"{fn}: k and v must be uint8 [tokens, heads, head_dim / 2]")
     tokens = k.shape[0]
     for name, t in (("k_param", k_param), ("v_param", v_param)):
-        _check(t.dtype == torch.float16 and tuple(t.shape) == (tokens, heads, 2), f"{fn}: {name} must be fp16 [tokens, heads, 2]")
+        if not (t.dtype == torch.float16 and tuple(t.shape) == (tokens, heads, 2)):
+            raise RuntimeError(f"{fn}: {name} must be fp16 [tokens, heads, 2]")
     if seqlen_indptr is None:
-        _check(tokens == batch, f"{fn}: one token per sequence expected")
+        if not (tokens == batch):
+            raise RuntimeError(f"{fn}: one token per sequence expected")
     else:
-        _check(seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32
-               and tuple(seqlen_indptr.shape) == (batch + 1,), f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
+        if not (seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32 and tuple(seqlen_indptr.shape) == (batch + 1,)):
+            raise RuntimeError(f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
     dev = kv_data.device
     with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_kv_append_i4(
@@ -144,17 +171,20 @@ def quantize_append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_of
     fn = "quantize_append_kv_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     batch = last_page_offset.shape[0]
-    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    if not (kv_indptr.shape[0] == batch + 1):
+        raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
     for name, t in (("k", k), ("v", v)):
-        _check(t.is_cuda and t.is_contiguous() and t.dtype == torch.float16 and t.dim() == 3
-               and tuple(t.shape[1:]) == (heads, head_dim), f"{fn}: {name} must be a contiguous fp16 [tokens, heads, 128] CUDA tensor")
-    _check(k.shape == v.shape, f"{fn}: k and v differ in shape")
+        if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float16 and t.dim() == 3 and tuple(t.shape[1:]) == (heads, head_dim)):
+            raise RuntimeError(f"{fn}: {name} must be a contiguous fp16 [tokens, heads, 128] CUDA tensor")
+    if not (k.shape == v.shape):
+        raise RuntimeError(f"{fn}: k and v differ in shape")
     tokens = k.shape[0]
     if seqlen_indptr is None:
-        _check(tokens == batch, f"{fn}: one token per sequence expected")
+        if not (tokens == batch):
+            raise RuntimeError(f"{fn}: one token per sequence expected")
     else:
-        _check(seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32
-               and tuple(seqlen_indptr.shape) == (batch + 1,), f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
+        if not (seqlen_indptr.is_cuda and seqlen_indptr.is_contiguous() and seqlen_indptr.dtype == torch.int32 and tuple(seqlen_indptr.shape) == (batch + 1,)):
+            raise RuntimeError(f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
     dev = kv_data.device
     with _lib.on_device(dev):
         _lib.check(_lib.lib().qr_kv_quant_append_f16_i4(
@@ -182,14 +212,21 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
     fn = "batch_decode_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     for name, t in (("o", o), ("q", q)):
-        _check(t.is_cuda and t.is_contiguous(), f"{fn}: {name} must be a contiguous CUDA tensor")
-        _check(t.dim() == 3, f"{fn}: {name} must be a 3D tensor")
-        _check(t.dtype == torch.float16, f"{fn}: {name} must be fp16")
-    _check(o.shape == q.shape, f"{fn}: o.size() != q.size()")
+        if not (t.is_cuda and t.is_contiguous()):
+            raise RuntimeError(f"{fn}: {name} must be a contiguous CUDA tensor")
+        if not (t.dim() == 3):
+            raise RuntimeError(f"{fn}: {name} must be a 3D tensor")
+        if not (t.dtype == torch.float16):
+            raise RuntimeError(f"{fn}: {name} must be fp16")
+    if not (o.shape == q.shape):
+        raise RuntimeError(f"{fn}: o.size() != q.size()")
     batch = o.shape[0]
-    _check(tuple(q.shape[1:]) == (heads, head_dim), f"{fn}: q must be [batch_size, {heads}, {head_dim}]")
-    _check(kv_indptr.shape[0] == batch + 1, f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
-    _check(last_page_offset.shape[0] == batch, f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
+    if not (tuple(q.shape[1:]) == (heads, head_dim)):
+        raise RuntimeError(f"{fn}: q must be [batch_size, {heads}, {head_dim}]")
+    if not (kv_indptr.shape[0] == batch + 1):
+        raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    if not (last_page_offset.shape[0] == batch):
+        raise RuntimeError(f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
     dev = kv_data.device
     with _lib.on_device(dev):
         ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len), dev.index) if max_seq_len else 0
@@ -264,13 +301,17 @@ class MultiLayerPagedKVCache4Bit:
     def _decode_workspace(self, num_heads):
         """Scratch for decode attention split along the sequence, kept with the cache (every layer of every decode
         step would otherwise allocate its own): sized for the longer of the current and the maximum length."""
+        key = (self.length, num_heads)
+        if getattr(self, "_decode_ws_key", None) == key:
+            return self._decode_ws
         dev = self.pages.device
         with _lib.on_device(dev):
             need = max((_decode_workspace_bytes(self.batch_size, num_heads, int(n), dev.index)
                         for n in (self.length, self.max_seq_len) if n), default=0)
         ws = getattr(self, "_decode_ws", None)
         if need and (ws is None or ws.numel() < need):
-            ws = self._decode_ws = torch.empty((need,), dtype=torch.uint8, device=dev)
+            ws = torch.empty((need,), dtype=torch.uint8, device=dev)
+        self._decode_ws, self._decode_ws_key = ws, key
         return ws
 
     def _ensure_page_cnt_per_batch(self, expected_page_cnt_per_batch):
