@@ -235,8 +235,8 @@ int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, const void*
  * 70B down_proj, 28672 = 1024 x 28), mode QR_DTYPE_F16: a single kernel in which every workgroup
  * transforms and quantises the row itself and goes straight on to its dot products -- the same codes,
  * scale, sums and epilogue, so y carries the same bits, and the weight stream starts while the row is
- * still being transformed.  ONE token with had_K == 0 (K up to 32768): likewise one kernel, every
- * workgroup quantising the row itself.  The workspace is checked as always; what it holds afterwards
+ * still being transformed.  ONE or TWO tokens with had_K == 0 (K up to 32768): likewise one kernel, every
+ * workgroup quantising the rows itself.  The workspace is checked as always; what it holds afterwards
  * is unspecified.
  *   x fp16 [M, K]; had_K, hadK, mode, scale as in qr_hadamard_quantize_f16_i4; W uint8 [N, K/2],
  *   sW fp16 [N], bias fp16 [N] or NULL -> y fp16 [M, N].

@@ -48,8 +48,8 @@ extern "C" int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int 
                                                           (hipStream_t)stream);
         if (rc1 != QR_E_UNSUPPORTED) return rc1;
     }
-    if (M == 1 && had_K == 0 && ((uintptr_t)y & 1) == 0) {
-        const int rc1 = qr_internal_token_quant_linear(x, K, clip, W, sW, bias_or_null, N, y, (hipStream_t)stream);
+    if (M <= 2 && had_K == 0 && ((uintptr_t)y & 1) == 0) {
+        const int rc1 = qr_internal_token_quant_linear(x, M, K, clip, W, sW, bias_or_null, N, y, (hipStream_t)stream);
         if (rc1 != QR_E_UNSUPPORTED) return rc1;
     }
     int rc = had_K == 0 ? qr_quantize_rows_f16_i4(x, clip, M, K, codes, scales, stream)

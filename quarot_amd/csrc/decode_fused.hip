@@ -405,6 +405,159 @@ __global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restric
         if (it + r < total) consume(ring[r]);
 }
 
+// ---- Quantizer -> Linear4bit for two tokens -------------------------------------------------------------------------
+// MB tokens: 16 / MB waves quantise each row (a lane keeps up to eight 16-byte pieces of its row in registers: rows of up
+// to 65536 / MB halves) and every wave then takes its pairs of weight rows against all tokens.  Built for MB = 2 only:
+// with four and eight tokens every workgroup pulls 64 / 128 KB of rows through its CU's memory path before its weight
+// stream can be consumed, and the launch (70B gate_up: 43.7 / 41.8 us) is no faster than the quantiser kernel followed
+// by the shared-token decode kernel (43.5 / 43.7 us); with two tokens it is 38.2 against 43.4 us.
+template <int MB>
+__global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __restrict__ x, int M, int cols8, float clip,
+                                                             const uint8_t* __restrict__ B, const f16* __restrict__ sB,
+                                                             const f16* __restrict__ bias, int N, int ng, f16* __restrict__ Y) {
+    constexpr int NW = 16, R = 2, RD = 5, WPR = NW / MB, NV = 8, NS = R * MB;
+    extern __shared__ f32x4 smem_raw[];
+    __shared__ u32 red[NW];
+    __shared__ f16 sc[MB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int Kb = cols8 * 4, nseg = (Kb + 1023) >> 10;
+    u32* xq = (u32*)smem_raw;                    // [MB][nseg * 256] words: codes of the rows, zero-filled to whole segments
+    const int row = wave / WPR, part = wave % WPR;
+    const u32x4* xr = x + (int64_t)(row < M ? row : M - 1) * cols8;
+    u32x4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (i * WPR + part) * 64 + lane;
+        v[i] = xr[c < cols8 ? c : 0];
+    }
+    const int groups = (N + R - 1) / R;
+    const int g0 = (blockIdx.x * NW + wave) * ng;
+    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
+    const int total = gcount * nseg;
+    // which of a pair's NS sums this lane stores at the end of the exchange (log2(NS) lane bits from bit 5 downwards)
+    constexpr int LV = NS == 2 ? 1 : NS == 4 ? 2 : NS == 8 ? 3 : 4;
+    const int vidx = lane >> (6 - LV);
+    const int my_m = vidx / R, my_r = vidx % R;
+    struct Seg {
+        u32x4 w[R];
+        f16 sb, bi;
+    };
+    int fg = 0, fs = 0;
+    auto fetch = [&](Seg& s) {
+        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int nr = (g0 + fg) * R + r;
+            nr = nr < N ? nr : N - 1;
+            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
+        }
+        int col = (g0 + fg) * R + my_r;
+        col = col < N ? col : N - 1;
+        s.sb = sB[col];
+        s.bi = (bias ? bias : sB)[col];
+        if (fs + 1 < nseg) ++fs;
+        else if (fg + 1 < gcount) { ++fg; fs = 0; }
+    };
+    Seg ring[RD];
+    fetch(ring[0]);
+    fetch(ring[1]);
+    u32 m = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const u32 mi = (i * WPR + part) * 64 + lane < cols8 ? absmax_bits8(v[i]) : 0u;
+        m = m > mi ? m : mi;
+    }
+    m = wave_max_u32(m);
+    if (lane == 0) red[wave] = m;
+    fetch(ring[2]);
+    fetch(ring[3]);
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < WPR; ++w) m = m > red[row * WPR + w] ? m : red[row * WPR + w];
+    const f16 sh = quantizer_scale(f16_from_bits((unsigned short)m), clip);
+    const float s = (float)sh;
+    if (part == 0 && lane == 0) sc[row] = sh;
+    u32* xrow = xq + row * (nseg * 256);
+    auto codes_of_row = [&](auto form) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int c = (i * WPR + part) * 64 + lane;
+            if (c < nseg * 256) xrow[c] = c < cols8 ? form(v[i]) : 0u;
+        }
+    };
+    if (fast_quant_ok(m, s)) {                   // (uniform over the waves of a row)
+        const FastRecip fr = make_fast_recip(s);
+        if (clamp_cannot_act(clip, s)) codes_of_row([&](u32x4 h) { return sym_codes8_fast<false>(h, fr); });
+        else codes_of_row([&](u32x4 h) { return sym_codes8_fast<true>(h, fr); });
+    } else {
+        const bool fast = scale_fast_ok(s);
+        const float rs = fast ? 1.0f / s : 0.0f;
+        codes_of_row([&](u32x4 h) { return sym_codes8(h, s, rs, fast); });
+    }
+    fetch(ring[4]);
+    __syncthreads();
+    if (gcount == 0) return;
+    const f16 my_sa = sc[my_m < M ? my_m : M - 1];
+    const u32x4* xs = (const u32x4*)xq + lane;
+    int acc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) acc[i] = 0;
+    int cg = 0, cs = 0;
+    auto consume = [&](const Seg& sg) {
+#pragma unroll
+        for (int mt = 0; mt < MB; ++mt) {
+            const u32x4 xv = xs[(mt * nseg + cs) * 64];
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    acc[mt * R + r] = __builtin_amdgcn_sdot8((int)sg.w[r][d], (int)xv[d], acc[mt * R + r], false);
+        }
+        if (++cs < nseg) return;
+        // end of a pair of rows: halving exchange (each step gives away half of the values a lane still holds)
+        int vals[NS];
+#pragma unroll
+        for (int i = 0; i < NS; ++i) vals[i] = acc[i];
+        int off = 32;
+#pragma unroll
+        for (int cur = NS; cur > 1; cur >>= 1) {
+            const bool upper = (lane & off) != 0;
+#pragma unroll
+            for (int i = 0; i < cur / 2; ++i) {
+                const int give = upper ? vals[i] : vals[i + cur / 2];
+                const int keep = upper ? vals[i + cur / 2] : vals[i];
+                vals[i] = keep + __shfl_xor(give, off, QR_WAVE);
+            }
+            off >>= 1;
+        }
+        int sum = vals[0];
+        for (; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
+        if ((lane & ((1 << (6 - LV)) - 1)) == 0) {
+            const int col = (g0 + cg) * R + my_r;
+            if (my_m < M && col < N) {
+                f16 yo = (f16)(my_sa * sg.sb) * (f16)(float)sum;
+                if (bias) yo = yo + sg.bi;
+                Y[(int64_t)my_m * N + col] = yo;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NS; ++i) acc[i] = 0;
+        cs = 0;
+        ++cg;
+    };
+    int it = 0;
+    for (; it + RD <= total; it += RD) {
+#pragma unroll
+        for (int r = 0; r < RD; ++r) {
+            consume(ring[r]);
+            fetch(ring[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RD - 1; ++r)
+        if (it + r < total) consume(ring[r]);
+}
+
 }  // namespace
 
 // api.hip: the whole layer for one token where the row is 1024 K halves behind a table of order K <= 32.
@@ -428,18 +581,23 @@ __attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(cons
     return qr_launch_status();
 }
 
-// api.hip: Quantizer + Linear4bit for one token in one launch (rows of up to 32768 halves, a multiple of 64).
-__attribute__((visibility("hidden"))) int qr_internal_token_quant_linear(const void* x, int64_t K, float clip, const void* W,
-                                                                         const void* sW, const void* bias, int64_t N, void* y,
-                                                                         hipStream_t st) {
-    if (K <= 0 || K % 64 != 0 || K > 32768 || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
+// api.hip: Quantizer + Linear4bit for one or two tokens in one launch (rows of up to 32768 halves, a multiple of 64).
+__attribute__((visibility("hidden"))) int qr_internal_token_quant_linear(const void* x, int64_t M, int64_t K, float clip,
+                                                                         const void* W, const void* sW, const void* bias,
+                                                                         int64_t N, void* y, hipStream_t st) {
+    if (M < 1 || M > 2 || K <= 0 || K % 64 != 0 || K > 32768 || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)W & 15)) return QR_E_UNSUPPORTED;
     const int cols8 = (int)(K / 8), nseg = (cols8 * 4 + 1023) / 1024;
     const int cus = qr_device().cus;
     const int64_t groups = (N + 1) / 2;
     const int ng = (int)((groups + (int64_t)cus * 16 - 1) / ((int64_t)cus * 16));
     const unsigned grid = (unsigned)(((groups + ng - 1) / ng + 15) / 16);
-    const size_t lds = (size_t)nseg * 1024;
+    const size_t lds = (size_t)nseg * 1024 * (size_t)M;
+    if (M == 2) {
+        quant_gemv_mt_kernel<2><<<dim3(grid), dim3(1024), lds, st>>>((const u32x4*)x, 2, cols8, clip, (const uint8_t*)W,
+                                                                     (const f16*)sW, (const f16*)bias, (int)N, ng, (f16*)y);
+        return qr_launch_status();
+    }
 #define QR_QG(NV)                                                                                                          \
     quant_gemv_kernel<NV><<<dim3(grid), dim3(1024), lds, st>>>((const u32x4*)x, cols8, clip, (const uint8_t*)W, (const f16*)sW, \
                                                                (const f16*)bias, (int)N, ng, (f16*)y)

@@ -102,9 +102,10 @@ int qr_internal_heads_matrix_quantize(const void* x, int64_t rows, int heads, co
 int qr_internal_token_hadamard_linear(const void* x, int n, int K, const void* hadK, float scale, float clip,
                                       const void* W, const void* sW, const void* bias, int64_t N, void* y, hipStream_t st);
 
-// decode_fused.hip: quantiser + linear layer of ONE token in one launch (rows of up to 32768 halves)
-int qr_internal_token_quant_linear(const void* x, int64_t K, float clip, const void* W, const void* sW, const void* bias,
-                                   int64_t N, void* y, hipStream_t st);
+// decode_fused.hip: quantiser + linear layer of one or two tokens in one launch; QR_E_UNSUPPORTED, with nothing
+// launched, for anything else
+int qr_internal_token_quant_linear(const void* x, int64_t M, int64_t K, float clip, const void* W, const void* sW,
+                                   const void* bias, int64_t N, void* y, hipStream_t st);
 
 static inline int qr_launch_status() {
     hipError_t e = hipGetLastError();

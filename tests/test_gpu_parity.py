@@ -1361,13 +1361,14 @@ def test_one_token_hadamard_linear_in_one_launch(n):
         assert np.array_equal(bits(got.cpu().numpy()), bits(want.cpu().numpy())), (n, case)
 
 
-def test_one_token_quantizer_linear_in_one_launch():
-    """One token through Quantizer -> Linear4bit: qr_quantized_linear_f16 (had_K = 0) runs ONE kernel in which every
-    workgroup quantises the row itself.  Bit for bit the two-launch chain, on rows of 64 to 32768 columns (short last
-    segments of the weight rows included), one to 57344 weight rows, with bias, with a clip that lets the clamp act,
-    on rows of zeros and rows holding an infinity or a NaN; and the oracle's Quantizer + Linear4bit on the smaller
-    shapes."""
-    rng = np.random.default_rng(4)
+@pytest.mark.parametrize("M", [1, 2])
+def test_one_or_two_tokens_quantizer_linear_in_one_launch(M):
+    """One or two tokens through Quantizer -> Linear4bit: qr_quantized_linear_f16 (had_K = 0) runs ONE kernel in which
+    every workgroup quantises the rows itself.  Bit for bit the two-launch chain, on rows of 64 to 32768 columns (short
+    last segments of the weight rows included), one to 57344 weight rows, with bias, with a clip that lets the clamp
+    act, on rows of zeros and rows holding an infinity or a NaN (with two tokens: in the second row, beside a finite
+    first one); and the oracle's Quantizer + Linear4bit on the smaller shapes."""
+    rng = np.random.default_rng(4 + M)
     for K, N, bias, clip in [(8192, 57344, False, 1.0), (4096, 4097, True, 1.0), (4096, 11008, False, 0.9), (5120, 300, True, 1.0),
                              (64, 7, False, 1.0), (11008, 4096, False, 1.0), (32768, 33, True, 1.0), (8192, 1, False, 1.0),
                              (2112, 513, True, 0.8), (16448, 64, False, 1.0)]:
@@ -1375,18 +1376,20 @@ def test_one_token_quantizer_linear_in_one_launch():
         sw = gpu((np.abs(rng.standard_normal((N, 1))) * 0.01 + 0.001).astype(F16))
         b = gpu(rng.standard_normal(N).astype(F16)) if bias else None
         for case in ("plain", "outliers", "zeros", "inf", "nan"):
-            x = synth_x(1, K, seed=K + N, outliers=case == "outliers")
+            x = synth_x(M, K, seed=K + N, outliers=case == "outliers")
+            if M == 2:
+                x[1] *= F16(0.37)
             if case == "zeros":
-                x[:] = 0
+                x[M - 1] = 0
             elif case == "inf":
-                x[0, K // 2] = -np.inf
+                x[M - 1, K // 2] = -np.inf
             elif case == "nan":
-                x[0, K - 1] = np.nan
+                x[M - 1, K - 1] = np.nan
             xg = gpu(x)
             got = quarot_amd.quantized_linear(xg, w, sw, b, None, 0, clip_ratio=clip)
             q, s = quarot_amd.quantize_rows(xg, clip)
             want = quarot_amd.linear_i4(q, s, w, sw, b)
-            assert got.shape == (1, N) and np.array_equal(bits(got.cpu().numpy()), bits(want.cpu().numpy())), (K, N, case)
+            assert got.shape == (M, N) and np.array_equal(bits(got.cpu().numpy()), bits(want.cpu().numpy())), (K, N, case)
             if N <= 4097 and case in ("plain", "outliers"):
                 xq, xs = o.quantizer(x, clip)
                 ref_y = o.linear4bit(xq, xs, w.cpu().numpy(), sw.cpu().numpy(), None if b is None else b.cpu().numpy())
