@@ -645,16 +645,19 @@ def run_attention(name, dev, steps, warmup, repeats, kernel_reps, cpu_baseline):
     specs = cache.get_cache_specs_for_flash_infer(None)
     qh = kv.matmul_had_cuda(q1.view(B, H, 128), torch.float16)
     out = torch.empty_like(qh)
-    a_ms = kernel_ms(lambda: kv.batch_decode_i4(out, qh, **specs, layer_idx=0, max_seq_len=S), kernel_reps)
+    # the step's one launch by itself: the new token quantised and stored, the query transformed, attention over the cache
+    k3, v3, q3 = k1.view(B, H, 128), v1.view(B, H, 128), q1.view(B, H, 128)
+    a_ms = kernel_ms(lambda: kv.batch_decode_i4(out, q3, **specs, layer_idx=0, max_seq_len=S, q_hadamard=True,
+                                                append=(k3, v3, True)), kernel_reps)
     cache_bytes = B * H * S * (2 * 64 + 2 * 4)               # codes and {scale, zero} of K and V
     roof = {"bound": "hbm", "achieved": round(cache_bytes / (a_ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s"}
     roof["frac"] = round(roof["achieved"] / roof["peak"], 4)
-    roof["kernel"] = "paged_decode_i4_kernel (single-query attention, in-register dequantisation)"
+    roof["kernel"] = "paged_decode_i4_kernel (quantise-and-append of the new token, query Hadamard and single-query attention with in-register dequantisation, one launch)"
     roof["kernel_ms"] = round(a_ms, 5)
     res = {"ms": ms, "value": round(cache_bytes / (ms * 1e-3) / 1e9, 1), "unit": "GB/s", "timing": sp, "roofline": roof,
            "step_frac": round(cache_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
            "workload": f"{name}: decode step on the paged int4 KV cache, {B} sequences x {S} tokens x {H} heads x 128, pages of {P}: "
-                       "quantise-and-append of one token per sequence, query Hadamard, attention over the cache"}
+                       "quantise-and-append of one token per sequence, query Hadamard, attention over the cache (one launch)"}
     if cpu_baseline:
         from oracle import quarot_oracle as o
         nb = 1                                               # one sequence, all heads

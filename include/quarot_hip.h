@@ -345,6 +345,26 @@ int qr_batch_decode_qhad_i4(void* o, const void* q, const void* kv_data, const v
                             size_t workspace_bytes, void* stream);
 
 /*
+ * One decode step of the paged cache in ONE launch: qr_kv_quant_append_f16_i4 (one new token per sequence,
+ * append_indptr NULL) followed by qr_batch_decode_i4 / qr_batch_decode_qhad_i4 -- what
+ * MultiLayerPagedKVCache4Bit.update and the callable it returns do for a decode step
+ * (quarot/transformers/kv_cache.py:104-129,224-251).  The page tables already count the new token (it is the
+ * LAST position of its sequence, as for qr_kv_quant_append_f16_i4); the first wave of every (sequence, head)
+ * quantises the token's key (through H_128 when k_had_mode = 1) and value with the arithmetic of that entry
+ * point -- the same codes, scales and zeros, written to the same page slots -- and attends to them from its
+ * registers while the other waves walk the cached positions.
+ *   k, v fp16 [batch_size, num_heads, 128] (16-byte aligned); q_had_mode 0 / 1 as the two entry points above;
+ *   everything else as qr_batch_decode_i4.  A sequence whose page list is empty is skipped by the append and
+ *   gets a NaN output row, as there.
+ */
+int qr_kv_quant_append_batch_decode_f16_i4(void* o, const void* q, int q_had_mode, const void* k, const void* v,
+                                           int k_had_mode, void* kv_data, void* kv_param, const void* kv_indptr,
+                                           const void* kv_indices, const void* last_page_offset,
+                                           int64_t num_pages, int num_layers, int layer_idx, int num_heads,
+                                           int page_size, int head_dim, int64_t batch_size, int64_t max_seq_len,
+                                           void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Measurement aids.  NO counterpart in the reference and no caller in the product path: kernels whose
  * work is known exactly, run by bench.py next to the workloads to calibrate the rooflines.
  *

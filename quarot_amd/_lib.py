@@ -44,6 +44,8 @@ SIGNATURES = {
                                   _c.c_size_t, _ptr)),
     "qr_batch_decode_qhad_i4": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int, _i64, _i64, _ptr,
                                        _c.c_size_t, _ptr)),
+    "qr_kv_quant_append_batch_decode_f16_i4": (_int, (_ptr, _ptr, _int, _ptr, _ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int,
+                                                      _int, _int, _int, _int, _i64, _i64, _ptr, _c.c_size_t, _ptr)),
     "qr_calib_mfma_i8": (_int, (_int, _int, _int, _ptr, _ptr)),
     "qr_calib_copy": (_int, (_ptr, _ptr, _i64, _ptr)),
 }

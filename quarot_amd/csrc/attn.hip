@@ -1,6 +1,6 @@
 // Paged int4 KV cache: appending quantised vectors to their pages, and single-query (decode) attention
 // over the cache with the dequantisation done in registers.
-#include "qr_paged.h"
+#include "qr_kvq.h"
 
 namespace {
 
@@ -90,18 +90,25 @@ __device__ __forceinline__ float row_rotate(float v) {   // DPP row_ror within e
 
 // ALIGNED: page_size is a multiple of 16, so the 16 positions of a wave step lie in one page.
 // NW: waves per workgroup (4 or 16): a (sequence, head) gets NW * splits waves in all.
-template <bool ALIGNED, int NW>
+// APPEND: the sequence's LAST position is the token of this step, and its key and value arrive as fp16 vectors
+// (knew, vnew: [batch, heads, 128]) instead of lying in the cache already: the first wave of the (sequence, head)
+// quantises them itself (kv_quant_one_vector: the bits of the quantise-and-append kernel), writes codes and parameters
+// to the position's page slot, and takes the position into its softmax state from its own registers; the walk over
+// the cache stops one position short.  A decode step is then ONE launch instead of append + attention.
+template <bool ALIGNED, int NW, bool APPEND = false>
 __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void paged_decode_i4_kernel(
     const f16* __restrict__ q, PagedKV c, f16* __restrict__ o, float sm_scale_log2, int splits, float* __restrict__ part,
-    int q_had) {
+    int q_had, const u32x4* __restrict__ knew = nullptr, const u32x4* __restrict__ vnew = nullptr, int k_had = 0) {
     __shared__ float st[NW * 4 * 4 * 36];                  // [wave * 4 + row][quarter][m, d, -, -, acc[32]]
     __shared__ float st2[(NW / 2) * 128 * 3];              // second merge level: [part][dimension][m, d, o]
+    __shared__ u32x4 fresh[APPEND ? 26 : 1];               // APPEND: staging [16], the new key's codes [4], the value's [4], parameters
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int slot = lane >> 2, c4 = lane & 3;
     const int bh = blockIdx.x / splits, sp = blockIdx.x - bh * splits;
     const int b = bh / c.num_heads, h = bh - b * c.num_heads;
     const int p0 = c.indptr[b], npages = c.indptr[b + 1] - p0;
-    const int seq_len = npages > 0 ? (npages - 1) * c.page_size + c.last_page_offset[b] : 0;
+    const int seq_all = npages > 0 ? (npages - 1) * c.page_size + c.last_page_offset[b] : 0;
+    const int seq_len = APPEND ? seq_all - 1 : seq_all;     // positions read from the cache
     if (npages <= 0) {
         // A sequence without pages (uniform over the workgroup): nothing may be read -- its slice of kv_indices is
         // empty, and so may be the whole list and the page pool.  The result is the empty softmax state, i.e. the
@@ -119,6 +126,40 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
             }
         }
         return;
+    }
+
+    const bool appends = APPEND && sp == 0 && wave == 0;    // wave-uniform
+    if (APPEND && appends) {
+        const int64_t vec = (int64_t)bh * 16;
+        u32 W[8];
+        f16 sc, zp;
+        const int pos = seq_all - 1, it = pos / c.page_size, entry = pos - it * c.page_size;
+        const int64_t page = c.indices[p0 + it];
+        const bool page_ok = page >= 0 && page < c.num_pages;
+        const float hs = 0.08838834764831845f;                 // 1 / sqrt(128)
+        const u32x4 piece[2] = {knew[vec + (lane & 15)], vnew[vec + (lane & 15)]};      // both in flight at once
+#pragma unroll
+        for (int kv = 0; kv < 2; ++kv) {
+            if (kv == 0 && k_had) kv_quant_one_vector<true>(piece[0], fresh, hs, W, sc, zp);
+            else kv_quant_one_vector<false>(piece[kv], fresh, hs, W, sc, zp);
+            const u32 prm = pack_scale_zero(sc, zp);
+            const int hh = lane >> 5;
+            if (page_ok && (lane & 31) == 0) {
+                const int64_t s = paged_slot(c, page, kv, h, entry);
+                u32x4* dst = (u32x4*)c.data + s * 4 + 2 * hh;
+                dst[0] = u32x4{W[0], W[1], W[2], W[3]};
+                dst[1] = u32x4{W[4], W[5], W[6], W[7]};
+                if (hh == 0) c.param[s] = prm;
+            }
+            // for the position's own turn after the walk: pieces 2 hh, 2 hh + 1 of the 64 code bytes, and the parameters
+            if ((lane & 31) == 0) {
+                fresh[16 + 4 * kv + 2 * hh] = u32x4{W[0], W[1], W[2], W[3]};
+                fresh[16 + 4 * kv + 2 * hh + 1] = u32x4{W[4], W[5], W[6], W[7]};
+                if (hh == 0) ((u32*)(fresh + 24))[kv] = page_ok ? prm : 0u;
+                if (hh == 0 && kv == 0) ((u32*)(fresh + 24))[2] = page_ok ? 1u : 0u;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 
     // this lane's 32 query values as fp16 pairs in the order the codes are consumed: word j of a 16-byte
@@ -324,6 +365,21 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
         if (g + gs < chunks) consume(sb);                  // (no loads inside: the branch does not disturb the wait counts)
         __builtin_amdgcn_sched_barrier(0);
     }
+    if (APPEND && appends) {
+        // the new position, from the codes this wave made: lane group 0 takes it, the others sit the turn out
+        Step tn;
+        const u32* prm = (const u32*)(fresh + 24);
+        const bool valid = prm[2] != 0u;
+#pragma unroll
+        for (int u = 0; u < AU; ++u) {
+            tn.kw[u] = fresh[16 + c4];
+            tn.vw[u] = fresh[20 + c4];
+            tn.kp[u] = prm[0];
+            tn.vp[u] = prm[1];
+            tn.ok[u] = u == 0 && slot == 0 && valid;
+        }
+        consume(tn);
+    }
     // ---- merge: first the four lane groups of each row of 16 lanes (two DPP rotations: every lane ends
     // with its row's state), then the NW * 4 row states of the workgroup through LDS
 #pragma unroll
@@ -509,7 +565,8 @@ namespace {
 int batch_decode(void* o, const void* q, const void* kv_data, const void* kv_param, const void* kv_indptr,
                  const void* kv_indices, const void* last_page_offset, int64_t num_pages, int num_layers, int layer_idx,
                  int num_heads, int page_size, int head_dim, int64_t batch_size, int64_t max_seq_len, void* workspace,
-                 size_t workspace_bytes, void* stream, int q_had) {
+                 size_t workspace_bytes, void* stream, int q_had, const void* knew = nullptr, const void* vnew = nullptr,
+                 int k_had = 0) {
     const int rc = check_cache(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
                                num_heads, page_size, head_dim, batch_size);
     if (rc != QR_OK) return rc;
@@ -528,8 +585,14 @@ int batch_decode(void* o, const void* q, const void* kv_data, const void* kv_par
     const unsigned grid = (unsigned)(batch_size * num_heads * splits);
     hipStream_t st = (hipStream_t)stream;
 #define QR_DECODE(AL, NWV)                                                                                              \
-    paged_decode_i4_kernel<AL, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits,      \
-                                                                          (float*)workspace, q_had)
+    do {                                                                                                                \
+        if (knew)                                                                                                       \
+            paged_decode_i4_kernel<AL, NWV, true><<<dim3(grid), dim3(64 * NWV), 0, st>>>(                               \
+                (const f16*)q, c, (f16*)o, sm, splits, (float*)workspace, q_had, (const u32x4*)knew, (const u32x4*)vnew, k_had); \
+        else                                                                                                            \
+            paged_decode_i4_kernel<AL, NWV><<<dim3(grid), dim3(64 * NWV), 0, st>>>((const f16*)q, c, (f16*)o, sm, splits, \
+                                                                                  (float*)workspace, q_had);           \
+    } while (0)
     if (page_size % 16 == 0) {
         if (plan.nw == 16) QR_DECODE(true, 16);
         else if (plan.nw == 8) QR_DECODE(true, 8);
@@ -562,4 +625,23 @@ extern "C" int qr_batch_decode_qhad_i4(void* o, const void* q, const void* kv_da
                                        int64_t max_seq_len, void* workspace, size_t workspace_bytes, void* stream) {
     return batch_decode(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
                         num_heads, page_size, head_dim, batch_size, max_seq_len, workspace, workspace_bytes, stream, 1);
+}
+
+// One decode step in one launch: the new token's key and value (fp16 [batch, heads, 128], one token per sequence, its
+// place the LAST position of the sequence as the page tables already count it) are quantised inside the attention kernel
+// -- the codes and parameters of qr_kv_quant_append_f16_i4, written to the same page slots -- and attended to along with
+// the cached positions: qr_kv_quant_append_f16_i4 followed by qr_batch_decode_i4 / _qhad_i4
+// (MultiLayerPagedKVCache4Bit.update and the callable it returns, quarot/transformers/kv_cache.py:104-129,224-251).
+extern "C" int qr_kv_quant_append_batch_decode_f16_i4(void* o, const void* q, int q_had_mode, const void* k, const void* v,
+                                                      int k_had_mode, void* kv_data, void* kv_param, const void* kv_indptr,
+                                                      const void* kv_indices, const void* last_page_offset, int64_t num_pages,
+                                                      int num_layers, int layer_idx, int num_heads, int page_size, int head_dim,
+                                                      int64_t batch_size, int64_t max_seq_len, void* workspace,
+                                                      size_t workspace_bytes, void* stream) {
+    if ((q_had_mode != 0 && q_had_mode != 1) || (k_had_mode != 0 && k_had_mode != 1)) return QR_E_DTYPE;
+    if (batch_size > 0 && (!k || !v)) return QR_E_NULL;
+    if (((uintptr_t)k & 15) || ((uintptr_t)v & 15)) return QR_E_ALIGN;
+    return batch_decode(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx,
+                        num_heads, page_size, head_dim, batch_size, max_seq_len, workspace, workspace_bytes, stream, q_had_mode,
+                        k, v, k_had_mode);
 }

@@ -1,7 +1,7 @@
 // KV-cache path: per-head Hadamard (optional) + per-vector asymmetric int4 quantise/pack, and the
 // inverse dequantiser.  A vector of `dim` halves is spread over dim/8 adjacent lanes, 16 bytes each;
 // a wave handles 512/dim vectors, so all global accesses are full-width and coalesced.
-#include "qr_paged.h"
+#include "qr_kvq.h"
 
 namespace {
 
@@ -48,41 +48,6 @@ __device__ __forceinline__ f16x2 kv_pair_min(f16x2 p) {
     else r = __builtin_amdgcn_ds_swizzle(i, 0x401F);
     return __builtin_elementwise_min(p, __builtin_bit_cast(f16x2, r));
 }
-
-// Eight codes clamp(round_half_even(fp16(fp16(x + zero) / scale)), 0, 15) for all-finite input: the
-// add is one packed fp16 add, the division the one-multiplication form of sym_codes8_fast (the
-// shifted value is an fp16 number like any other), the rounding the +1536 trick.
-// CLAMP = false leaves the clamp out: the shifted values lie in [0, range] by construction, so with a
-// scale that is a NORMAL fp16 number (relative rounding error <= 2^-11: range >= 2^-10 is enough) the
-// quotient is at most 15 (1 + 2^-11) and rounds to 15 at most.  A subnormal scale can be off by several
-// per cent and needs the clamp (range / 15 = 10.5 units of 2^-24 -> scale 10 units -> quotient 15.75).
-template <bool CLAMP = true>
-__device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) {
-    const f16x2 z2 = {zero, zero};
-    u32 b[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const f16x2 sh = as_f16x2(v[i]) + z2;
-        // the quotient straight from the packed pair to the packed fp16 quotient (one mixed-precision instruction per
-        // value; see sym_pair_fast for why its single rounding is still the correctly rounded division), then + 1536
-        f16x2 h = {(f16)__builtin_fmaf((float)sh[0], f.r, 0.0f), (f16)__builtin_fmaf((float)sh[1], f.r, 0.0f)};
-        h = h + f16x2{(f16)1536.0f, (f16)1536.0f};
-        if (CLAMP) {
-            // on the bit patterns: 1536 + code in [1536, 1551] is 0x6600 .. 0x660f; patterns of positive halves order
-            // like signed 16-bit integers, negative sums are negative integers, +inf (0x7c00) lies above
-            typedef short i16x2 __attribute__((ext_vector_type(2)));
-            i16x2 c = __builtin_bit_cast(i16x2, h);
-            c = __builtin_elementwise_max(c, i16x2{0x6600, 0x6600});
-            c = __builtin_elementwise_min(c, i16x2{0x660f, 0x660f});
-            b[i] = __builtin_bit_cast(u32, c);
-        } else {
-            b[i] = __builtin_bit_cast(u32, h);
-        }
-    }
-    return pack_nibbles8(b);
-}
-// ranges from which the clamp-free form is exact (see above)
-__device__ __forceinline__ bool asym_range_normal(f16 rng) { return rng >= (f16)0.0009765625f; }
 
 // LG = log2(lanes per vector) = log2(dim) - 3, 1..5
 // PAGED (head dimension 128 only): codes and {scale, zero} go straight to the vector's place in the paged

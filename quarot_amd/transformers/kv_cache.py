@@ -201,14 +201,17 @@ def _decode_workspace_bytes(batch, heads, max_seq_len, device_index=None):
 
 
 def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, max_seq_len=0,
-                    q_hadamard=False, workspace=None):
+                    q_hadamard=False, workspace=None, append=None):
     """o[b, h] = softmax(q[b, h] . K^T / sqrt(128)) . V over the int4 cache of sequence b, dequantised in
     registers as float(code) * scale - zero (kv_cache.py:60-67 -> bindings.cpp:118-153).  Writes into `o`
     and returns None, like the reference's binding.  max_seq_len (optional, an upper bound of the
     sequence lengths) lets a small batch be split along the sequence.  q_hadamard: `q` is the
     untransformed query and the kernel applies matmul_had_cuda(q, torch.float16) itself (one launch
     instead of two).  workspace: a uint8 tensor on the cache's device to hold the partial states of a split along
-    the sequence; one is allocated per call when it is missing or too small."""
+    the sequence; one is allocated per call when it is missing or too small.  append = (k, v, hadamard): the fp16
+    key and value [batch_size, heads, 128] of the step's new token, which the page tables already count as every
+    sequence's last position: the kernel quantises them as quantize_append_kv_i4 would (same codes, scales and zeros,
+    written to the same page slots) and attends to them along with the cache -- append and attention in one launch."""
     fn = "batch_decode_i4"
     pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
     for name, t in (("o", o), ("q", q)):
@@ -227,6 +230,10 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
         raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
     if not (last_page_offset.shape[0] == batch):
         raise RuntimeError(f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
+    if append is not None:
+        for name, t in (("k", append[0]), ("v", append[1])):
+            if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float16 and tuple(t.shape) == (batch, heads, head_dim)):
+                raise RuntimeError(f"{fn}: append {name} must be a contiguous fp16 [batch_size, {heads}, {head_dim}] CUDA tensor")
     dev = kv_data.device
     with _lib.on_device(dev):
         ws_bytes = _decode_workspace_bytes(batch, heads, int(max_seq_len), dev.index) if max_seq_len else 0
@@ -235,6 +242,13 @@ def batch_decode_i4(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
             fits = (workspace is not None and workspace.device == dev and workspace.dtype == torch.uint8
                     and workspace.is_contiguous() and workspace.numel() >= ws_bytes)
             ws = workspace if fits else torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+        if append is not None:
+            _lib.check(_lib.lib().qr_kv_quant_append_batch_decode_f16_i4(
+                o.data_ptr(), q.data_ptr(), 1 if q_hadamard else 0, append[0].data_ptr(), append[1].data_ptr(),
+                1 if append[2] else 0, kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
+                last_page_offset.data_ptr(), pages, layers, int(layer_idx), heads, page_size, head_dim, batch, int(max_seq_len),
+                None if ws is None else ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev)))
+            return
         entry = _lib.lib().qr_batch_decode_qhad_i4 if q_hadamard else _lib.lib().qr_batch_decode_i4
         _lib.check(entry(
             o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
@@ -252,7 +266,7 @@ class _AttentionStub(object):
         self.disable_quant = disable_quant
         self.hadamard_dtype = hadamard_dtype
 
-    def forward(self, q, num_kv_heads, attention_kwargs, layer_idx, max_seq_len=0, workspace=None):
+    def forward(self, q, num_kv_heads, attention_kwargs, layer_idx, max_seq_len=0, workspace=None, take_pending=None):
         batch_size, q_len, num_qo_heads, head_dim = q.shape
         assert q_len == 1
         q = q.view(batch_size, num_qo_heads, head_dim)
@@ -260,8 +274,10 @@ class _AttentionStub(object):
         if self.hadamard_dtype is not None and not fused:
             q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
         attn_output = torch.empty_like(q)
+        # the step's new token, if the cache still holds it back for this call (see MultiLayerPagedKVCache4Bit.update)
+        append = take_pending() if take_pending is not None else None
         batch_decode_i4(attn_output, q, **attention_kwargs, layer_idx=layer_idx, max_seq_len=max_seq_len, q_hadamard=fused,
-                        workspace=workspace)
+                        workspace=workspace, append=append)
         return attn_output.unsqueeze(1)
 
 
@@ -283,10 +299,11 @@ class MultiLayerPagedKVCache4Bit:
         self.batch_size = batch_size
         max_page_cnt = self.page_cnt_from_length(max_seq_len)
         self.disable_quant = disable_quant
-        self.pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
-                                 dtype=torch.uint8, device=device)
-        self.scales = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=torch.float16,
-                                  device=device)
+        self._pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
+                                  dtype=torch.uint8, device=device)
+        self._scales = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=torch.float16,
+                                   device=device)
+        self._pending = {}      # layer -> (token, k, v, specs, hadamard): a decode step's new token, held for the attention call
         self.max_seq_len = max_seq_len
         self._needs_init = [True] * n_layers
         self.length = 0
@@ -298,13 +315,41 @@ class MultiLayerPagedKVCache4Bit:
     def page_cnt_from_length(self, length):
         return (length + self.page_size - 1) // self.page_size
 
+    # A decode step's new token is quantised and stored by the attention launch that follows update() (one launch per
+    # step instead of two).  Whoever looks at the cache before that call -- the page tensors, the tables, the next
+    # update -- first gets the token stored by the quantise-and-append kernel, so the cache never shows a state the
+    # reference's would not.
+    @property
+    def pages(self):
+        self._flush()
+        return self._pages
+
+    @property
+    def scales(self):
+        self._flush()
+        return self._scales
+
+    def _flush(self, layer_idx=None):
+        for layer in ([layer_idx] if layer_idx is not None else list(self._pending)):
+            held = self._pending.pop(layer, None)
+            if held is not None:
+                _, k, v, specs, hadamard = held
+                quantize_append_kv_i4(**specs, k=k, v=v, seqlen_indptr=None, layer_idx=layer, hadamard=hadamard)
+
+    def _take_pending(self, layer_idx, token):
+        held = self._pending.get(layer_idx)
+        if held is None or held[0] is not token:
+            return None                          # stored meanwhile (or this callable was used before): plain attention
+        del self._pending[layer_idx]
+        return held[1], held[2], held[4]
+
     def _decode_workspace(self, num_heads):
         """Scratch for decode attention split along the sequence, kept with the cache (every layer of every decode
         step would otherwise allocate its own): sized for the longer of the current and the maximum length."""
         key = (self.length, num_heads)
         if getattr(self, "_decode_ws_key", None) == key:
             return self._decode_ws
-        dev = self.pages.device
+        dev = self._pages.device
         with _lib.on_device(dev):
             need = max((_decode_workspace_bytes(self.batch_size, num_heads, int(n), dev.index)
                         for n in (self.length, self.max_seq_len) if n), default=0)
@@ -315,7 +360,7 @@ class MultiLayerPagedKVCache4Bit:
         return ws
 
     def _ensure_page_cnt_per_batch(self, expected_page_cnt_per_batch):
-        if expected_page_cnt_per_batch * self.batch_size <= self.pages.shape[0]:
+        if expected_page_cnt_per_batch * self.batch_size <= self._pages.shape[0]:
             return
         raise NotImplementedError
 
@@ -327,6 +372,8 @@ class MultiLayerPagedKVCache4Bit:
         b_sz, added_length, num_heads, head_dim = key_states.shape
         assert b_sz == self.batch_size
         cache_kwargs = cache_kwargs or {}
+        if self._pending:
+            self._flush()
         if layer_idx == 0:
             new_length = self.length + added_length
             self._ensure_page_cnt_per_batch(self.page_cnt_from_length(new_length))
@@ -358,15 +405,24 @@ class MultiLayerPagedKVCache4Bit:
                                       layer_idx=layer_idx, hadamard=fused_had)
             return key_states, value_states
         assert added_length == 1
-        quantize_append_kv_i4(**specs, k=k_in.reshape(self.batch_size, num_heads, head_dim).contiguous(),
-                              v=value_states.reshape(self.batch_size, num_heads, head_dim).contiguous(), seqlen_indptr=None,
-                              layer_idx=layer_idx, hadamard=fused_had)
+        k3 = k_in.reshape(self.batch_size, num_heads, head_dim).contiguous()
+        v3 = value_states.reshape(self.batch_size, num_heads, head_dim).contiguous()
+        if k3.dtype == torch.float16 and v3.dtype == torch.float16 and head_dim == 128:
+            # held for the attention call, which quantises and stores the token itself
+            token = object()
+            self._pending[layer_idx] = (token, k3, v3, specs, fused_had)
+            take = functools.partial(self._take_pending, layer_idx, token)
+        else:
+            quantize_append_kv_i4(**specs, k=k3, v=v3, seqlen_indptr=None, layer_idx=layer_idx, hadamard=fused_had)
+            take = None
         return functools.partial(self._stub.forward, num_kv_heads=num_heads, attention_kwargs=specs, layer_idx=layer_idx,
-                                 max_seq_len=self.length, workspace=self._decode_workspace(num_heads))
+                                 max_seq_len=self.length, workspace=self._decode_workspace(num_heads), take_pending=take)
 
     def get_cache_specs_for_flash_infer(self, attention_mask):
         """Page tables of the current state (kv_cache.py:253-275): page i of sequence b is page number
         i * batch_size + b; every sequence must span the same number of pages."""
+        if self._pending:
+            self._flush()
         if attention_mask is None:
             # every sequence holds self.length tokens: the tables depend on that number alone and are built
             # once per length (every layer of a decode step asks for them), with host arithmetic
@@ -378,11 +434,11 @@ class MultiLayerPagedKVCache4Bit:
             ptr = self.page_size if (self.length != 0 and ptr == 0) else ptr
             arange = functools.partial(torch.arange, device=self.device, dtype=torch.int32)
             specs = {
-                "kv_data": self.pages,
+                "kv_data": self._pages,
                 "kv_indptr": arange(0, self.batch_size + 1) * page_cnt,
                 "kv_indices": (arange(page_cnt).unsqueeze(0) * self.batch_size + arange(self.batch_size).unsqueeze(1)).reshape(-1),
                 "last_page_offset": torch.full((self.batch_size,), ptr, dtype=torch.int32, device=self.device),
-                "kv_param": self.scales,
+                "kv_param": self._scales,
             }
             self._specs = (self.length, specs)
             return specs
@@ -395,11 +451,11 @@ class MultiLayerPagedKVCache4Bit:
         page_ptr = torch.where((seqlens_in_batch != 0) & (page_ptr == 0), self.page_size, page_ptr).to(torch.int32).contiguous()
         arange = functools.partial(torch.arange, device=self.device, dtype=torch.int32)
         return {
-            "kv_data": self.pages,
+            "kv_data": self._pages,
             "kv_indptr": (arange(0, self.batch_size + 1) * page_cnt).to(torch.int32),
             "kv_indices": ((arange(int(page_cnt)) * self.batch_size).unsqueeze(0) + arange(self.batch_size).unsqueeze(1)).reshape(-1).contiguous(),
             "last_page_offset": page_ptr,
-            "kv_param": self.scales,
+            "kv_param": self._scales,
         }
 
     def get_seq_length(self, layer_idx=0):
