@@ -246,7 +246,10 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
     // ALIGNED: chunk g lies in page g / cpp at entry 16 (g % cpp); both advance without divisions
     const int cpp = ALIGNED ? c.page_size >> 4 : 1;
     const int it_step = stride / cpp, r_step = stride - it_step * cpp;
-    int g = sp * NW + wave;
+    // APPEND: the wave that quantises the new token leaves its first two chunks (one step's worth) to its two
+    // neighbours, which take one each after their own walk: its extra work would otherwise stand at the launch's end
+    const int g_first = sp * NW + wave;
+    int g = g_first + ((APPEND && appends) ? stride * AU : 0);
     int it_u = g / cpp, r_u = g - it_u * cpp;
     // Two sets of AU positions per lane group: the loads of the next set are issued before the current
     // one is consumed, so their latency hides under the arithmetic.  Loads are unconditional (a position
@@ -364,6 +367,16 @@ __global__ __launch_bounds__(64 * NW, (NW == 16 ? 1 : NW == 8 ? 2 : 4)) void pag
         __builtin_amdgcn_sched_barrier(0);
         if (g + gs < chunks) consume(sb);                  // (no loads inside: the branch does not disturb the wait counts)
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if (APPEND && sp == 0 && (wave == 1 || wave == 2)) {
+        const int extra = sp * NW + (wave == 2 ? stride : 0);           // the quantising wave's first or second chunk
+        if (extra < chunks) {
+            it_u = extra / cpp;
+            r_u = extra - it_u * cpp;
+            issue(sb, extra);
+            sb.ok[1] = false;                                           // (the step's second chunk is not this wave's)
+            consume(sb);
+        }
     }
     if (APPEND && appends) {
         // the new position, from the codes this wave made: lane group 0 takes it, the others sit the turn out
