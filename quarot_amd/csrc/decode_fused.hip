@@ -1,5 +1,6 @@
-// One token through OnlineHadamard -> Quantizer -> Linear4bit in ONE launch (quarot/nn/hadamard.py:17-23,
-// quarot/nn/quantization.py:10, quarot/nn/linear.py:42-56 on a single row).
+// A decode step's whole linear layer in ONE launch: one token through OnlineHadamard -> Quantizer -> Linear4bit
+// (bm_gemv_kernel), one or two tokens through Quantizer -> Linear4bit (quant_gemv_kernel, quant_gemv_mt_kernel)
+// (quarot/nn/hadamard.py:17-23, quarot/nn/quantization.py:10, quarot/nn/linear.py:42-56 on one or two rows).
 // A decode step at one token is latency: the transform of a 57 KB row keeps one CU busy for a few microseconds
 // while the others wait, and only then does the weight stream start.  Here EVERY workgroup transforms and
 // quantises the row itself (the row comes out of L2; the arithmetic is that of hadamard_bm_kernel's register
@@ -7,6 +8,7 @@
 // requested, keeps the codes in LDS and goes on as the dot-product kernel does (v_dot8_i32_i4 over 1 KB segments of
 // the weight rows, gemv_i4_kernel's arithmetic and epilogue).  Nothing is exchanged between workgroups.
 #include "qr_common.h"
+
 namespace {
 
 // Weight segments a wave requests at each point of the front (after the first barrier, after its part of the power-of-two
