@@ -1122,6 +1122,43 @@ def test_decode_step_replays_from_a_hip_graph():
         assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
 
 
+@pytest.mark.parametrize("k,m,had", [(12288, 1, True), (28672, 1, True), (4096, 1, False), (8192, 2, False)])
+def test_one_launch_decode_steps_replay_from_a_hip_graph(k, m, had):
+    """The decode steps that are ONE kernel (one token behind a 1024-point Hadamard factor; one or two tokens behind the
+    plain quantiser) captured into a HIP graph: every replay, with fresh inputs copied into the static buffer and eager
+    work plus synchronisation in between, equals the eager two-launch chain bit for bit."""
+    n = 2048
+    w, sw = synth_w(n, k, seed=12)
+    gw, gsw = gpu(w), gpu(sw)
+    hadK, K = (quarot_amd.functional.hadamard.get_hadK(k) if had else (None, 0))
+    if hadK is not None:
+        hadK = hadK.to(dev()).half()
+    xs = [gpu(synth_x(m, k, seed=30 + i, outliers=i % 2 == 0)) for i in range(4)]
+    static_x = xs[0].clone()
+    step = lambda x: quarot_amd.quantized_linear(x, gw, gsw, None, hadK, K)
+
+    def chain(x):
+        if had:
+            p = quarot_amd.hadamard_quantize(x, hadK, K)
+            return quarot_amd.linear_i4(p.quantized_x, p.scales_x, gw, gsw, None)
+        q, s = quarot_amd.quantize_rows(x, 1.0)
+        return quarot_amd.linear_i4(q, s, gw, gsw, None)
+
+    for _ in range(2):
+        step(static_x)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = step(static_x)
+    for i, x in enumerate(xs):
+        eager = chain(x)
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(static_y, eager), f"replay {i}"
+
+
 def test_kv_hadamard_128_blocks_tails_and_infinities():
     """Head dimension 128 with the Hadamard runs on the matrix cores, 32 vectors per wave step: vector
     counts around the block size, equality of the fused codes with the quantiser applied to the plain
