@@ -20,6 +20,120 @@ namespace {
 // rings are slower ({1,2,2,1} 21.0, {1,2,2,2} 22.2: more requests queue ahead of what the front waits for).
 constexpr int F0 = 1, F1 = 2, F2 = 2, F3 = 0, RING = F0 + F1 + F2 + F3;
 
+// The dot products that all kernels of this file end in: a wave takes `ng` consecutive pairs of weight rows as one
+// flattened sequence of 1 KB segments (lane l: bytes [16 l, 16 l + 16) of each row's segment), a ring of segments in
+// flight, against the MB tokens' codes in LDS (v_dot8_i32_i4: eight signed 4-bit products per lane and instruction).
+// The kernels place the first requests between the phases of their fronts (fetch) and consume the ring once the codes
+// are in LDS (run).  A row's last segment may be short: the lanes past its end re-read the row's start against zero
+// codes.  The 64 partial sums of each (row, token) pair are added across the wave by a halving exchange, and the lane
+// that ends up with a pair's sum applies Linear4bit's epilogue: y = fp16(fp16(sA sW) fp16(sum)) (+ bias).
+template <int MB>
+struct RowPairStream {
+    static constexpr int R = 2, NS = R * MB, LV = NS == 2 ? 1 : NS == 4 ? 2 : NS == 8 ? 3 : 4;
+    struct Seg {
+        u32x4 w[R];
+        f16 sb, bi;                              // scale and bias of the output this lane will store
+    };
+    const uint8_t* B;
+    const f16* sB;
+    const f16* bias;
+    int N, Kb, nseg, g0, gcount, lane, my_m, my_r, fg, fs;
+
+    __device__ __forceinline__ void init(const uint8_t* B_, const f16* sB_, const f16* bias_, int N_, int Kb_, int ng, int wave,
+                                         int lane_) {
+        B = B_, sB = sB_, bias = bias_, N = N_, Kb = Kb_, lane = lane_;
+        nseg = (Kb + 1023) >> 10;
+        const int groups = (N + R - 1) / R;
+        g0 = ((int)blockIdx.x * 16 + wave) * ng;
+        gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
+        const int vidx = lane >> (6 - LV);       // which of a pair's NS sums this lane stores at the end of the exchange
+        my_m = vidx / R, my_r = vidx % R;
+        fg = fs = 0;
+    }
+    __device__ __forceinline__ void fetch(Seg& s) {
+        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int nr = (g0 + fg) * R + r;
+            nr = nr < N ? nr : N - 1;
+            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
+        }
+        // every segment carries its pair's scale along: loading it at the pair's end would make the wave wait for
+        // everything it has in flight
+        int col = (g0 + fg) * R + my_r;
+        col = col < N ? col : N - 1;
+        s.sb = sB[col];
+        s.bi = (bias ? bias : sB)[col];          // (no bias: a harmless second read of the scale)
+        if (fs + 1 < nseg) ++fs;
+        else if (fg + 1 < gcount) { ++fg; fs = 0; }
+    }
+    // xq: the tokens' codes in LDS, nseg * 1024 bytes per token (zero-filled past the row's end); my_sa: the scale of
+    // the token whose sums this lane stores; M: tokens that exist
+    template <int RD>
+    __device__ __forceinline__ void run(Seg (&ring)[RD], const void* xq, f16 my_sa, int M, f16* __restrict__ Y) {
+        if (gcount == 0) return;
+        const u32x4* xs = (const u32x4*)xq + lane;
+        const int total = gcount * nseg;
+        int acc[NS];
+#pragma unroll
+        for (int i = 0; i < NS; ++i) acc[i] = 0;
+        int cg = 0, cs = 0;
+        auto consume = [&](const Seg& sg) {
+#pragma unroll
+            for (int mt = 0; mt < MB; ++mt) {
+                const u32x4 xv = xs[(mt * nseg + cs) * 64];
+#pragma unroll
+                for (int d = 0; d < 4; ++d)
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        acc[mt * R + r] = __builtin_amdgcn_sdot8((int)sg.w[r][d], (int)xv[d], acc[mt * R + r], false);
+            }
+            if (++cs < nseg) return;
+            // end of a pair of rows: each step of the exchange gives away half of the values a lane still holds
+            int vals[NS];
+#pragma unroll
+            for (int i = 0; i < NS; ++i) vals[i] = acc[i];
+            int off = 32;
+#pragma unroll
+            for (int cur = NS; cur > 1; cur >>= 1) {
+                const bool upper = (lane & off) != 0;
+#pragma unroll
+                for (int i = 0; i < cur / 2; ++i) {
+                    const int give = upper ? vals[i] : vals[i + cur / 2];
+                    const int keep = upper ? vals[i + cur / 2] : vals[i];
+                    vals[i] = keep + __shfl_xor(give, off, QR_WAVE);
+                }
+                off >>= 1;
+            }
+            int sum = vals[0];
+            for (; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
+            if ((lane & ((1 << (6 - LV)) - 1)) == 0) {
+                const int col = (g0 + cg) * R + my_r;
+                if (my_m < M && col < N) {
+                    f16 yo = (f16)(my_sa * sg.sb) * (f16)(float)sum;
+                    if (bias) yo = yo + sg.bi;
+                    Y[(int64_t)my_m * N + col] = yo;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NS; ++i) acc[i] = 0;
+            cs = 0;
+            ++cg;
+        };
+        int it = 0;
+        for (; it + RD <= total; it += RD) {                    // whole turns of the ring: no branch around the loads
+#pragma unroll
+            for (int r = 0; r < RD; ++r) {
+                consume(ring[r]);
+                fetch(ring[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RD - 1; ++r)
+            if (it + r < total) consume(ring[r]);
+    }
+};
+
 // n = 1024 K (K = order of the table, a multiple of 4, at most 32).  A wave takes `ng` consecutive pairs of weight
 // rows as one flattened sequence of 1 KB segments, RD segments in flight (first requested while the row is transformed).
 template <int RD>
@@ -27,7 +141,7 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
                                                        float scale, float clip, const uint8_t* __restrict__ B,
                                                        const f16* __restrict__ sB, const f16* __restrict__ bias, int N,
                                                        int ng, f16* __restrict__ Y) {
-    constexpr int NW = 16, M_ = 1024, CT = M_ / 16, RT = 2, TS = 17, R = 2;
+    constexpr int NW = 16, M_ = 1024, CT = M_ / 16, RT = 2, TS = 17;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[NW];
     u32x4* Tl = (u32x4*)smem_raw;                // [4][CT][TS]
@@ -54,31 +168,10 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
     // them as they lie and swapping lanes through LDS was measured 0.1 us slower.)
 
     // ---- the weight stream of this wave ----------------------------------------------------------------------
-    const int groups = (N + R - 1) / R;
-    const int g0 = (blockIdx.x * NW + wave) * ng;
-    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
-    const int nseg = Kb / 1024;
-    const int total = gcount * nseg;
-    const int my_r = lane >> 5;                  // which of a pair's two sums this lane ends up with
-    struct Seg {
-        u32x4 w[R];
-        f16 sb, bi;
-    };
-    int fg = 0, fs = 0;
-    auto fetch = [&](Seg& s) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int nr = (g0 + fg) * R + r;
-            nr = nr < N ? nr : N - 1;
-            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + fs * 1024 + lane * 16));
-        }
-        int col = (g0 + fg) * R + my_r;
-        col = col < N ? col : N - 1;
-        s.sb = sB[col];
-        s.bi = (bias ? bias : sB)[col];
-        if (fs + 1 < nseg) ++fs;
-        else if (fg + 1 < gcount) { ++fg; fs = 0; }
-    };
+    RowPairStream<1> ws;
+    ws.init(B, sB, bias, N, Kb, ng, wave, lane);
+    auto fetch = [&](RowPairStream<1>::Seg& sg) { ws.fetch(sg); };
+    using Seg = RowPairStream<1>::Seg;
 
     // ---- fragments: Sylvester factors of both stages -----------------------------------------------------------
     f16x8 ha[2], hb[2];
@@ -239,47 +332,7 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
     __syncthreads();
 
     // ---- the dot products -----------------------------------------------------------------------------------
-    if (gcount == 0) return;
-    const u32x4* xs = (const u32x4*)xq + lane;
-    int acc[R] = {0, 0};
-    int cg = 0, cs = 0;
-    auto consume = [&](const Seg& s) {
-        const u32x4 xv = xs[cs * 64];
-#pragma unroll
-        for (int d = 0; d < 4; ++d)
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_sdot8((int)s.w[r][d], (int)xv[d], acc[r], false);
-        if (++cs < nseg) return;
-        // end of a pair of rows: lanes 0..31 end with the first row's sum, lanes 32..63 with the second's
-        const bool upper = (lane & 32) != 0;
-        const int give = upper ? acc[0] : acc[1];
-        const int keep = upper ? acc[1] : acc[0];
-        int sum = keep + __shfl_xor(give, 32, QR_WAVE);
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
-        if ((lane & 31) == 0) {
-            const int col = (g0 + cg) * R + my_r;
-            if (col < N) {
-                f16 yo = (f16)(sh * s.sb) * (f16)(float)sum;
-                if (bias) yo = yo + s.bi;
-                Y[col] = yo;
-            }
-        }
-        acc[0] = acc[1] = 0;
-        cs = 0;
-        ++cg;
-    };
-    int it = 0;
-    for (; it + RD <= total; it += RD) {                    // whole turns of the ring: no branch around the loads
-#pragma unroll
-        for (int r = 0; r < RD; ++r) {
-            consume(ring[r]);
-            fetch(ring[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RD - 1; ++r)
-        if (it + r < total) consume(ring[r]);
+    ws.run(ring, xq, sh, 1, Y);
 }
 
 // ---- Quantizer -> Linear4bit for one token (no Hadamard in front) ---------------------------------------------
@@ -292,7 +345,7 @@ template <int NV>
 __global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restrict__ x, int cols8, float clip,
                                                           const uint8_t* __restrict__ B, const f16* __restrict__ sB,
                                                           const f16* __restrict__ bias, int N, int ng, f16* __restrict__ Y) {
-    constexpr int NW = 16, R = 2, RD = 5;
+    constexpr int NW = 16, RD = 5;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[NW];
     u32* xq = (u32*)smem_raw;                    // codes of the row, a word per piece, zero-filled to whole segments
@@ -304,31 +357,10 @@ __global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restric
         const int c = tid + i * 1024;
         v[i] = x[c < cols8 ? c : 0];
     }
-    const int groups = (N + R - 1) / R;
-    const int g0 = (blockIdx.x * NW + wave) * ng;
-    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
-    const int total = gcount * nseg;
-    const int my_r = lane >> 5;
-    struct Seg {
-        u32x4 w[R];
-        f16 sb, bi;
-    };
-    int fg = 0, fs = 0;
-    auto fetch = [&](Seg& s) {
-        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int nr = (g0 + fg) * R + r;
-            nr = nr < N ? nr : N - 1;
-            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
-        }
-        int col = (g0 + fg) * R + my_r;
-        col = col < N ? col : N - 1;
-        s.sb = sB[col];
-        s.bi = (bias ? bias : sB)[col];
-        if (fs + 1 < nseg) ++fs;
-        else if (fg + 1 < gcount) { ++fg; fs = 0; }
-    };
+    RowPairStream<1> ws;
+    ws.init(B, sB, bias, N, Kb, ng, wave, lane);
+    auto fetch = [&](RowPairStream<1>::Seg& sg) { ws.fetch(sg); };
+    using Seg = RowPairStream<1>::Seg;
     Seg ring[RD];
     fetch(ring[0]);
     fetch(ring[1]);
@@ -365,46 +397,7 @@ __global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restric
     }
     fetch(ring[4]);
     __syncthreads();
-    if (gcount == 0) return;
-    const u32x4* xs = (const u32x4*)xq + lane;
-    int acc[R] = {0, 0};
-    int cg = 0, cs = 0;
-    auto consume = [&](const Seg& sg) {
-        const u32x4 xv = xs[cs * 64];
-#pragma unroll
-        for (int d = 0; d < 4; ++d)
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r] = __builtin_amdgcn_sdot8((int)sg.w[r][d], (int)xv[d], acc[r], false);
-        if (++cs < nseg) return;
-        const bool upper = (lane & 32) != 0;
-        const int give = upper ? acc[0] : acc[1];
-        const int keep = upper ? acc[1] : acc[0];
-        int sum = keep + __shfl_xor(give, 32, QR_WAVE);
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
-        if ((lane & 31) == 0) {
-            const int col = (g0 + cg) * R + my_r;
-            if (col < N) {
-                f16 yo = (f16)(sh * sg.sb) * (f16)(float)sum;
-                if (bias) yo = yo + sg.bi;
-                Y[col] = yo;
-            }
-        }
-        acc[0] = acc[1] = 0;
-        cs = 0;
-        ++cg;
-    };
-    int it = 0;
-    for (; it + RD <= total; it += RD) {
-#pragma unroll
-        for (int r = 0; r < RD; ++r) {
-            consume(ring[r]);
-            fetch(ring[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RD - 1; ++r)
-        if (it + r < total) consume(ring[r]);
+    ws.run(ring, xq, sh, 1, Y);
 }
 
 // ---- Quantizer -> Linear4bit for two tokens -------------------------------------------------------------------------
@@ -417,7 +410,7 @@ template <int MB>
 __global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __restrict__ x, int M, int cols8, float clip,
                                                              const uint8_t* __restrict__ B, const f16* __restrict__ sB,
                                                              const f16* __restrict__ bias, int N, int ng, f16* __restrict__ Y) {
-    constexpr int NW = 16, R = 2, RD = 5, WPR = NW / MB, NV = 8, NS = R * MB;
+    constexpr int NW = 16, RD = 5, WPR = NW / MB, NV = 8;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[NW];
     __shared__ f16 sc[MB];
@@ -432,34 +425,10 @@ __global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __rest
         const int c = (i * WPR + part) * 64 + lane;
         v[i] = xr[c < cols8 ? c : 0];
     }
-    const int groups = (N + R - 1) / R;
-    const int g0 = (blockIdx.x * NW + wave) * ng;
-    const int gcount = g0 >= groups ? 0 : (groups - g0 < ng ? groups - g0 : ng);
-    const int total = gcount * nseg;
-    // which of a pair's NS sums this lane stores at the end of the exchange (log2(NS) lane bits from bit 5 downwards)
-    constexpr int LV = NS == 2 ? 1 : NS == 4 ? 2 : NS == 8 ? 3 : 4;
-    const int vidx = lane >> (6 - LV);
-    const int my_m = vidx / R, my_r = vidx % R;
-    struct Seg {
-        u32x4 w[R];
-        f16 sb, bi;
-    };
-    int fg = 0, fs = 0;
-    auto fetch = [&](Seg& s) {
-        const int off = (fs * 1024 + lane * 16 < Kb) ? fs * 1024 + lane * 16 : 0;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            int nr = (g0 + fg) * R + r;
-            nr = nr < N ? nr : N - 1;
-            s.w[r] = __builtin_nontemporal_load((const u32x4*)(B + (int64_t)nr * Kb + off));
-        }
-        int col = (g0 + fg) * R + my_r;
-        col = col < N ? col : N - 1;
-        s.sb = sB[col];
-        s.bi = (bias ? bias : sB)[col];
-        if (fs + 1 < nseg) ++fs;
-        else if (fg + 1 < gcount) { ++fg; fs = 0; }
-    };
+    RowPairStream<MB> ws;
+    ws.init(B, sB, bias, N, Kb, ng, wave, lane);
+    auto fetch = [&](typename RowPairStream<MB>::Seg& sg) { ws.fetch(sg); };
+    using Seg = typename RowPairStream<MB>::Seg;
     Seg ring[RD];
     fetch(ring[0]);
     fetch(ring[1]);
@@ -498,66 +467,7 @@ __global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __rest
     }
     fetch(ring[4]);
     __syncthreads();
-    if (gcount == 0) return;
-    const f16 my_sa = sc[my_m < M ? my_m : M - 1];
-    const u32x4* xs = (const u32x4*)xq + lane;
-    int acc[NS];
-#pragma unroll
-    for (int i = 0; i < NS; ++i) acc[i] = 0;
-    int cg = 0, cs = 0;
-    auto consume = [&](const Seg& sg) {
-#pragma unroll
-        for (int mt = 0; mt < MB; ++mt) {
-            const u32x4 xv = xs[(mt * nseg + cs) * 64];
-#pragma unroll
-            for (int d = 0; d < 4; ++d)
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-                    acc[mt * R + r] = __builtin_amdgcn_sdot8((int)sg.w[r][d], (int)xv[d], acc[mt * R + r], false);
-        }
-        if (++cs < nseg) return;
-        // end of a pair of rows: halving exchange (each step gives away half of the values a lane still holds)
-        int vals[NS];
-#pragma unroll
-        for (int i = 0; i < NS; ++i) vals[i] = acc[i];
-        int off = 32;
-#pragma unroll
-        for (int cur = NS; cur > 1; cur >>= 1) {
-            const bool upper = (lane & off) != 0;
-#pragma unroll
-            for (int i = 0; i < cur / 2; ++i) {
-                const int give = upper ? vals[i] : vals[i + cur / 2];
-                const int keep = upper ? vals[i + cur / 2] : vals[i];
-                vals[i] = keep + __shfl_xor(give, off, QR_WAVE);
-            }
-            off >>= 1;
-        }
-        int sum = vals[0];
-        for (; off > 0; off >>= 1) sum += __shfl_xor(sum, off, QR_WAVE);
-        if ((lane & ((1 << (6 - LV)) - 1)) == 0) {
-            const int col = (g0 + cg) * R + my_r;
-            if (my_m < M && col < N) {
-                f16 yo = (f16)(my_sa * sg.sb) * (f16)(float)sum;
-                if (bias) yo = yo + sg.bi;
-                Y[(int64_t)my_m * N + col] = yo;
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < NS; ++i) acc[i] = 0;
-        cs = 0;
-        ++cg;
-    };
-    int it = 0;
-    for (; it + RD <= total; it += RD) {
-#pragma unroll
-        for (int r = 0; r < RD; ++r) {
-            consume(ring[r]);
-            fetch(ring[r]);
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RD - 1; ++r)
-        if (it + r < total) consume(ring[r]);
+    ws.run(ring, xq, sc[ws.my_m < M ? ws.my_m : M - 1], M, Y);
 }
 
 }  // namespace
