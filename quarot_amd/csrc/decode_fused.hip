@@ -478,7 +478,7 @@ __attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(cons
                                                                             float scale, float clip, const void* W,
                                                                             const void* sW, const void* bias, int64_t N,
                                                                             void* y, hipStream_t st) {
-    if (K < 4 || K > 32 || (K & 3) != 0 || n != 1024 * K || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
+    if (K < 4 || K > 32 || (K & 3) != 0 || n != 1024 * K || N <= 0 || N > (1 << 30)) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)W & 15) || ((uintptr_t)hadK & 15)) return QR_E_UNSUPPORTED;
     const int cus = qr_device().cus;
     const int64_t groups = (N + 1) / 2;
@@ -497,7 +497,7 @@ __attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(cons
 __attribute__((visibility("hidden"))) int qr_internal_token_quant_linear(const void* x, int64_t M, int64_t K, float clip,
                                                                          const void* W, const void* sW, const void* bias,
                                                                          int64_t N, void* y, hipStream_t st) {
-    if (M < 1 || M > 2 || K <= 0 || K % 64 != 0 || K > 32768 || N <= 0 || N > 0x7fffffff) return QR_E_UNSUPPORTED;
+    if (M < 1 || M > 2 || K <= 0 || K % 64 != 0 || K > 32768 || N <= 0 || N > (1 << 30)) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)W & 15)) return QR_E_UNSUPPORTED;
     const int cols8 = (int)(K / 8), nseg = (cols8 * 4 + 1023) / 1024;
     const int cus = qr_device().cus;
