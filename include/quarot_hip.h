@@ -231,10 +231,10 @@ int qr_linear_f6_f16(const void* A6, const void* sA, const void* W6, const void*
  * qr_hadamard_quantize_f16_i4 (or qr_quantize_rows_f16_i4) and qr_linear_i4_f16_ws on `stream`, with
  * the codes and scales between them in `workspace`: same results bit for bit, one call instead of
  * two for hosts whose per-call cost matters (a decode step launched from Python).
- * ONE token (M == 1) behind a 1024-point factor (K == 1024 * had_K, had_K a multiple of 4 up to 32: the
- * 70B down_proj, 28672 = 1024 x 28), mode QR_DTYPE_F16: a single kernel in which every workgroup
- * transforms and quantises the row itself and goes straight on to its dot products -- the same codes,
- * scale, sums and epilogue, so y carries the same bits, and the weight stream starts while the row is
+ * ONE or TWO tokens (M <= 2) behind a 1024-point factor (K == 1024 * had_K, had_K a multiple of 4 up to 32:
+ * the 70B down_proj, 28672 = 1024 x 28), mode QR_DTYPE_F16: a single kernel in which every workgroup
+ * transforms and quantises the rows itself and goes straight on to its dot products -- the same codes,
+ * scales, sums and epilogue, so y carries the same bits, and the weight stream starts while the rows are
  * still being transformed.  ONE or TWO tokens with had_K == 0 (K up to 32768): likewise one kernel, every
  * workgroup quantising the rows itself.  The workspace is checked as always; what it holds afterwards
  * is unspecified.

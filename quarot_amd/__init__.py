@@ -338,7 +338,7 @@ def _quantized_linear_workspace_bytes(M, N, K, device_index=None):
 def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_ratio=1.0, force_fp32=False):
     """Sequential(OnlineHadamard, Quantizer, Linear4bit) -- or, with K == 0, Sequential(Quantizer,
     Linear4bit) -- in ONE call into the library (e2e/quantized_llama/modeling_llama.py:99-102,111-115):
-    the same two launches as hadamard_quantize / quantize_rows followed by linear_i4 (one token, plain or behind a
+    the same two launches as hadamard_quantize / quantize_rows followed by linear_i4 (one or two tokens, plain or behind a
     1024-point Hadamard factor: one kernel that does both), same results bit for bit, half the host-side
     cost.  x fp16 [..., in_features] -> fp16 [..., out_features]."""
     assert x.dtype == torch.float16

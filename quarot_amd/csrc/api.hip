@@ -43,8 +43,8 @@ extern "C" int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int 
     uint8_t* rest = scales + scales_bytes;
     const size_t rest_bytes = workspace_bytes - codes_bytes - scales_bytes;
     // one token behind a long power-of-two factor: the front and the dot products in one launch (same codes, same sums)
-    if (M == 1 && had_K > 1 && mode == QR_DTYPE_F16 && hadK && ((uintptr_t)y & 1) == 0) {
-        const int rc1 = qr_internal_token_hadamard_linear(x, (int)K, had_K, hadK, scale, clip, W, sW, bias_or_null, N, y,
+    if (M <= 2 && had_K > 1 && mode == QR_DTYPE_F16 && hadK && ((uintptr_t)y & 1) == 0) {
+        const int rc1 = qr_internal_token_hadamard_linear(x, M, (int)K, had_K, hadK, scale, clip, W, sW, bias_or_null, N, y,
                                                           (hipStream_t)stream);
         if (rc1 != QR_E_UNSUPPORTED) return rc1;
     }

@@ -1,5 +1,5 @@
-// A decode step's whole linear layer in ONE launch: one token through OnlineHadamard -> Quantizer -> Linear4bit
-// (bm_gemv_kernel), one or two tokens through Quantizer -> Linear4bit (quant_gemv_kernel, quant_gemv_mt_kernel)
+// A decode step's whole linear layer in ONE launch: one or two tokens through OnlineHadamard -> Quantizer -> Linear4bit
+// (bm_gemv_kernel) or through Quantizer -> Linear4bit (quant_gemv_kernel, quant_gemv_mt_kernel)
 // (quarot/nn/hadamard.py:17-23, quarot/nn/quantization.py:10, quarot/nn/linear.py:42-56 on one or two rows).
 // A decode step at one token is latency: the transform of a 57 KB row keeps one CU busy for a few microseconds
 // while the others wait, and only then does the weight stream start.  Here EVERY workgroup transforms and
@@ -134,19 +134,22 @@ struct RowPairStream {
     }
 };
 
-// n = 1024 K (K = order of the table, a multiple of 4, at most 32).  A wave takes `ng` consecutive pairs of weight
+// n = 1024 K (K = order of the table, a multiple of 4, at most 32), MB = 1 or 2 tokens (the rows are transformed one
+// after the other, the second row's pieces requested when the first's are consumed).  A wave takes `ng` consecutive pairs of weight
 // rows as one flattened sequence of 1 KB segments, RD segments in flight (first requested while the row is transformed).
-template <int RD>
+template <int MB>
 __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x, int K, const f16* __restrict__ hadK,
                                                        float scale, float clip, const uint8_t* __restrict__ B,
                                                        const f16* __restrict__ sB, const f16* __restrict__ bias, int N,
                                                        int ng, f16* __restrict__ Y) {
+    constexpr int RD = RING;
     constexpr int NW = 16, M_ = 1024, CT = M_ / 16, RT = 2, TS = 17;
     extern __shared__ f32x4 smem_raw[];
     __shared__ u32 red[NW];
+    __shared__ f16 sc[MB];
     u32x4* Tl = (u32x4*)smem_raw;                // [4][CT][TS]
-    u32x2* xq = (u32x2*)(Tl + 4 * CT * TS);      // codes of the transformed row, K * 512 bytes
-    u32x4* hk = (u32x4*)(xq + K * 64);           // the table, K * K halves
+    u32x2* xq = (u32x2*)(Tl + 4 * CT * TS);      // codes of the transformed rows, K * 512 bytes each
+    u32x4* hk = (u32x4*)(xq + MB * K * 64);      // the table, K * K halves
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l16 = lane & 15, g = lane >> 4;
     const int Kb = K * (M_ / 2);
@@ -159,19 +162,22 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
     const bool works = wave * 2 < K;
     const int pair = works ? wave : 0;
     u32x4 raw[4];
+    auto request = [&](int row) {
 #pragma unroll
-    for (int sg = 0; sg < 2; ++sg)
+        for (int sg = 0; sg < 2; ++sg)
 #pragma unroll
-        for (int bt = 0; bt < 2; ++bt)
-            raw[sg * 2 + bt] = *((const u32x4*)x + (pair * 2 + sg) * 128 + bt * 64 + l16 * 4 + g);
+            for (int bt = 0; bt < 2; ++bt)
+                raw[sg * 2 + bt] = *((const u32x4*)x + (int64_t)row * (K * 128) + (pair * 2 + sg) * 128 + bt * 64 + l16 * 4 + g);
+    };
+    request(0);
     // (Lanes take the pieces in the order the matrix instruction wants them, neighbouring lanes 64 bytes apart; loading
     // them as they lie and swapping lanes through LDS was measured 0.1 us slower.)
 
     // ---- the weight stream of this wave ----------------------------------------------------------------------
-    RowPairStream<1> ws;
+    RowPairStream<MB> ws;
     ws.init(B, sB, bias, N, Kb, ng, wave, lane);
-    auto fetch = [&](RowPairStream<1>::Seg& sg) { ws.fetch(sg); };
-    using Seg = RowPairStream<1>::Seg;
+    auto fetch = [&](typename RowPairStream<MB>::Seg& sg) { ws.fetch(sg); };
+    using Seg = typename RowPairStream<MB>::Seg;
 
     // ---- fragments: Sylvester factors of both stages -----------------------------------------------------------
     f16x8 ha[2], hb[2];
@@ -187,10 +193,13 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
     __syncthreads();
     // every wave's requests for the row now stand before every weight request in the CU's memory queue
     Seg ring[RD];
-#pragma unroll
-    for (int r = 0; r < F0; ++r) fetch(ring[r]);
+    static_assert(F0 == 1 && F1 == 2 && F2 == 2 && F3 == 0 && RD == 5, "the request points below spell this schedule out");
+    fetch(ring[0]);
     if (tid < 128) hk[tid] = hpiece;        // (read after the next barrier)
+    f16 sh_one = (f16)0;                         // MB == 1: the row's scale stays in a register
 
+#pragma unroll
+    for (int row = 0; row < MB; ++row) {
     // ---- H_1024 of the wave's two segments as H_32 (x) H_32, into the fragment order of the table stage ------
     if (works) {
 #pragma unroll
@@ -231,8 +240,14 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
                 }
         }
     }
-#pragma unroll
-    for (int r = F0; r < F0 + F1; ++r) fetch(ring[r]);
+    if (row + 1 < MB) request(row + 1);          // (the row's pieces are consumed: the next row's take their registers)
+    // (two tokens: one segment at each of the four points of the two fronts instead of two at each of the two)
+    if constexpr (MB == 1) {
+        fetch(ring[1]);
+        fetch(ring[2]);
+    } else {
+        fetch(ring[1 + 2 * row]);
+    }
     __syncthreads();
 
     // ---- the table stage, the row's maximum, the codes (into LDS) -------------------------------------------
@@ -284,13 +299,19 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
     }
     mx = wave_max_u32_dpp(mx);
     if (lane == 0) red[wave] = mx;
-#pragma unroll
-    for (int r = F0 + F1; r < F0 + F1 + F2; ++r) fetch(ring[r]);
+    if constexpr (MB == 1) {
+        fetch(ring[3]);
+        fetch(ring[4]);
+    } else {
+        fetch(ring[2 + 2 * row]);
+    }
     __syncthreads();
 #pragma unroll
     for (int w = 0; w < NW; ++w) mx = mx > red[w] ? mx : red[w];
     const f16 sh = quantizer_scale(f16_from_bits((unsigned short)mx), clip);
     const float sp = (float)sh;
+    if (MB > 1 && tid == 0) sc[row] = sh;
+    sh_one = sh;
     u32 c01[RT], c23[RT];
     auto codes_from = [&](auto pair) {
 #pragma unroll
@@ -325,14 +346,15 @@ __global__ __launch_bounds__(1024) void bm_gemv_kernel(const f16* __restrict__ x
         const u32 od = __builtin_amdgcn_perm(s1[1], s1[0], 0x07060302u);
         const auto s2 = __builtin_amdgcn_permlane16_swap(ev, od, false, false);
         const u32x2 outv = {__builtin_amdgcn_perm(s2[1], s2[0], 0x05040100u), __builtin_amdgcn_perm(s2[1], s2[0], 0x07060302u)};
-        if (dval[rt]) xq[(rt * 16 + l16) * (M_ / 16) + wave * 4 + g] = outv;
+        if (dval[rt]) xq[row * (K * 64) + (rt * 16 + l16) * (M_ / 16) + wave * 4 + g] = outv;
     }
-#pragma unroll
-    for (int r = F0 + F1 + F2; r < RD; ++r) fetch(ring[r]);
+    // (the next row's first stage writes the table stage's operand only after the barrier above, behind every wave's
+    // reads of it; the maxima are next written behind the next barrier)
+    }
     __syncthreads();
 
     // ---- the dot products -----------------------------------------------------------------------------------
-    ws.run(ring, xq, sh, 1, Y);
+    ws.run(ring, xq, MB == 1 ? sh_one : sc[ws.my_m], MB, Y);
 }
 
 // ---- Quantizer -> Linear4bit for one token (no Hadamard in front) ---------------------------------------------
@@ -472,24 +494,30 @@ __global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __rest
 
 }  // namespace
 
-// api.hip: the whole layer for one token where the row is 1024 K halves behind a table of order K <= 32.
+// api.hip: the whole layer for one or two tokens whose rows are 1024 K halves behind a table of order K <= 32.
 // QR_E_UNSUPPORTED (nothing launched) for every other shape: the caller then chains the two kernels.
-__attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(const void* x, int n, int K, const void* hadK,
-                                                                            float scale, float clip, const void* W,
-                                                                            const void* sW, const void* bias, int64_t N,
-                                                                            void* y, hipStream_t st) {
-    if (K < 4 || K > 32 || (K & 3) != 0 || n != 1024 * K || N <= 0 || N > (1 << 30)) return QR_E_UNSUPPORTED;
+__attribute__((visibility("hidden"))) int qr_internal_token_hadamard_linear(const void* x, int64_t M, int n, int K,
+                                                                            const void* hadK, float scale, float clip,
+                                                                            const void* W, const void* sW, const void* bias,
+                                                                            int64_t N, void* y, hipStream_t st) {
+    if (M < 1 || M > 2 || K < 4 || K > 32 || (K & 3) != 0 || n != 1024 * K || N <= 0 || N > (1 << 30)) return QR_E_UNSUPPORTED;
     if (((uintptr_t)x & 15) || ((uintptr_t)W & 15) || ((uintptr_t)hadK & 15)) return QR_E_UNSUPPORTED;
     const int cus = qr_device().cus;
     const int64_t groups = (N + 1) / 2;
     const int ng = (int)((groups + (int64_t)cus * 16 - 1) / ((int64_t)cus * 16));
     const unsigned grid = (unsigned)(((groups + ng - 1) / ng + 15) / 16);
-    const size_t lds = (size_t)4 * 64 * 17 * 16 + (size_t)K * 512 + 128 * 16;
-    auto kern = bm_gemv_kernel<RING>;
-    hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);
-    if (e != hipSuccess) return (int)e;
-    kern<<<dim3(grid), dim3(1024), lds, st>>>((const f16*)x, K, (const f16*)hadK, scale, clip, (const uint8_t*)W,
-                                                        (const f16*)sW, (const f16*)bias, (int)N, ng, (f16*)y);
+    const size_t lds = (size_t)4 * 64 * 17 * 16 + (size_t)M * K * 512 + 128 * 16;
+#define QR_BG(MBV)                                                                                                        \
+    do {                                                                                                                  \
+        auto kern = bm_gemv_kernel<MBV>;                                                                                  \
+        hipError_t e = qr_allow_dynamic_lds((const void*)kern, lds);                                                      \
+        if (e != hipSuccess) return (int)e;                                                                               \
+        kern<<<dim3(grid), dim3(1024), lds, st>>>((const f16*)x, K, (const f16*)hadK, scale, clip, (const uint8_t*)W,     \
+                                                  (const f16*)sW, (const f16*)bias, (int)N, ng, (f16*)y);                 \
+    } while (0)
+    if (M == 1) QR_BG(1);
+    else QR_BG(2);
+#undef QR_BG
     return qr_launch_status();
 }
 

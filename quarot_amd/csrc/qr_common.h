@@ -97,9 +97,9 @@ int qr_internal_hadamard128_f16(const void* x, void* y, int64_t rows, float scal
 int qr_internal_heads_matrix_quantize(const void* x, int64_t rows, int heads, const void* hadK, float clip, void* q,
                                       void* scales, void* y_or_null, hipStream_t st);
 
-// decode_fused.hip: Hadamard + quantiser + linear layer of ONE token in one launch (rows of 1024 K halves, K <= 32);
-// QR_E_UNSUPPORTED, with nothing launched, for any other shape
-int qr_internal_token_hadamard_linear(const void* x, int n, int K, const void* hadK, float scale, float clip,
+// decode_fused.hip: Hadamard + quantiser + linear layer of one or two tokens in one launch (rows of 1024 K halves,
+// K <= 32); QR_E_UNSUPPORTED, with nothing launched, for any other shape
+int qr_internal_token_hadamard_linear(const void* x, int64_t M, int n, int K, const void* hadK, float scale, float clip,
                                       const void* W, const void* sW, const void* bias, int64_t N, void* y, hipStream_t st);
 
 // decode_fused.hip: quantiser + linear layer of one or two tokens in one launch; QR_E_UNSUPPORTED, with nothing

@@ -1122,7 +1122,7 @@ def test_decode_step_replays_from_a_hip_graph():
         assert np.array_equal(p.quantized_x.cpu().numpy(), wq)
 
 
-@pytest.mark.parametrize("k,m,had", [(12288, 1, True), (28672, 1, True), (4096, 1, False), (8192, 2, False)])
+@pytest.mark.parametrize("k,m,had", [(12288, 1, True), (28672, 1, True), (20480, 2, True), (4096, 1, False), (8192, 2, False)])
 def test_one_launch_decode_steps_replay_from_a_hip_graph(k, m, had):
     """The decode steps that are ONE kernel (one token behind a 1024-point Hadamard factor; one or two tokens behind the
     plain quantiser) captured into a HIP graph: every replay, with fresh inputs copied into the static buffer and eager
@@ -1346,15 +1346,16 @@ def test_runs_on_the_current_stream():
     assert np.array_equal(q.cpu().numpy(), wq)
 
 
+@pytest.mark.parametrize("M", [1, 2])
 @pytest.mark.parametrize("n", [12288, 20480, 28672])
-def test_one_token_hadamard_linear_in_one_launch(n):
-    """One token behind a 1024-point factor and a table of order 12, 20 or 28: qr_quantized_linear_f16 runs the front
-    and the dot products in ONE kernel in which every workgroup transforms the row itself.  Its output must carry the
+def test_one_token_hadamard_linear_in_one_launch(n, M):
+    """One or two tokens behind a 1024-point factor and a table of order 12, 20 or 28: qr_quantized_linear_f16 runs the front
+    and the dot products in ONE kernel in which every workgroup transforms the rows itself.  Its output must carry the
     bits of the two-launch chain (same codes, same scale, same sums, same epilogue) for any number of weight rows
     (odd, one, more than one pass per wave), with and without bias, with a clip that lets the clamp act, and on rows
     holding zeros only, an infinity, a NaN or values that overflow the transform; the oracle's Quantizer + Linear4bit on
     the kernel's own transformed row (itself within rtol / atol 1e-3 of the oracle's transform) closes the chain."""
-    rng = np.random.default_rng(n)
+    rng = np.random.default_rng(n + M)
     hadK, K = quarot_amd.functional.hadamard.get_hadK(n)
     hadK = hadK.to(dev()).half()
     had = quarot_amd.nn.OnlineHadamard(n).to(dev())
@@ -1363,11 +1364,14 @@ def test_one_token_hadamard_linear_in_one_launch(n):
         w = gpu(rng.integers(0, 256, (N, n // 2), dtype=np.uint8))
         sw = gpu((np.abs(rng.standard_normal((N, 1))) * 0.01 + 0.001).astype(F16))
         b = gpu(rng.standard_normal(N).astype(F16)) if bias else None
-        x = gpu(synth_x(1, n, seed=N + n, outliers=N % 2 == 1))
+        xn = synth_x(M, n, seed=N + n, outliers=N % 2 == 1)
+        if M == 2:
+            xn[1] *= F16(0.21)
+        x = gpu(xn)
         got = quarot_amd.quantized_linear(x, w, sw, b, hadK, K, clip_ratio=clip)
         p = quarot_amd.hadamard_quantize(x, hadK, K, clip_ratio=clip)
         want = quarot_amd.linear_i4(p.quantized_x, p.scales_x, w, sw, b)
-        assert got.shape == (1, N) and torch.equal(got, want), (n, N)
+        assert got.shape == (M, N) and torch.equal(got, want), (n, N)
         if N <= 4097:
             xh = had(x).cpu().numpy()
             ref = o.online_hadamard(x.cpu().numpy()).astype(np.float64)
@@ -1379,13 +1383,13 @@ def test_one_token_hadamard_linear_in_one_launch(n):
     w = gpu(rng.integers(0, 256, (N, n // 2), dtype=np.uint8))
     sw = gpu((np.abs(rng.standard_normal((N, 1))) * 0.01 + 0.001).astype(F16))
     for case in ("zeros", "inf", "nan", "overflow", "tiny"):
-        x = synth_x(1, n, seed=5)
+        x = synth_x(M, n, seed=5)
         if case == "zeros":
-            x[:] = 0
+            x[M - 1] = 0
         elif case == "inf":
-            x[0, 5] = np.inf
+            x[M - 1, 5] = np.inf
         elif case == "nan":
-            x[0, n - 3] = np.nan
+            x[M - 1, n - 3] = np.nan
         elif case == "overflow":
             with np.errstate(over="ignore"):
                 x = (x.astype(F32) * F32(900)).astype(F16)          # infinities where the product leaves the fp16 range
