@@ -116,3 +116,26 @@ def test_cache_class_holds_the_token_for_the_attention_call_and_never_shows_a_st
     c4 = fresh()
     c4.update(*steps[0][:2], 0, {})(steps[0][2])
     assert torch.equal(specs["kv_data"], c4.pages)
+
+
+@pytest.mark.parametrize("page_size", [16, 5])
+@pytest.mark.parametrize("B,heads", [(40, 32), (12, 24)])
+def test_append_and_attention_with_many_sequence_head_pairs(B, heads, page_size):
+    """Batches with 288 and 1280 (sequence, head) pairs: the entry point then forms workgroups of eight and of four
+    waves; pages and outputs as in the test above."""
+    rng = np.random.default_rng(B + heads + page_size)
+    lens = [int(v) for v in rng.integers(1, 90, B)]
+    data, param, indptr, indices, last = paged_case(rng, heads, page_size, lens, layers=1)
+    k, v = synth_kv(rng, B, heads), synth_kv(rng, B, heads)
+    q = (rng.standard_normal((B, heads, 128)) * 2).astype(F16)
+    tabs = (gpu(indptr), gpu(indices), gpu(last))
+    gd2, gp2 = gpu(data), gpu(param)
+    kv.quantize_append_kv_i4(gd2, gp2, *tabs, gpu(k), gpu(v), None, 0, hadamard=True)
+    two = torch.empty((B, heads, 128), dtype=torch.float16, device="cuda:0")
+    kv.batch_decode_i4(two, gpu(q), gd2, gp2, *tabs, 0, q_hadamard=True)
+    want = o.paged_batch_decode(o.kv_hadamard(q), gd2.cpu().numpy(), gp2.cpu().numpy(), indptr, indices, last, 0)
+    gd1, gp1 = gpu(data), gpu(param)
+    one = torch.full_like(two, float("nan"))
+    kv.batch_decode_i4(one, gpu(q), gd1, gp1, *tabs, 0, q_hadamard=True, append=(gpu(k), gpu(v), True))
+    assert torch.equal(gd1, gd2) and torch.equal(gp1.view(torch.int16), gp2.view(torch.int16))
+    assert close(one.cpu().numpy(), want) and close(one.cpu().numpy(), two.cpu().numpy())
