@@ -3,8 +3,8 @@ quantiser and its inverse, the paged int4 cache (append, quantise-and-append, si
 the cache) and the cache class the model code drives.  Pages of fp16 (the reference's disable_quant
 debugging mode) are not built."""
 import functools
-import weakref
 import math
+import weakref
 
 import torch
 
