@@ -139,3 +139,43 @@ def test_append_and_attention_with_many_sequence_head_pairs(B, heads, page_size)
     kv.batch_decode_i4(one, gpu(q), gd1, gp1, *tabs, 0, q_hadamard=True, append=(gpu(k), gpu(v), True))
     assert torch.equal(gd1, gd2) and torch.equal(gp1.view(torch.int16), gp2.view(torch.int16))
     assert close(one.cpu().numpy(), want) and close(one.cpu().numpy(), two.cpu().numpy())
+
+
+def test_one_launch_decode_step_replays_from_a_hip_graph_and_rejects_wrong_shapes():
+    """The step's one launch captured into a HIP graph: replays with fresh keys, values and queries copied into the
+    static buffers, eager work and synchronisation in between, store the same pages and give the same outputs as the
+    eager two-launch step.  The Python mirror refuses new-token tensors of the wrong shape, dtype or layout."""
+    rng = np.random.default_rng(21)
+    heads, P, lens = 8, 16, [300, 17, 64]
+    B = len(lens)
+    data, param, indptr, indices, last = paged_case(rng, heads, P, lens, layers=1)
+    tabs = (gpu(indptr), gpu(indices), gpu(last))
+    gd1, gp1 = gpu(data), gpu(param)
+    sk, sv, sq = (torch.zeros((B, heads, 128), dtype=torch.float16, device="cuda:0") for _ in range(3))
+    out = torch.empty_like(sq)
+    step = lambda: kv.batch_decode_i4(out, sq, gd1, gp1, *tabs, 0, q_hadamard=True, append=(sk, sv, True))
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(4):
+        k, v = gpu(synth_kv(rng, B, heads)), gpu(synth_kv(rng, B, heads))
+        q = gpu((rng.standard_normal((B, heads, 128)) * 2).astype(F16))
+        gd2, gp2 = gpu(data), gpu(param)
+        kv.quantize_append_kv_i4(gd2, gp2, *tabs, k, v, None, 0, hadamard=True)          # eager work between the replays
+        two = torch.empty_like(out)
+        kv.batch_decode_i4(two, q, gd2, gp2, *tabs, 0, q_hadamard=True)
+        torch.cuda.synchronize()
+        sk.copy_(k); sv.copy_(v); sq.copy_(q)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gd1, gd2) and torch.equal(gp1.view(torch.int16), gp2.view(torch.int16)), f"replay {i}"
+        assert close(out.cpu().numpy(), two.cpu().numpy()), f"replay {i}"
+    q = gpu(rng.standard_normal((B, heads, 128)).astype(F16))
+    good = gpu(synth_kv(rng, B, heads))
+    for bad in (good[:, :, :64], good.float(), good[:2].contiguous(), good.view(B, heads * 128), good.transpose(0, 1)):
+        with pytest.raises(RuntimeError):
+            kv.batch_decode_i4(out, q, gd1, gp1, *tabs, 0, q_hadamard=True, append=(bad, good, True))
+        with pytest.raises(RuntimeError):
+            kv.batch_decode_i4(out, q, gd1, gp1, *tabs, 0, q_hadamard=True, append=(good, bad, True))
