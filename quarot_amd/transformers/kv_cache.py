@@ -318,7 +318,8 @@ class MultiLayerPagedKVCache4Bit:
     # A decode step's new token is quantised and stored by the attention launch that follows update() (one launch per
     # step instead of two).  Whoever looks at the cache before that call -- the page tensors, the tables, the next
     # update -- first gets the token stored by the quantise-and-append kernel, so the cache never shows a state the
-    # reference's would not.
+    # reference's would not.  The key and value tensors handed to update() are read by that later launch: they must
+    # keep their contents until the returned callable has run (the reference reads them inside update()).
     @property
     def pages(self):
         self._flush()
