@@ -96,6 +96,9 @@ int qr_quantize_rows_f16_i4(const void* x, float clip, int64_t rows, int64_t col
  *   hadK is then fp32 [K,K]), optionally | QR_HADK_SIGNS (hadK is then the table's sign words, see above);
  *   y_or_null: optional fp16 [rows, n] copy of the transformed rows.
  *   x and y 16-byte aligned, q 8-byte aligned.
+ *   Rows of 128 in fp16 mode need y_or_null (qr_hadamard's kernel for that length writes them and the quantiser reads
+ *   them back: two launches); without it, and for rows shorter than 8 K, QR_E_UNSUPPORTED: call qr_hadamard and
+ *   qr_quantize_rows_f16_i4.
  */
 int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, int K, const void* hadK,
                                 int mode, float scale, float clip, void* q, void* scales,

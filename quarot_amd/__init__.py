@@ -205,6 +205,12 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
         if rc == _lib.QR_E_UNSUPPORTED:
             rc = _lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
                                                         float(clip_ratio), _ptr(q), _ptr(s), _ptr(y), _lib.stream_ptr(dev))
+        if rc == _lib.QR_E_UNSUPPORTED and n <= 128:
+            # rows this short are not fused (rows of 128 only with a place for the transformed rows): the two kernels
+            # that Sequential(OnlineHadamard, Quantizer) runs, so the bits are those of the two modules
+            y = functional.matmul_hadU_cuda(x2.float() if force_fp32 else x2, hadK, int(K)).to(torch.float16)
+            q, s = quantize_rows(y, clip_ratio)
+            rc = 0
         _lib.check(rc)
     s_shape = tuple(lead[:1]) + (1,) + tuple(lead[1:])
     packed = PackedQuantizedTensor(q.view(*lead, q.shape[-1]), s.view(s_shape))

@@ -26,7 +26,9 @@ inline size_t align16(size_t v) { return (v + 15) & ~(size_t)15; }
 
 extern "C" size_t qr_quantized_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return align16((size_t)M * (size_t)((K + 1) / 2)) + align16((size_t)M * 2) + qr_workspace_bytes(M, N, K);
+    // (rows of 128: room for the transformed rows, which the fused front of that length writes and reads back)
+    return align16((size_t)M * (size_t)((K + 1) / 2)) + align16((size_t)M * 2) + (K == 128 ? align16((size_t)M * 256) : 0) +
+           qr_workspace_bytes(M, N, K);
 }
 
 extern "C" int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int had_K, const void* hadK, int mode,
@@ -41,7 +43,14 @@ extern "C" int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int 
     uint8_t* codes = (uint8_t*)workspace;
     uint8_t* scales = codes + codes_bytes;
     uint8_t* rest = scales + scales_bytes;
-    const size_t rest_bytes = workspace_bytes - codes_bytes - scales_bytes;
+    size_t rest_bytes = workspace_bytes - codes_bytes - scales_bytes;
+    void* transformed = nullptr;                            // rows of 128 behind a Hadamard: see qr_hadamard_quantize_f16_i4
+    if (K == 128 && had_K == 1 && mode == QR_DTYPE_F16) {
+        const size_t t_bytes = align16((size_t)M * 256);
+        if (rest_bytes < t_bytes) return QR_E_WORKSPACE;
+        transformed = rest;
+        rest += t_bytes, rest_bytes -= t_bytes;
+    }
     // one token behind a long power-of-two factor: the front and the dot products in one launch (same codes, same sums)
     if (M <= 2 && had_K > 1 && mode == QR_DTYPE_F16 && hadK && ((uintptr_t)y & 1) == 0) {
         const int rc1 = qr_internal_token_hadamard_linear(x, M, (int)K, had_K, hadK, scale, clip, W, sW, bias_or_null, N, y,
@@ -54,7 +63,7 @@ extern "C" int qr_quantized_linear_f16(const void* x, int64_t M, int64_t K, int 
     }
     int rc = had_K == 0 ? qr_quantize_rows_f16_i4(x, clip, M, K, codes, scales, stream)
                         : qr_hadamard_quantize_f16_i4(x, M, (int)K, had_K, hadK, mode, scale, clip, codes, scales,
-                                                      nullptr, stream);
+                                                      transformed, stream);
     if (rc != QR_OK) return rc;
     return qr_linear_i4_f16_ws(codes, scales, W, sW, bias_or_null, M, N, K, y, rest_bytes ? rest : nullptr, rest_bytes,
                                stream);

@@ -2480,6 +2480,16 @@ extern "C" int qr_hadamard_quantize_f16_i4(const void* x, int64_t rows, int n, i
         return launch_hadamard_mm<true, true>(x, nullptr, rows, n, K, hadK, scale, clip, q, scales, st, 0, 1);
     }
     if (tiny_applies(n, K)) return QR_E_UNSUPPORTED;       // rows this short: qr_hadamard, then qr_quantize_rows_f16_i4
+    if (mode == QR_DTYPE_F16 && K == 1 && n == 128) {
+        // head-dimension rows: qr_hadamard's kernel for this length adds in another order than the general kernel below
+        // (results one fp16 step apart now and then), so the transformed rows are written by THAT kernel and quantised
+        // from memory: this call and qr_hadamard followed by the quantiser stay on the same bits.  Without a place for
+        // the transformed rows nothing is launched.
+        if (!y_or_null) return QR_E_UNSUPPORTED;
+        rc = qr_internal_hadamard128_f16(x, y_or_null, rows, scale, st);
+        if (rc != QR_OK) return rc;
+        return qr_quantize_rows_f16_i4(y_or_null, clip, rows, n, q, scales, stream);
+    }
     if (K == 1 && pow2_split(n))
         return launch_hadamard_mm<true, true>(x, y_or_null, rows, n, pow2_split(n), nullptr, scale, clip, q, scales, st);
     if (mode == QR_DTYPE_F16 && bm_applies(n, K))

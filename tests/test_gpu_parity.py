@@ -643,6 +643,47 @@ def test_fused_fronts_random_shapes_scales_and_clips():
         assert torch.equal(p2.scales_x.reshape(-1)[ok].view(torch.int16), scale.reshape(-1)[ok].view(torch.int16)), tag
 
 
+@pytest.mark.parametrize("n", [128, 112, 80, 48, 24])
+def test_fused_front_on_short_rows_carries_the_bits_of_the_two_modules(n):
+    """Rows of 128 (the head dimension: qr_hadamard has a kernel of its own for them, which adds in another order
+    than the general one) and rows too short for the fused kernels: OnlineHadamardQuantizer must return what
+    Sequential(OnlineHadamard, Quantizer) returns, bit for bit, also on data whose dynamic range makes the order of
+    the fp32 additions visible in the last fp16 bit; the one-call linear layer likewise."""
+    torch.manual_seed(n)
+    rows = 20000 if n == 128 else 3000
+    x = torch.randn(rows, n, device="cuda") * 300
+    x[:, ::7] *= 20
+    x = x.half()
+    for fp32 in (False, True):
+        had = quarot_amd.nn.OnlineHadamard(n, force_fp32=fp32).cuda()
+        fused = quarot_amd.nn.OnlineHadamardQuantizer(n, force_fp32=fp32, input_clip_ratio=0.9).cuda()
+        y = had(x)
+        want = quarot_amd.nn.Quantizer(0.9)(y)
+        p = fused(x)
+        p2, y2 = quarot_amd.hadamard_quantize(x, fused.had_rem_dim, fused.rem_dim, 0.9, force_fp32=fp32, return_transformed=True)
+        assert torch.equal(y2, y), (n, fp32)
+        for got in (p, p2):
+            assert torch.equal(got.quantized_x, want.quantized_x), (n, fp32)
+            assert torch.equal(got.scales_x.view(torch.int16), want.scales_x.view(torch.int16)), (n, fp32)
+        wq, ws = o.quantizer(y[:500].cpu().numpy(), 0.9)
+        assert np.array_equal(p.quantized_x[:500].cpu().numpy(), wq)
+        assert np.array_equal(p.scales_x.reshape(-1)[:500].cpu().numpy(), ws)
+        # (values of a few thousand next to values of a few: the roundings of the large ones are what separates two
+        # correct fp16 results, so the tolerance follows the row's largest magnitude)
+        ref = o.online_hadamard(x[:64].cpu().numpy(), force_fp32=fp32).astype(np.float64)
+        err = np.abs(y[:64].cpu().numpy().astype(np.float64) - ref).max(axis=1)
+        assert np.all(err <= 2e-3 * np.abs(ref).max(axis=1) + ATOL), (n, fp32)
+    if n % 64 == 0:
+        g = torch.Generator().manual_seed(n)
+        w = torch.randint(0, 256, (96, n // 2), dtype=torch.uint8, generator=g).cuda()
+        sw = (torch.rand(96, 1, generator=g) * 0.02 + 1e-3).half().cuda()
+        for m in (1, 2, 70, 700):
+            pm = quarot_amd.nn.Quantizer(0.9)(quarot_amd.nn.OnlineHadamard(n).cuda()(x[:m]))
+            want_y = quarot_amd.linear_i4(pm.quantized_x, pm.scales_x, w, sw)
+            got_y = quarot_amd.quantized_linear(x[:m], w, sw, None, None, 1, 0.9)
+            assert torch.equal(got_y.view(torch.int16), want_y.view(torch.int16)), m
+
+
 @pytest.mark.parametrize("n", [11008, 8960, 6912, 13824, 5120, 4608, 17920])
 def test_fused_hadamard_quantize_lean_kernel_rows_of_every_kind(n):
     """Without the copy of the transformed rows the m = 64 widths (and m = 128 behind a table of order 36 .. 60 or
