@@ -32,7 +32,7 @@ __device__ __forceinline__ void kv_butterfly(float (&v)[8], int lane) {
 template <int MASK>
 __device__ __forceinline__ void kv_minmax(float& mn, float& mx) {
     float a = kv_lane_xor<MASK>(mn), b = kv_lane_xor<MASK>(mx);
-    mn = a < mn ? a : mn;
+    mn = __builtin_fminf(a, mn);                                   // (the instruction's minimum: see min_of_pair)
     mx = b > mx ? b : mx;
 }
 
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
                 mn2 = __builtin_elementwise_min(mn2, as_f16x2(hp[i]));
                 mx2 = __builtin_elementwise_max(mx2, as_f16x2(hp[i]));
             }
-            const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+            const f16 mn0 = min_of_pair(mn2);
             const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
             f16x2 pr = {mn0, -mx0};
             if (LG > 0) pr = kv_pair_min<1>(pr);
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(KT) void kv_quant_kernel(const u32x4* __restrict__ 
             float nan_seen = amax > 0x7c00u ? 1.0f : 0.0f;       // magnitude bits above infinity's: a NaN in this lane
 #pragma unroll
             for (int e = 1; e < 8; ++e) {
-                mn = v[e] < mn ? v[e] : mn;
+                mn = __builtin_fminf(v[e], mn);
                 mx = v[e] > mx ? v[e] : mx;
             }
             float nan_lo = 0.0f;                                 // (unused minimum of the flag; the maximum is the "any")
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                     mn2 = __builtin_elementwise_min(mn2, as_f16x2(yw[jt][qq][w]));
                     mx2 = __builtin_elementwise_max(mx2, as_f16x2(yw[jt][qq][w]));
                 }
-        const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+        const f16 mn0 = min_of_pair(mn2);
         const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
         f16x2 pr = {mn0, -mx0};                                    // (min, -max): one packed min across the two lanes
         const f16x2 other = as_f16x2((u32)__shfl_xor((int)__builtin_bit_cast(u32, pr), 32, 64));
@@ -456,14 +456,14 @@ __global__ __launch_bounds__(64 * KM_WAVES, 2) void kv_had128_kernel(const u32x4
                         for (int e = 0; e < 2; ++e) {
                             const float t = (float)p[e];
                             has_nan = has_nan || (t != t);
-                            mn = t < mn ? t : mn;
+                            mn = __builtin_fminf(t, mn);
                             mx = t > mx ? t : mx;
                         }
                     }
             const float omn = __shfl_xor(mn, 32, 64), omx = __shfl_xor(mx, 32, 64);
             const int other_nan = __shfl_xor((int)has_nan, 32, 64);    // (every lane takes part: behind a short-circuit
             has_nan = has_nan || other_nan != 0;                       //  `||` the lanes that hold the NaN would sit the exchange out)
-            mn = omn < mn ? omn : mn;
+            mn = __builtin_fminf(omn, mn);
             mx = omx > mx ? omx : mx;
             if (has_nan) mn = mx = __builtin_nanf("");
             f16 rng = (f16)(mx - mn);

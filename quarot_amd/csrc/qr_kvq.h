@@ -36,6 +36,11 @@ __device__ __forceinline__ u32 asym_codes8_fast(u32x4 v, f16 zero, FastRecip f) 
     }
     return pack_nibbles8(b);
 }
+// A vector's minimum decides the sign of a zero `zero` (= -min): a vector that holds both zeros must give the same one in
+// every kernel, whatever the order of its reduction.  All minima of the quantisers are therefore taken with the
+// hardware's minimum instructions, for which -0 is below +0 (a comparison and a selection returns whichever of two
+// zeros stands second): -0.0 if the vector holds one, and +0.0 -- hence zero = -0.0, as -min gives -- if all its zeros are +0.0.
+__device__ __forceinline__ f16 min_of_pair(f16x2 v) { return __builtin_fminf16(v[0], v[1]); }
 // ranges from which the clamp-free form is exact (see above)
 __device__ __forceinline__ bool asym_range_normal(f16 rng) { return rng >= (f16)0.0009765625f; }
 
@@ -108,7 +113,7 @@ __device__ __forceinline__ void kv_quant_one_vector(u32x4 piece, u32x4* stage, f
                 mx2 = __builtin_elementwise_max(mx2, as_f16x2(yw[jt][qq][w]));
                 am2 = __builtin_elementwise_max(am2, __builtin_bit_cast(u16x2, yw[jt][qq][w] & 0x7fff7fffu));
             }
-    const f16 mn0 = mn2[0] < mn2[1] ? mn2[0] : mn2[1];
+    const f16 mn0 = min_of_pair(mn2);
     const f16 mx0 = mx2[0] > mx2[1] ? mx2[0] : mx2[1];
     f16x2 pr = {mn0, -mx0};
     const f16x2 other = as_f16x2((u32)__shfl_xor((int)__builtin_bit_cast(u32, pr), 32, 64));
@@ -153,14 +158,14 @@ __device__ __forceinline__ void kv_quant_one_vector(u32x4 piece, u32x4* stage, f
                     for (int e = 0; e < 2; ++e) {
                         const float t = (float)p[e];
                         has_nan = has_nan || (t != t);
-                        fmn = t < fmn ? t : fmn;
+                        fmn = __builtin_fminf(t, fmn);
                         fmx = t > fmx ? t : fmx;
                     }
                 }
         const float omn = __shfl_xor(fmn, 32, 64), omx = __shfl_xor(fmx, 32, 64);
         const int other_nan = __shfl_xor((int)has_nan, 32, 64);
         has_nan = has_nan || other_nan != 0;
-        fmn = omn < fmn ? omn : fmn;
+        fmn = __builtin_fminf(omn, fmn);
         fmx = omx > fmx ? omx : fmx;
         if (has_nan) fmn = fmx = __builtin_nanf("");
         f16 rng = (f16)(fmx - fmn);

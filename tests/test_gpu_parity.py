@@ -1067,6 +1067,55 @@ def test_kv_tiny_ranges_and_sums_too_large_for_fp16(dim, hadamard):
     assert (wq[:200] >> 4).max() == 15 and (wq[:200] & 15).min() == 0
 
 
+@pytest.mark.parametrize("dim", [16, 64, 128, 256])
+def test_kv_sign_of_a_zero_minimum_does_not_depend_on_where_the_zeros_stand(dim):
+    """`zero` = -min carries the sign of the minimum when that is a zero.  A vector that holds -0.0 and +0.0 must give
+    the same `zero` in every kernel, wherever its zeros stand: the minimum is -0.0 if the vector holds one (zero =
+    +0.0) and +0.0 otherwise (zero = -0.0, as the reference's -min gives for a vector without negative zeros).  The
+    fused Hadamard + quantiser and the quantiser on the transformed vectors agree bit for bit on inputs whose
+    transform is full of zeros of both signs."""
+    from quarot_amd.transformers import kv_cache as kvc
+    g = torch.Generator().manual_seed(dim)
+    vecs = 4096
+    x = torch.rand(vecs, dim, generator=g)                                     # >= 0
+    z = torch.rand(vecs, dim, generator=g)
+    x = torch.where(z < 0.3, torch.zeros(()), x)
+    x = torch.where(z < 0.15, -torch.zeros(()), x)                             # both zeros, in random places
+    x[::4] = x[::4].abs()                                                      # every fourth vector: +0.0 only
+    x[1::8] = x[1::8] + 0.5                                                    # and some without a zero at all
+    x = x.half().cuda()
+    has_neg0 = ((x == 0) & torch.signbit(x)).any(dim=1)
+    min0 = x.amin(dim=1) == 0
+    assert bool((has_neg0 & min0).any()) and bool((~has_neg0 & min0).any()) and bool((~min0).any())
+    for xin in (x, x.flip(1).contiguous()):                                    # the same values in the opposite order
+        q, s, zero = kvc.asym_quantize_and_pack_i4(xin)
+        zb = zero.view(-1).view(torch.int16)
+        assert bool((zb[min0 & has_neg0] == 0).all())                          # +0.0
+        assert bool((zb[min0 & ~has_neg0] == -32768).all())                    # -0.0
+        wq, ws, wz = o.kv_asym_quant(xin.cpu().numpy())
+        assert np.array_equal(q.cpu().numpy(), wq) and np.array_equal(s.cpu().numpy(), ws) and np.array_equal(zero.cpu().numpy(), wz)
+        plain = ~has_neg0.cpu().numpy()                                        # (no tie between zeros: the oracle's bits too)
+        assert np.array_equal(bits(zero.cpu().numpy())[plain], bits(wz)[plain])
+    if dim == 128:
+        # one subnormal entry per vector: every transformed value is a sum too small for fp16, -0.0 or +0.0 by the
+        # signs of that entry's Hadamard column; constant vectors: one large value and exact (+0.0) zeros
+        t = torch.zeros(vecs, dim)
+        t[torch.arange(vecs), torch.randint(0, dim, (vecs,), generator=g)] = 6e-8
+        t[::2] = -t[::2]
+        t[::5] = 0.75
+        t = t.half().cuda()
+        y = kvc.matmul_had_cuda(t, torch.float16)
+        q1, s1, z1 = kvc.asym_quantize_and_pack_i4(t, hadamard=True)
+        q2, s2, z2 = kvc.asym_quantize_and_pack_i4(y)
+        assert torch.equal(q1, q2) and torch.equal(s1.view(torch.int16), s2.view(torch.int16))
+        assert torch.equal(z1.view(torch.int16), z2.view(torch.int16))
+        mins0 = y.amin(dim=1) == 0
+        neg0 = ((y == 0) & torch.signbit(y)).any(dim=1)
+        assert bool((mins0 & neg0).any()) and bool((mins0 & ~neg0).any())
+        zb = z1.view(-1).view(torch.int16)
+        assert bool((zb[mins0 & neg0] == 0).all()) and bool((zb[mins0 & ~neg0] == -32768).all())
+
+
 def test_kv_vectors_with_infinities_take_the_ieee_path():
     """An infinite element makes range and scale infinite: every finite element then gets code 0 and
     inf / inf (NaN) converts to 0, as round/clamp/cast give in the reference; neighbouring finite
