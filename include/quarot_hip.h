@@ -368,6 +368,28 @@ int qr_kv_quant_append_batch_decode_f16_i4(void* o, const void* q, int q_had_mod
                                            void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The paged cache with fp16 pages (the reference's disable_quant mode, quarot/transformers/kv_cache.py:134-151,189-193):
+ *   kv_data fp16 [num_pages, num_layers, 2 (K, V), num_heads, page_size, 128]; kv_param and the page tables as above.
+ *
+ * qr_kv_append_f16 replaces quarot._CUDA.init_kv_f16 and append_kv_f16 (quarot/kernels/bindings.cpp:287-374):
+ *   k, v fp16 [tokens, num_heads, 128]; k_param, v_param fp16 [tokens, num_heads, 2] (the cache class passes
+ *   {1, 0}); append_indptr_or_null, tokens and the alignment rules as qr_kv_append_i4.
+ * qr_batch_decode_f16 replaces quarot._CUDA.batch_decode_f16 (quarot/kernels/bindings.cpp:247-285):
+ *   o[b, h, :] = sum_j softmax_j( q[b, h, :] . k_j / sqrt(128) ) v_j over the cached fp16 vectors, fp32 arithmetic,
+ *   within rtol 1e-3 / atol 1e-3 of the exact result; kv_param is not read.  q, o fp16 [batch_size, num_heads, 128].
+ *   One workgroup per (sequence, head); a sequence without pages gets a NaN row, as qr_batch_decode_i4 gives.
+ */
+int qr_kv_append_f16(void* kv_data, void* kv_param, const void* kv_indptr, const void* kv_indices,
+                     const void* last_page_offset, int64_t num_pages, const void* k, const void* v,
+                     const void* k_param, const void* v_param, const void* append_indptr_or_null,
+                     int64_t tokens, int num_layers, int layer_idx, int num_heads, int page_size,
+                     int head_dim, int64_t batch_size, void* stream);
+int qr_batch_decode_f16(void* o, const void* q, const void* kv_data, const void* kv_param,
+                        const void* kv_indptr, const void* kv_indices, const void* last_page_offset,
+                        int64_t num_pages, int num_layers, int layer_idx, int num_heads, int page_size,
+                        int head_dim, int64_t batch_size, void* stream);
+
+/*
  * Measurement aids.  NO counterpart in the reference and no caller in the product path: kernels whose
  * work is known exactly, run by bench.py next to the workloads to calibrate the rooflines.
  *

@@ -435,3 +435,25 @@ def paged_batch_decode(q, kv_data, kv_param, kv_indptr, kv_indices, last_page_of
         w /= w.sum(axis=1, keepdims=True)
         out[b] = np.einsum("hs,shd->hd", w, vf)
     return out
+
+
+def paged_batch_decode_f16(q, kv_data, kv_indptr, kv_indices, last_page_offset, layer_idx):
+    """The same kernel over fp16 pages (quarot/kernels/bindings.cpp:247-285, the reference's disable_quant cache,
+    quarot/transformers/kv_cache.py:134-151): kv_data fp16 [pages, L, 2, H, P, D] holds the vectors themselves, the
+    parameters are not read.  float64 here; q fp16 [B, H, D] -> float64 [B, H, D]."""
+    q = np.asarray(q, dtype=F16).astype(np.float64)
+    batch, heads, dim = q.shape
+    page_size = kv_data.shape[4]
+    seq = paged_seq_lens(kv_indptr, last_page_offset, page_size)
+    out = np.zeros((batch, heads, dim), np.float64)
+    for b in range(batch):
+        pos = np.arange(int(seq[b]))
+        pages = np.asarray(kv_indices)[int(kv_indptr[b]) + pos // page_size]
+        kf = kv_data[pages, layer_idx, 0, :, pos % page_size, :].astype(np.float64)      # [seq, H, D]
+        vf = kv_data[pages, layer_idx, 1, :, pos % page_size, :].astype(np.float64)
+        logits = np.einsum("hd,shd->hs", q[b], kf) / np.sqrt(np.float64(dim))
+        logits -= logits.max(axis=1, keepdims=True)
+        w = np.exp(logits)
+        w /= w.sum(axis=1, keepdims=True)
+        out[b] = np.einsum("hs,shd->hd", w, vf)
+    return out

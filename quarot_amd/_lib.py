@@ -46,13 +46,16 @@ SIGNATURES = {
                                        _c.c_size_t, _ptr)),
     "qr_kv_quant_append_batch_decode_f16_i4": (_int, (_ptr, _ptr, _int, _ptr, _ptr, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int,
                                                       _int, _int, _int, _int, _i64, _i64, _ptr, _c.c_size_t, _ptr)),
+    "qr_kv_append_f16": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int,
+                                _i64, _ptr)),
+    "qr_batch_decode_f16": (_int, (_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _int, _int, _int, _int, _int, _i64, _ptr)),
     "qr_calib_mfma_i8": (_int, (_int, _int, _int, _ptr, _ptr)),
     "qr_calib_copy": (_int, (_ptr, _ptr, _i64, _ptr)),
 }
 
 QR_DTYPE_F16, QR_DTYPE_F32 = 0, 1
 QR_HADK_SIGNS = 0x100          # or-ed into a `mode`: hadK is passed as sign words (include/quarot_hip.h)
-QR_E_UNSUPPORTED = -3
+QR_E_NULL, QR_E_SHAPE, QR_E_UNSUPPORTED = -1, -2, -3
 
 _lib = None
 

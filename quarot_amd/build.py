@@ -13,7 +13,8 @@ PKG = pathlib.Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libquarot_hip.so"
 OBJ = PKG.parent / "build" / "obj"
-SOURCES = ("api.hip", "quant.hip", "gemm.hip", "gemm_f6.hip", "hadamard.hip", "kv.hip", "attn.hip", "calib.hip", "decode_fused.hip")
+SOURCES = ("api.hip", "quant.hip", "gemm.hip", "gemm_f6.hip", "hadamard.hip", "kv.hip", "attn.hip", "calib.hip", "decode_fused.hip",
+           "paged_f16.hip")
 FLAGS = ("--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
          # every fp16/fp32 operation must round on its own (the reference's results are defined that
          # way): no fused multiply-add contraction unless a kernel spells fma out

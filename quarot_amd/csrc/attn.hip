@@ -505,6 +505,16 @@ int check_cache(const void* kv_data, const void* kv_param, const void* kv_indptr
 
 }  // namespace
 
+// paged_f16.hip: the same argument checks for the cache with fp16 pages
+__attribute__((visibility("hidden"))) int qr_internal_check_paged_cache(const void* kv_data, const void* kv_param,
+                                                                        const void* kv_indptr, const void* kv_indices,
+                                                                        const void* last_page_offset, int64_t num_pages,
+                                                                        int num_layers, int layer_idx, int num_heads,
+                                                                        int page_size, int head_dim, int64_t batch_size) {
+    return check_cache(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, num_pages, num_layers, layer_idx, num_heads,
+                       page_size, head_dim, batch_size);
+}
+
 __attribute__((visibility("hidden"))) PagedKV qr_internal_paged_kv(void* kv_data, void* kv_param, const void* kv_indptr,
                                                                     const void* kv_indices, const void* last_page_offset,
                                                                     int64_t num_pages, int num_layers, int layer_idx,

@@ -76,3 +76,6 @@ __device__ __forceinline__ u32 pack_scale_zero(f16 scale, f16 zero) {
 PagedKV qr_internal_paged_kv(void* kv_data, void* kv_param, const void* kv_indptr, const void* kv_indices,
                              const void* last_page_offset, int64_t num_pages, int num_layers, int layer_idx,
                              int num_heads, int page_size, int64_t batch_size);
+int qr_internal_check_paged_cache(const void* kv_data, const void* kv_param, const void* kv_indptr, const void* kv_indices,
+                                  const void* last_page_offset, int64_t num_pages, int num_layers, int layer_idx,
+                                  int num_heads, int page_size, int head_dim, int64_t batch_size);

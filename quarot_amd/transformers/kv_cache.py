@@ -1,7 +1,7 @@
 """KV-cache path (mirror of quarot/transformers/kv_cache.py) on HIP kernels: the asymmetric int4
 quantiser and its inverse, the paged int4 cache (append, quantise-and-append, single-query attention over
-the cache) and the cache class the model code drives.  Pages of fp16 (the reference's disable_quant
-debugging mode) are not built."""
+the cache) and the cache class the model code drives; and the same cache with fp16 pages (the reference's
+disable_quant mode: init_kv_f16 / append_kv_f16 / batch_decode_f16)."""
 import functools
 import math
 import weakref
@@ -73,8 +73,9 @@ def matmul_had_cuda(X, dtype):
 _CHECKED = None     # the five cache tensors validated last (weak references), their element counts, their dimensions
 
 
-def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx):
-    """The checks of quarot/kernels/bindings.cpp:118-245 (CHECK_INPUT / CHECK_DIM / CHECK_EQ) as RuntimeError.
+def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx, f16=False):
+    """The checks of quarot/kernels/bindings.cpp:118-374 (CHECK_INPUT / CHECK_DIM / CHECK_EQ) as RuntimeError; f16: the
+    cache with fp16 pages (the *_f16 bindings).
     A decode step passes the same five tensor objects to the append and to the attention of every layer: the
     objects validated last (same identity, same element counts) are not walked through again."""
     global _CHECKED
@@ -82,7 +83,7 @@ def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, 
     if seen is not None:
         refs, counts, dims = seen
         if (refs[0]() is kv_data and refs[1]() is kv_param and refs[2]() is kv_indptr and refs[3]() is kv_indices
-                and refs[4]() is last_page_offset
+                and refs[4]() is last_page_offset and kv_data.dtype == (torch.float16 if f16 else torch.uint8)
                 and counts == (kv_data.numel(), kv_param.numel(), kv_indptr.numel(), kv_indices.numel(), last_page_offset.numel())):
             if not (0 <= int(layer_idx) < dims[1]):
                 raise RuntimeError(f"{fn}: layer_idx out of range")
@@ -99,8 +100,8 @@ def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, 
         raise RuntimeError(f"{fn}: kv_param must be a 6D tensor")
     if not (kv_indptr.dim() == 1 and kv_indices.dim() == 1 and last_page_offset.dim() == 1):
         raise RuntimeError(f"{fn}: kv_indptr, kv_indicies and last_page_offset must be 1D tensors")
-    if not (kv_data.dtype == torch.uint8):
-        raise RuntimeError(f"{fn}: kv_data must be uint8 (fp16 pages are not built)")
+    if not (kv_data.dtype == (torch.float16 if f16 else torch.uint8)):
+        raise RuntimeError(f"{fn}: kv_data must be {'fp16' if f16 else 'uint8'}")
     if not (kv_param.dtype == torch.float16):
         raise RuntimeError(f"{fn}: kv_param must be fp16")
     for name, t in (("kv_indptr", kv_indptr), ("kv_indicies", kv_indices), ("last_page_offset", last_page_offset)):
@@ -109,25 +110,31 @@ def _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, 
     pages, layers, two, heads, page_size, half_dim = kv_data.shape
     if not (two == 2 and tuple(kv_param.shape) == (pages, layers, 2, heads, page_size, 2)):
         raise RuntimeError(f"{fn}: kv_param must be [pages, layers, 2, heads, page_size, 2]")
-    if not (half_dim * 2 == 128):
-        raise RuntimeError(f"{fn}: CHECK_EQ(head_dim, 128) failed. {half_dim * 2} vs 128")
+    head_dim = half_dim if f16 else half_dim * 2           # (the last axis holds halves or packed pairs of codes)
+    if not (head_dim == 128):
+        raise RuntimeError(f"{fn}: CHECK_EQ(head_dim, 128) failed. {head_dim} vs 128")
     if not (0 <= int(layer_idx) < layers):
         raise RuntimeError(f"{fn}: layer_idx out of range")
-    dims = (pages, layers, heads, page_size, half_dim * 2)
+    dims = (pages, layers, heads, page_size, head_dim)
     five = (kv_data, kv_param, kv_indptr, kv_indices, last_page_offset)
     _CHECKED = (tuple(weakref.ref(t) for t in five), tuple(t.numel() for t in five), dims)
     return dims
 
 
-def _append(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
-    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx)
+def _append(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx,
+            f16=False):
+    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset,
+                                                            layer_idx, f16)
     batch = last_page_offset.shape[0]
     if not (kv_indptr.shape[0] == batch + 1):
         raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
     for name, t in (("k", k), ("v", v), ("k_param", k_param), ("v_param", v_param)):
         if not (t.is_cuda and t.is_contiguous() and t.dim() == 3):
             raise RuntimeError(f"{fn}: {name} must be a contiguous 3D CUDA tensor")
-    if not (k.shape == v.shape and k.dtype == v.dtype == torch.uint8 and tuple(k.shape[1:]) == (heads, head_dim // 2)):
+    if f16:
+        if not (k.shape == v.shape and k.dtype == v.dtype == torch.float16 and tuple(k.shape[1:]) == (heads, head_dim)):
+            raise RuntimeError(f"{fn}: k and v must be fp16 [tokens, heads, head_dim]")
+    elif not (k.shape == v.shape and k.dtype == v.dtype == torch.uint8 and tuple(k.shape[1:]) == (heads, head_dim // 2)):
         raise RuntimeError(f"{fn}: k and v must be uint8 [tokens, heads, head_dim / 2]")
     tokens = k.shape[0]
     for name, t in (("k_param", k_param), ("v_param", v_param)):
@@ -141,7 +148,8 @@ def _append(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v
             raise RuntimeError(f"{fn}: seqlen_indptr must be int32 [batch_size + 1]")
     dev = kv_data.device
     with _lib.on_device(dev):
-        _lib.check(_lib.lib().qr_kv_append_i4(
+        entry = _lib.lib().qr_kv_append_f16 if f16 else _lib.lib().qr_kv_append_i4
+        _lib.check(entry(
             kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(), last_page_offset.data_ptr(),
             pages, k.data_ptr(), v.data_ptr(), k_param.data_ptr(), v_param.data_ptr(),
             None if seqlen_indptr is None else seqlen_indptr.data_ptr(), tokens, layers, int(layer_idx), heads, page_size,
@@ -160,6 +168,44 @@ def append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, 
     """Write one new quantised K / V vector per sequence at its last position (kv_cache.py:49-58 ->
     bindings.cpp:200-245)."""
     _append("append_kv_i4", kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, None, layer_idx)
+
+
+def init_kv_f16(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr, layer_idx):
+    """init_kv_i4 for the cache with fp16 pages (kv_cache.py:69-79 -> bindings.cpp:287-330): k, v fp16
+    [tokens, heads, 128], kv_data fp16 [pages, layers, 2, heads, page_size, 128]."""
+    _append("init_kv_f16", kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, seqlen_indptr,
+            layer_idx, f16=True)
+
+
+def append_kv_f16(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, layer_idx):
+    """append_kv_i4 for the cache with fp16 pages (kv_cache.py:82-91 -> bindings.cpp:332-374)."""
+    _append("append_kv_f16", kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, k_param, v_param, None, layer_idx,
+            f16=True)
+
+
+def batch_decode_f16(o, q, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, layer_idx):
+    """o[b, h] = softmax(q[b, h] . K^T / sqrt(128)) . V over the fp16 pages of sequence b (kv_cache.py:93-101 ->
+    bindings.cpp:247-285).  Writes into `o` and returns None, like the reference's binding."""
+    fn = "batch_decode_f16"
+    pages, layers, heads, page_size, head_dim = _cache_args(fn, kv_data, kv_param, kv_indptr, kv_indices, last_page_offset,
+                                                            layer_idx, f16=True)
+    for name, t in (("o", o), ("q", q)):
+        if not (t.is_cuda and t.is_contiguous() and t.dim() == 3 and t.dtype == torch.float16):
+            raise RuntimeError(f"{fn}: {name} must be a contiguous 3D fp16 CUDA tensor")
+    if not (o.shape == q.shape):
+        raise RuntimeError(f"{fn}: o.size() != q.size()")
+    batch = o.shape[0]
+    if not (tuple(q.shape[1:]) == (heads, head_dim)):
+        raise RuntimeError(f"{fn}: q must be [batch_size, {heads}, {head_dim}]")
+    if not (kv_indptr.shape[0] == batch + 1):
+        raise RuntimeError(f"{fn}: CHECK_EQ(kv_indptr.size(0), batch_size + 1) failed")
+    if not (last_page_offset.shape[0] == batch):
+        raise RuntimeError(f"{fn}: CHECK_EQ(last_page_offset.size(0), batch_size) failed")
+    dev = kv_data.device
+    with _lib.on_device(dev):
+        _lib.check(_lib.lib().qr_batch_decode_f16(
+            o.data_ptr(), q.data_ptr(), kv_data.data_ptr(), kv_param.data_ptr(), kv_indptr.data_ptr(), kv_indices.data_ptr(),
+            last_page_offset.data_ptr(), pages, layers, int(layer_idx), heads, page_size, head_dim, batch, _lib.stream_ptr(dev)))
 
 
 def quantize_append_kv_i4(kv_data, kv_param, kv_indptr, kv_indices, last_page_offset, k, v, seqlen_indptr, layer_idx,
@@ -270,6 +316,12 @@ class _AttentionStub(object):
         batch_size, q_len, num_qo_heads, head_dim = q.shape
         assert q_len == 1
         q = q.view(batch_size, num_qo_heads, head_dim)
+        if self.disable_quant:                   # fp16 pages (kv_cache.py:116-119)
+            if self.hadamard_dtype is not None:
+                q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
+            attn_output = torch.empty_like(q)
+            batch_decode_f16(attn_output, q.contiguous(), **attention_kwargs, layer_idx=layer_idx)
+            return attn_output.unsqueeze(1)
         fused = self.hadamard_dtype == torch.float16 and q.dtype == torch.float16 and q.is_contiguous()
         if self.hadamard_dtype is not None and not fused:
             q = matmul_had_cuda(q, dtype=self.hadamard_dtype)
@@ -293,14 +345,13 @@ class MultiLayerPagedKVCache4Bit:
 
     def __init__(self, batch_size, page_size, max_seq_len, device, n_layers, num_heads, head_dim, disable_quant=False,
                  hadamard_dtype=torch.float16):
-        if disable_quant:
-            raise NotImplementedError("fp16 pages (disable_quant=True) are not built: this cache is int4 only")
         self.page_size = page_size
         self.batch_size = batch_size
         max_page_cnt = self.page_cnt_from_length(max_seq_len)
-        self.disable_quant = disable_quant
-        self._pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, head_dim // 2),
-                                  dtype=torch.uint8, device=device)
+        self.disable_quant = disable_quant       # fp16 pages instead of int4 codes (kv_cache.py:134-151)
+        self._pages = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size,
+                                   head_dim if disable_quant else head_dim // 2),
+                                  dtype=torch.float16 if disable_quant else torch.uint8, device=device)
         self._scales = torch.empty((max_page_cnt * batch_size, n_layers, 2, num_heads, page_size, 2), dtype=torch.float16,
                                    device=device)
         self._pending = {}      # layer -> (token, k, v, specs, hadamard): a decode step's new token, held for the attention call
@@ -382,6 +433,8 @@ class MultiLayerPagedKVCache4Bit:
         attention_mask = cache_kwargs.get("attention_mask")
         first = self._needs_init[layer_idx]
         specs = self.get_cache_specs_for_flash_infer(attention_mask)
+        if self.disable_quant:
+            return self._update_f16(key_states, value_states, layer_idx, attention_mask, first, specs)
         k_in, fused_had = key_states, self.hadamard_dtype is not None
         if self.hadamard_dtype is not None and self.hadamard_dtype != torch.float16:
             k_in, fused_had = matmul_had_cuda(key_states, dtype=self.hadamard_dtype), False   # e.g. the fp32 transform
@@ -418,6 +471,31 @@ class MultiLayerPagedKVCache4Bit:
             take = None
         return functools.partial(self._stub.forward, num_kv_heads=num_heads, attention_kwargs=specs, layer_idx=layer_idx,
                                  max_seq_len=self.length, workspace=self._decode_workspace(num_heads), take_pending=take)
+
+    def _update_f16(self, key_states, value_states, layer_idx, attention_mask, first, specs):
+        """update() with fp16 pages (kv_cache.py:187-251 with disable_quant): the transformed keys and the values are
+        stored as they are, with parameters {1, 0} beside them."""
+        b_sz, added_length, num_heads, head_dim = key_states.shape
+        k = key_states if self.hadamard_dtype is None else matmul_had_cuda(key_states, dtype=self.hadamard_dtype)
+        rows = self.batch_size * added_length
+        k = k.reshape(rows, num_heads, head_dim).contiguous()
+        v = value_states.reshape(rows, num_heads, head_dim).contiguous()
+        param = torch.zeros((rows, num_heads, 2), dtype=torch.float16, device=k.device)
+        param[..., 0] = 1
+        if first:
+            self._needs_init[layer_idx] = False
+            if attention_mask is not None:
+                keep = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+                k, v, param = k.index_select(0, keep), v.index_select(0, keep), param.index_select(0, keep)
+                seqlens = torch.nn.functional.pad(torch.cumsum(attention_mask.sum(dim=-1, dtype=torch.int32), dim=0,
+                                                               dtype=torch.int32), (1, 0))
+            else:
+                seqlens = torch.arange(self.batch_size + 1, device=self.device, dtype=torch.int32) * added_length
+            init_kv_f16(**specs, k=k, v=v, k_param=param, v_param=param, seqlen_indptr=seqlens, layer_idx=layer_idx)
+            return key_states, value_states
+        assert added_length == 1
+        append_kv_f16(**specs, k=k, v=v, k_param=param, v_param=param, layer_idx=layer_idx)
+        return functools.partial(self._stub.forward, num_kv_heads=num_heads, attention_kwargs=specs, layer_idx=layer_idx)
 
     def get_cache_specs_for_flash_infer(self, attention_mask):
         """Page tables of the current state (kv_cache.py:253-275): page i of sequence b is page number

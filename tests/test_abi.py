@@ -29,7 +29,7 @@ def test_header_declares_expected_entry_points():
     syms = declared_symbols()
     for must in ("qr_hadamard", "qr_sym_quant_f16_i4", "qr_quantize_rows_f16_i4", "qr_hadamard_quantize_f16_i4",
                  "qr_matmul_i4_i32", "qr_sym_dequant_i32_f16", "qr_linear_i4_f16", "qr_kv_quant_f16_i4",
-                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4", "qr_quantized_linear_workspace_bytes", "qr_quantized_linear_f16", "qr_kv_quant_append_batch_decode_f16_i4",
+                 "qr_kv_dequant_i4_f16", "qr_version", "qr_strerror", "qr_rmsnorm_quantize_f16_i4", "qr_heads_hadamard_quantize_f16_i4", "qr_quantized_linear_workspace_bytes", "qr_quantized_linear_f16", "qr_kv_quant_append_batch_decode_f16_i4", "qr_kv_append_f16", "qr_batch_decode_f16",
                  "qr_workspace_bytes", "qr_linear_i4_f16_ws", "qr_linear_i4_f16_static", "qr_f6_bytes", "qr_convert_i4_f6",
                  "qr_linear_f6_f16"):
         assert must in syms

@@ -362,8 +362,6 @@ def test_cache_class_prefill_then_decode_steps(hadamard_dtype):
             assert close(attn.cpu().numpy().reshape(B, H, 128), want)
         assert np.array_equal(cache.pages.cpu().numpy(), data)
     assert cache.get_seq_length() == prompt + 2 and cache.to_legacy_cache() is cache and cache.get_max_length() is None
-    with pytest.raises(NotImplementedError):
-        kv.MultiLayerPagedKVCache4Bit(1, 16, 16, "cuda:0", 1, 1, 128, disable_quant=True)
 
 
 def test_cache_class_padded_prompt_and_the_reference_benchmarks_fake_prefill():

@@ -549,3 +549,42 @@ def test_paged_batch_decode_against_textbook_attention():
     np.testing.assert_allclose(g0[3], o.paged_dequant(vc, vp).astype(np.float64).mean(axis=0), rtol=1e-10, atol=1e-12)
     # the other layer holds different data: a wrong layer offset changes the result
     assert not np.allclose(o.paged_batch_decode(q, data, param, indptr, indices, last, 0), got)
+
+
+def test_paged_batch_decode_over_fp16_pages_against_textbook_attention():
+    """The fp16-page form: torch's scaled_dot_product_attention in float64 on the vectors gathered page by page with
+    explicit loops, a cache whose int4 twin holds the same values (both oracles must agree), and the one-token and
+    q = 0 cases."""
+    rng = np.random.default_rng(9)
+    heads, P = 3, 8
+    lens = [1, 8, 19, 40]
+    _, _, indptr, indices, last = _paged_case(rng, 4, heads, P, lens, layers=2)
+    pool = int(indices.max()) + 4
+    data = rng.standard_normal((pool, 2, 2, heads, P, 128)).astype(F16)
+    q = rng.standard_normal((4, heads, 128)).astype(F16)
+    got = o.paged_batch_decode_f16(q, data, indptr, indices, last, 1)
+    for b in range(4):
+        ks, vs = [], []
+        for pos in range(lens[b]):
+            page = int(indices[int(indptr[b]) + pos // P])
+            ks.append(data[page, 1, 0, :, pos % P, :])
+            vs.append(data[page, 1, 1, :, pos % P, :])
+        kf = torch.from_numpy(np.stack(ks)).double().permute(1, 0, 2)
+        vf = torch.from_numpy(np.stack(vs)).double().permute(1, 0, 2)
+        want = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q[b]).double().unsqueeze(1), kf, vf)
+        np.testing.assert_allclose(got[b], want.squeeze(1).numpy(), rtol=1e-10, atol=1e-10)
+        if b == 0:
+            np.testing.assert_allclose(got[0], np.stack(vs)[0].astype(np.float64), rtol=1e-12)      # one token: v_0
+        if b == 3:
+            g0 = o.paged_batch_decode_f16(np.zeros_like(q), data, indptr, indices, last, 1)
+            np.testing.assert_allclose(g0[3], np.stack(vs).astype(np.float64).mean(axis=0), rtol=1e-10, atol=1e-12)
+    assert not np.allclose(o.paged_batch_decode_f16(q, data, indptr, indices, last, 0), got)
+    # values that int4 codes hold exactly (code * 0.25 - 1): the int4 oracle over the coded cache gives the same
+    codes = rng.integers(0, 16, (pool, 2, 2, heads, P, 128)).astype(np.uint8)
+    packed = (codes[..., 0::2] | (codes[..., 1::2] << 4)).astype(np.uint8)
+    param = np.zeros((pool, 2, 2, heads, P, 2), F16)
+    param[..., 0], param[..., 1] = 0.25, 1.0
+    exact = (codes.astype(F32) * F32(0.25) - F32(1.0)).astype(F16)
+    np.testing.assert_allclose(o.paged_batch_decode_f16(q, exact, indptr, indices, last, 0),
+                               o.paged_batch_decode(q, packed, param, indptr, indices, last, 0), rtol=1e-12, atol=1e-12)
+
