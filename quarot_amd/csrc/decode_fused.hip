@@ -427,7 +427,9 @@ __global__ __launch_bounds__(1024) void quant_gemv_kernel(const u32x4* __restric
 // to 65536 / MB halves) and every wave then takes its pairs of weight rows against all tokens.  Built for MB = 2 only:
 // with four and eight tokens every workgroup pulls 64 / 128 KB of rows through its CU's memory path before its weight
 // stream can be consumed, and the launch (70B gate_up: 43.7 / 41.8 us) is no faster than the quantiser kernel followed
-// by the shared-token decode kernel (43.5 / 43.7 us); with two tokens it is 38.2 against 43.4 us.
+// by the shared-token decode kernel (43.5 / 43.7 us); with two tokens it is 38.2 against 43.4 us.  (Eight tokens once more
+// on the present form of this kernel, no spills, ring depths 3 to 6, alternating runs on one GPU: 44.1 .. 45.4 us against
+// 44.0 for the two launches.)
 template <int MB>
 __global__ __launch_bounds__(1024) void quant_gemv_mt_kernel(const u32x4* __restrict__ x, int M, int cols8, float clip,
                                                              const uint8_t* __restrict__ B, const f16* __restrict__ sB,
