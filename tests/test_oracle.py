@@ -130,6 +130,50 @@ def test_hadamard_staged_close_to_closed_form(n, dtype):
     np.testing.assert_allclose(np.linalg.norm(got, axis=-1), np.linalg.norm(x.astype(np.float64), axis=-1), rtol=1e-3)
 
 
+def test_fwht_butterfly_had_scale_and_online_hadamard_directly():
+    """The three thin helpers on their own (their callers pin them only indirectly):
+    fwht_butterfly on integer-valued input is the exact product with scipy's natural-order Hadamard matrix, in the
+    layout the reference's loop leaves ([rows, stop_len, n / stop_len], transformed index trailing); stopping at length K
+    leaves K untouched blocks; a swapped (a - b, a + b) pair or a transform over the wrong axis fails these.
+    had_scale is the float32 quotient 1 / sqrt(float32(n)).  online_hadamard casts to fp32 and back exactly when told
+    to, and otherwise rounds to fp16 between the two factors (it differs from the fp32 form in that case only)."""
+    rng = np.random.default_rng(21)
+    for n in (2, 8, 64):
+        x = rng.integers(-50, 50, (3, n)).astype(np.float64)
+        got = o.fwht_butterfly(x)
+        assert got.shape == (3, 1, n)
+        assert np.array_equal(got[:, 0, :], x @ scipy.linalg.hadamard(n).T)
+    # 24 = 12 blocks of 2 (the order in which matmul_hadU leaves them: block index k = i // 2 leading)
+    x = rng.integers(-50, 50, (2, 24)).astype(np.float64)
+    got = o.fwht_butterfly(x, stop_len=12)
+    assert got.shape == (2, 12, 2)
+    blocks = x.reshape(2, 12, 2)
+    assert np.array_equal(got[..., 0], blocks[..., 0] + blocks[..., 1]) and np.array_equal(got[..., 1], blocks[..., 0] - blocks[..., 1])
+    # fp16 input: every stage rounds (65504 + 65504 overflows in the first stage, whatever comes later)
+    big = np.array([[65504, 65504, -65504, -65504]], F16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        got = o.fwht_butterfly(big)[0, 0]
+    # exact result [0, 0, 4a, 0]; with a + b = inf and c + d = -inf: inf + -inf = NaN, inf - -inf = inf
+    assert got.dtype == F16 and np.isnan(got[0]) and got[1] == 0 and got[2] == np.inf and got[3] == 0
+    for n in (1, 2, 128, 11008, 28672):
+        s = o.had_scale(n)
+        assert s.dtype == F32 and s == F32(1.0) / np.sqrt(F32(n))
+        assert abs(float(s) * float(s) * n - 1.0) < 1e-6
+    assert o.had_scale(4096) == F32(1 / 64) and o.had_scale(64) == F32(0.125)
+    # online_hadamard: output dtype is the input's; force_fp32 = one rounding of the fp32 transform
+    x = (rng.standard_normal((4, 24)) * 3).astype(F16)
+    y16, y32 = o.online_hadamard(x), o.online_hadamard(x, force_fp32=True)
+    assert y16.dtype == F16 and y32.dtype == F16
+    exact = o.hadamard_closed_form(x.astype(np.float64))
+    assert np.all(np.abs(y32.astype(np.float64) - exact) <= np.abs(exact) * 2.0 ** -10 + 1e-6)     # half an fp16 step + fp32 noise
+    assert np.all(np.abs(y16.astype(np.float64) - exact) <= 4e-3 * np.abs(exact).max())
+    hadk, k = o.get_hadK(24)
+    assert np.array_equal(y16, o.hadamard_staged(x, hadk, k, F16)) and np.array_equal(y32, o.hadamard_staged(x.astype(F32), hadk, k, F32).astype(F16))
+    # a power of two: no second factor, so the two modes differ by nothing but the fp32 scale's rounding
+    x = (rng.standard_normal((4, 64))).astype(F16)
+    assert np.array_equal(o.online_hadamard(x), o.online_hadamard(x, force_fp32=True))
+
+
 def test_fwht_natural_brute_force():
     rng = np.random.default_rng(2)
     for m in (1, 2, 4, 32, 128):
