@@ -205,9 +205,9 @@ def hadamard_quantize(x, hadK, K, clip_ratio=1.0, force_fp32=False, return_trans
         if rc == _lib.QR_E_UNSUPPORTED:
             rc = _lib.lib().qr_hadamard_quantize_f16_i4(_ptr(x2), rows, n, int(K), _ptr(hadK), mode, scale,
                                                         float(clip_ratio), _ptr(q), _ptr(s), _ptr(y), _lib.stream_ptr(dev))
-        if rc == _lib.QR_E_UNSUPPORTED and n <= 128:
-            # rows this short are not fused (rows of 128 only with a place for the transformed rows): the two kernels
-            # that Sequential(OnlineHadamard, Quantizer) runs, so the bits are those of the two modules
+        if rc == _lib.QR_E_UNSUPPORTED and (n <= 128 or n > functional.hadamard.MAX_FUSED_ROW):
+            # rows this short are not fused (rows of 128 only with a place for the transformed rows), rows beyond 32768
+            # neither: the steps that Sequential(OnlineHadamard, Quantizer) runs, so the bits are those of the two modules
             y = functional.matmul_hadU_cuda(x2.float() if force_fp32 else x2, hadK, int(K)).to(torch.float16)
             q, s = quantize_rows(y, clip_ratio)
             rc = 0
@@ -378,5 +378,9 @@ def quantized_linear(x, weight, weight_scales, bias=None, hadK=None, K=0, clip_r
                 _SIGNS_REFUSED.add((n, int(K)))
         if rc == _lib.QR_E_UNSUPPORTED:
             rc = call(hadK, mode)
+        if rc == _lib.QR_E_UNSUPPORTED and K and n > functional.hadamard.MAX_FUSED_ROW:
+            # rows beyond the fused front's reach: the front's own fall-back, then the linear layer
+            p = hadamard_quantize(x2, table, K, clip_ratio, force_fp32)
+            return linear_i4(p.quantized_x, p.scales_x, weight, weight_scales, bias).view(*lead, N)
         _lib.check(rc)
     return y.view(*lead, N)

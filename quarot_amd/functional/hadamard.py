@@ -89,6 +89,9 @@ def random_hadamard_matrix(size, device):
     return matmul_hadU(torch.diag(signs)).to(device)
 
 
+MAX_FUSED_ROW = 32768      # longest row of the library's Hadamard kernels (qr_hadamard: n <= 32768)
+
+
 def hadamard_transform(x, scale=1.0):
     """Power-of-two Walsh-Hadamard transform along the last axis times `scale`: the call the
     reference makes into fast_hadamard_transform (hadamard.py:95,99; kv_cache.py:32).
@@ -125,6 +128,12 @@ def matmul_hadU_cuda(X, hadK, K):
     """X . (hadK (x) H_{n/K})^T / sqrt(n) on the GPU (hadamard.py:92-101); output in X's dtype and shape."""
     n = X.shape[-1]
     scale = had_scale(n)
+    if K > 1 and n > MAX_FUSED_ROW:
+        # rows longer than the two-factor kernels hold (e.g. 53248 = 52 x 1024): the reference's own two steps
+        # (hadamard.py:97-101) -- the power-of-two factor by the FWHT kernel on the [.., K, n / K] view, rounded to X's
+        # dtype, then the table by a library GEMM
+        t = _run(X.reshape(-1, K, n // K), None, 1, scale)
+        return (hadK.to(t.device).to(t.dtype) @ t).reshape(X.shape)
     return _run(X, hadK if K > 1 else None, K, scale).reshape(X.shape)
 
 

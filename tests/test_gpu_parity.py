@@ -643,6 +643,40 @@ def test_fused_fronts_random_shapes_scales_and_clips():
         assert torch.equal(p2.scales_x.reshape(-1)[ok].view(torch.int16), scale.reshape(-1)[ok].view(torch.int16)), tag
 
 
+@pytest.mark.parametrize("n", [53248, 40960])
+def test_rows_longer_than_the_fused_kernels_take_the_references_two_steps(n):
+    """53248 = 52 x 1024 (the widest Llama-3.1 MLP) and 40960 = 40 x 1024 are beyond the library's two-factor
+    kernels (n <= 32768): the Python layer runs the reference's own sequence (quarot/functional/hadamard.py:97-101) --
+    the FWHT kernel over the [.., K, n / K] view, then the table as a library GEMM -- and the quantiser kernel behind
+    it.  Transform within tolerance of the oracle's staged arithmetic, codes and scales the oracle quantiser's on the
+    transformed rows, the fused module and the one-call linear layer bit for bit the chain."""
+    x = gpu(synth_x(5, n, seed=n))
+    for fp32 in (False, True):
+        had = quarot_amd.nn.OnlineHadamard(n, force_fp32=fp32).cuda()
+        assert had.rem_dim == o.get_hadK(n)[1]
+        y = had(x)
+        assert y.dtype == torch.float16 and y.shape == x.shape
+        assert close(y.cpu().numpy(), o.online_hadamard(x.cpu().numpy(), force_fp32=fp32))
+        fused = quarot_amd.nn.OnlineHadamardQuantizer(n, force_fp32=fp32, input_clip_ratio=0.9).cuda()
+        p = fused(x)
+        wq, ws = o.quantizer(y.cpu().numpy(), 0.9)
+        assert np.array_equal(p.quantized_x.cpu().numpy(), wq) and np.array_equal(p.scales_x.cpu().numpy().reshape(-1), ws)
+        p2, y2 = quarot_amd.hadamard_quantize(x, fused.had_rem_dim, fused.rem_dim, 0.9, force_fp32=fp32, return_transformed=True)
+        assert torch.equal(y2, y) and torch.equal(p2.quantized_x, p.quantized_x)
+    g = torch.Generator().manual_seed(n)
+    w = torch.randint(0, 256, (70, n // 2), dtype=torch.uint8, generator=g).cuda()
+    sw = (torch.rand(70, 1, generator=g) * 0.02 + 1e-3).half().cuda()
+    b = torch.randn(70, generator=g).half().cuda()
+    fused = quarot_amd.nn.OnlineHadamardQuantizer(n, input_clip_ratio=1.0).cuda()
+    for m in (1, 5):
+        pm = fused(x[:m])
+        want = quarot_amd.linear_i4(pm.quantized_x, pm.scales_x, w, sw, b)
+        got = quarot_amd.quantized_linear(x[:m], w, sw, b, fused.had_rem_dim, fused.rem_dim, 1.0)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        ref = o.linear4bit(pm.quantized_x.cpu().numpy(), pm.scales_x.cpu().numpy().reshape(-1), w.cpu().numpy(), sw.cpu().numpy(), b.cpu().numpy())
+        assert np.array_equal(bits(got.cpu().numpy()), bits(np.asarray(ref).reshape(m, 70)))
+
+
 @pytest.mark.parametrize("n", [128, 112, 80, 48, 24])
 def test_fused_front_on_short_rows_carries_the_bits_of_the_two_modules(n):
     """Rows of 128 (the head dimension: qr_hadamard has a kernel of its own for them, which adds in another order
